@@ -1,0 +1,277 @@
+"""The cache manager: paged keys and values in groups, block tables, prefix reuse, state slots.
+
+Reference: KVCache and PagedSequence (src/kv-cache.ts:5-172).  Beyond the reference: cache slots
+are sorted into groups by what they need (all keys, or a window of them); every group has a pool
+and block tables of its own, and a windowed group gives pages back once the window has passed them.
+Requests also hold a slot for per-request state of fixed size.
+"""
+from __future__ import annotations
+
+import hashlib
+import struct
+from dataclasses import dataclass, field
+
+from .pages import PageError, PagePool
+from .spec import PagedKVSpec, StateSpec
+
+FREED = -1  # block-table entry of a page that a window has passed
+
+
+@dataclass
+class PagedGroup:
+    spec: PagedKVSpec
+    slots: list[int]              # cache slot ids that live in this group, in pool order
+    pool: PagePool
+    k: object = None              # device tensor [len(slots), pages, kv_heads, page_size, head_dim]
+    v: object = None
+
+
+@dataclass
+class StateGroup:
+    spec: StateSpec
+    slots: list[int]
+    data: object = None           # device tensor [len(slots), max_sequences, *shape]
+
+
+class SequenceCache:
+    """What one request holds: a block table per group, its computed length, a state slot."""
+
+    def __init__(self, manager: "CacheManager", state_slot: int):
+        self._manager = manager
+        self.blocks: list[list[int]] = [[] for _ in manager.groups]
+        self.length = 0
+        self.state_slot = state_slot
+        self.released = False
+        self.prefix_keys: list[bytes] = []   # chained keys of the full pages computed so far
+
+    def _live(self):
+        if self.released:
+            raise PageError("Sequence cache was released.")
+
+    def release(self) -> None:
+        self._manager.release(self)
+
+
+@dataclass
+class _PrefixEntry:
+    pages: list[int]
+    last_used: int
+
+
+class CacheManager:
+    def __init__(self, slot_specs: list[PagedKVSpec | StateSpec], block_size: int, num_blocks: int,
+                 max_sequences: int, prefix_caching: bool = True):
+        """`slot_specs[i]` is what cache slot i needs.  Storage is attached with `attach_storage`."""
+        for name, value in (("block_size", block_size), ("num_blocks", num_blocks), ("max_sequences", max_sequences)):
+            if isinstance(value, bool) or not isinstance(value, int) or value <= 0:
+                raise ValueError(f"{name} must be a positive integer.")
+        self.block_size, self.num_blocks, self.max_sequences = block_size, num_blocks, max_sequences
+        self.groups: list[PagedGroup] = []
+        self.state_groups: list[StateGroup] = []
+        self.slot_location: list[tuple[str, int, int]] = []   # slot -> ("paged" | "state", group, index in group)
+        for slot, spec in enumerate(slot_specs):
+            if isinstance(spec, PagedKVSpec):
+                groups, kind = self.groups, "paged"
+                make = lambda: PagedGroup(spec, [], PagePool(num_blocks))
+            elif isinstance(spec, StateSpec):
+                groups, kind = self.state_groups, "state"
+                make = lambda: StateGroup(spec, [])
+            else:
+                raise TypeError(f"Cache slot {slot}: unknown cache spec {spec!r}.")
+            for g, group in enumerate(groups):
+                if group.spec == spec:
+                    break
+            else:
+                groups.append(make())
+                g = len(groups) - 1
+            groups[g].slots.append(slot)
+            self.slot_location.append((kind, g, len(groups[g].slots) - 1))
+        # Pages may be shared between requests only if every key of the prefix stays in the cache and
+        # no other per-request state would have to be rebuilt.
+        self.prefix_caching = bool(prefix_caching and self.groups and not self.state_groups
+                                   and all(g.spec.window is None for g in self.groups))
+        self._prefixes: dict[bytes, _PrefixEntry] = {}
+        self._clock = 0
+        self.evictions = 0
+        self._free_state_slots = list(range(max_sequences - 1, -1, -1))
+        self.live: set[SequenceCache] = set()
+
+    # ------------------------------------------------------------------ storage
+    def attach_storage(self, dtype, device) -> None:
+        """Allocate the pools on the device.  Host-only users (tests, planning) never call this."""
+        import torch
+        for g in self.groups:
+            shape = (len(g.slots), self.num_blocks, g.spec.kv_heads, self.block_size, g.spec.head_dim)
+            g.k = torch.zeros(shape, dtype=dtype, device=device)
+            g.v = torch.zeros(shape, dtype=dtype, device=device)
+        for g in self.state_groups:
+            g.data = torch.zeros((len(g.slots), self.max_sequences, *g.spec.shape),
+                                 dtype=getattr(torch, g.spec.dtype), device=device)
+
+    def storage_bytes(self, element_size: int) -> int:
+        total = 0
+        for g in self.groups:
+            total += 2 * len(g.slots) * self.num_blocks * g.spec.kv_heads * self.block_size * g.spec.head_dim * element_size
+        return total
+
+    # ------------------------------------------------------------------ sequences
+    def create(self) -> SequenceCache:
+        if not self._free_state_slots:
+            raise PageError("No free sequence slot: more live sequences than max_sequences.")
+        slot = self._free_state_slots.pop()
+        for g in self.state_groups:
+            if g.data is not None:
+                g.data[:, slot].zero_()
+        seq = SequenceCache(self, slot)
+        self.live.add(seq)
+        return seq
+
+    @staticmethod
+    def _chain(parent: bytes, tokens) -> bytes:
+        return hashlib.blake2b(parent + struct.pack(f"<{len(tokens)}q", *tokens), digest_size=16).digest()
+
+    def reuse_prefix(self, tokens) -> SequenceCache:
+        """A new sequence that already holds the longest cached run of full pages of `tokens`.
+
+        At least one token is always left to compute, also when the tokens end on a page edge
+        (reference: src/kv-cache.ts:100-112).
+        """
+        seq = self.create()
+        if not self.prefix_caching:
+            return seq
+        bs, key = self.block_size, b""
+        end = bs
+        while end < len(tokens):
+            key = self._chain(key, tokens[end - bs:end])
+            entry = self._prefixes.get(key)
+            if entry is None:
+                break
+            self._clock += 1
+            entry.last_used = self._clock
+            for g, page in zip(self.groups, entry.pages):
+                g.pool.retain(page)
+            for blocks, page in zip(seq.blocks, entry.pages):
+                blocks.append(page)
+            seq.prefix_keys.append(key)
+            seq.length = end
+            end += bs
+        return seq
+
+    def publish(self, tokens, seq: SequenceCache) -> None:
+        """Offer the last full page of `seq` (whose tokens are `tokens`) for reuse; the first publisher wins."""
+        if not self.prefix_caching or seq.released or seq.length == 0 or seq.length % self.block_size:
+            return
+        if len(tokens) != seq.length:
+            raise ValueError("Prefix tokens must match the computed length.")
+        bs = self.block_size
+        n_pages = seq.length // bs
+        while len(seq.prefix_keys) < n_pages:
+            i = len(seq.prefix_keys)
+            parent = seq.prefix_keys[-1] if seq.prefix_keys else b""
+            seq.prefix_keys.append(self._chain(parent, tokens[i * bs:(i + 1) * bs]))
+        key = seq.prefix_keys[n_pages - 1]
+        if key in self._prefixes:
+            return
+        pages = [blocks[n_pages - 1] for blocks in seq.blocks]
+        for g, page in zip(self.groups, pages):
+            g.pool.retain(page)   # the cache's own reference, beside the live requests'
+        self._clock += 1
+        self._prefixes[key] = _PrefixEntry(pages, self._clock)
+
+    def _evict_one(self) -> bool:
+        """Drop the least recently used prefix entry that only the cache still holds."""
+        best_key, best = None, None
+        for key, entry in self._prefixes.items():
+            if all(g.pool.refs[p] == 1 for g, p in zip(self.groups, entry.pages)):
+                if best is None or entry.last_used < best.last_used:
+                    best_key, best = key, entry
+        if best is None:
+            return False
+        del self._prefixes[best_key]
+        for g, page in zip(self.groups, best.pages):
+            g.pool.release(page)
+        self.evictions += 1
+        return True
+
+    def pages_needed(self, seq: SequenceCache, new_length: int) -> list[int]:
+        """Pages each group must still allocate so that `seq` can hold `new_length` tokens."""
+        need = -(-new_length // self.block_size)
+        return [max(0, need - len(blocks)) for blocks in seq.blocks]
+
+    def reserve(self, seq: SequenceCache, new_length: int) -> bool:
+        """Allocate pages in every group for tokens up to `new_length`.  All or nothing.
+
+        When a pool is empty, cached prefix pages that no request uses are evicted, least recently
+        used first (reference: src/kv-cache.ts:125-140).
+        """
+        seq._live()
+        if new_length < seq.length:
+            raise ValueError("A sequence cannot shrink.")
+        taken: list[tuple[int, int]] = []
+        for gi, (g, count) in enumerate(zip(self.groups, self.pages_needed(seq, new_length))):
+            for _ in range(count):
+                page = g.pool.allocate()
+                while page is None and self._evict_one():
+                    page = g.pool.allocate()
+                if page is None:
+                    for gj, p in reversed(taken):
+                        self.groups[gj].pool.release(p)
+                        seq.blocks[gj].pop()
+                    return False
+                seq.blocks[gi].append(page)
+                taken.append((gi, page))
+        return True
+
+    def commit(self, seq: SequenceCache, new_length: int) -> None:
+        """The step has written tokens up to `new_length`: record it and give back what windows have passed."""
+        seq._live()
+        if new_length > min((len(b) for b in seq.blocks), default=new_length // self.block_size + 1) * self.block_size:
+            raise PageError("Committed more tokens than pages were reserved for.")
+        seq.length = new_length
+        for g, blocks in zip(self.groups, seq.blocks):
+            if g.spec.window is None:
+                continue
+            # the next token (position new_length) reads keys >= new_length - window + 1
+            first_needed = max(0, new_length - g.spec.window + 1)
+            for i in range(first_needed // self.block_size):
+                if blocks[i] != FREED:
+                    g.pool.release(blocks[i])
+                    blocks[i] = FREED
+
+    def release(self, seq: SequenceCache) -> None:
+        if seq.released:
+            return
+        for g, blocks in zip(self.groups, seq.blocks):
+            for page in blocks:
+                if page != FREED:
+                    g.pool.release(page)
+            blocks.clear()
+        self._free_state_slots.append(seq.state_slot)
+        seq.released = True
+        self.live.discard(seq)
+
+    def clear_prefixes(self) -> None:
+        for entry in self._prefixes.values():
+            for g, page in zip(self.groups, entry.pages):
+                g.pool.release(page)
+        self._prefixes.clear()
+
+    # ------------------------------------------------------------------ reports
+    def free_pages(self) -> list[int]:
+        return [g.pool.num_free for g in self.groups]
+
+    def snapshot(self) -> dict:
+        """Reference: src/kv-cache.ts:162-171, one record per group."""
+        groups = []
+        for gi, g in enumerate(self.groups):
+            cached = {e.pages[gi] for e in self._prefixes.values()}
+            groups.append({
+                "window": g.spec.window, "slots": list(g.slots), "total_pages": g.pool.num_pages,
+                "free_pages": g.pool.num_free, "cached_pages": len(cached),
+                "pages": [{"id": i, "refs": r, "cached": i in cached, "active_refs": r - (i in cached)}
+                          for i, r in enumerate(g.pool.refs)],
+            })
+        first = groups[0] if groups else {"total_pages": 0, "free_pages": 0, "cached_pages": 0, "pages": []}
+        return {"total_pages": first["total_pages"], "free_pages": first["free_pages"],
+                "cached_pages": first["cached_pages"], "evictions": self.evictions, "pages": first["pages"],
+                "groups": groups, "free_sequence_slots": len(self._free_state_slots)}

@@ -1,0 +1,37 @@
+"""Options of the serving engine (reference: EngineOptions, src/engine.ts:18-26, :55-65)."""
+from __future__ import annotations
+
+from dataclasses import dataclass, fields
+
+from .base import ConfigError
+
+
+@dataclass(frozen=True)
+class EngineOptions:
+    """Names and meanings follow the reference's EngineOptions, in snake_case.
+
+    block_size          tokens in one cache page
+    num_blocks          pages in every cache group's pool
+    max_sequences       requests that may run at a time
+    max_batch_tokens    token budget of one step
+    prefill_chunk_size  most prompt tokens of one request in one step
+    prefix_caching      share full prompt pages between requests
+    record_trace        keep every event in `engine.trace`
+    """
+
+    block_size: int = 16
+    num_blocks: int = 256
+    max_sequences: int = 64
+    max_batch_tokens: int = 2048
+    prefill_chunk_size: int = 512
+    prefix_caching: bool = True
+    record_trace: bool = False
+
+    def __post_init__(self):
+        for f in fields(self):
+            value = getattr(self, f.name)
+            if f.name in ("prefix_caching", "record_trace"):
+                if not isinstance(value, bool):
+                    raise ConfigError(f"{f.name} must be a boolean.")
+            elif isinstance(value, bool) or not isinstance(value, int) or value <= 0:
+                raise ConfigError(f"{f.name} must be a positive integer.")

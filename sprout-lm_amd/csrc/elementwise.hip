@@ -1,0 +1,187 @@
+// Embedding gather, RMSNorm, SiLU-gated product, casts, and rotation + cache write.
+// All arithmetic is float32; only loads and stores see the storage type.
+#include "common.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+// ---------------------------------------------------------------- embedding
+template <typename TW>
+__global__ void embed_kernel(const TW* __restrict__ table, const int32_t* __restrict__ tokens,
+                             float* __restrict__ residual, int H) {
+  const int t = blockIdx.x;
+  const TW* row = table + size_t(tokens[t]) * H;
+  float* out = residual + size_t(t) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = to_float(row[i]);
+}
+
+// ---------------------------------------------------------------- RMSNorm
+// y = (x * rsqrt(mean(x^2) + eps)) * w, the normalised value rounded to float32 before the weight.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
+                               const TW* __restrict__ w, float eps, TO* __restrict__ out, int H) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const float* in = x + size_t(rows ? rows[r] : r) * H;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float v = in[i];
+    sum = fmaf(v, v, sum);
+  }
+  sum = block_sum(sum, scratch);
+  const float scale = 1.0f / sqrtf(sum / float(H) + eps);
+  TO* o = out + size_t(r) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float n = in[i] * scale;
+    o[i] = from_float<TO>(n * to_float(w[i]));
+  }
+}
+
+// ---------------------------------------------------------------- SiLU(gate) * up
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const float g = to_float(gu[size_t(t) * 2 * I + i]);
+  const float u = to_float(gu[size_t(t) * 2 * I + I + i]);
+  const float s = g / (1.0f + expf(-g));
+  out[size_t(t) * I + i] = from_float<T>(s * u);
+}
+
+// ---------------------------------------------------------------- cast
+template <typename TS, typename TD>
+__global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, int64_t n) {
+  int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t step = int64_t(gridDim.x) * blockDim.x;
+  for (; i < n; i += step) dst[i] = from_float<TD>(to_float(src[i]));
+}
+
+// ---------------------------------------------------------------- rotation + cache write
+// One block per token.  Pair (d, d + rotary_dim/2) of each q and k head turns by
+// positions[t] * inv_freq[d]; k (rotated) and v go to the pools.
+template <typename T>
+__global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int rotary_dim,
+                                  const int32_t* __restrict__ slot_mapping, T* __restrict__ k_pool,
+                                  T* __restrict__ v_pool, int nq, int nkv, int hd, int page_size) {
+  const int t = blockIdx.x;
+  const int width = (nq + 2 * nkv) * hd;
+  T* row = qkv + size_t(t) * width;
+  const float pos = float(positions[t]);
+  const int half = rotary_dim / 2;
+  const int slot = nkv ? slot_mapping[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+
+  // rotate q heads in place, k heads in place and into the pool
+  const int pairs = (nq + nkv) * half;
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
+    const int head = i / half, d = i % half;
+    float sn, cs;
+    sincosf(pos * inv_freq[d], &sn, &cs);
+    T* h = row + size_t(head) * hd;
+    const float a = to_float(h[d]), b = to_float(h[d + half]);
+    const T ra = from_float<T>(a * cs - b * sn), rb = from_float<T>(b * cs + a * sn);
+    h[d] = ra;
+    h[d + half] = rb;
+    if (head >= nq && slot >= 0) {
+      T* dst = k_pool + ((size_t(page) * nkv + (head - nq)) * page_size + off) * hd;
+      dst[d] = ra;
+      dst[d + half] = rb;
+    }
+  }
+  if (slot < 0) return;
+  // the part of k heads beyond rotary_dim is cached as it is
+  if (rotary_dim < hd) {
+    const int rest = hd - rotary_dim;
+    for (int i = threadIdx.x; i < nkv * rest; i += blockDim.x) {
+      const int g = i / rest, d = rotary_dim + i % rest;
+      k_pool[((size_t(page) * nkv + g) * page_size + off) * hd + d] = row[size_t(nq + g) * hd + d];
+    }
+  }
+  for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
+    const int g = i / hd, d = i % hd;
+    v_pool[((size_t(page) * nkv + g) * page_size + off) * hd + d] = row[size_t(nq + nkv + g) * hd + d];
+  }
+}
+
+}  // namespace sprout
+
+using namespace sprout;
+
+extern "C" int sp_embed(void* stream, int table_dtype, const void* table, const int32_t* tokens,
+                        float* residual, int T, int H, int V) {
+  SP_REQUIRE(T >= 0 && H > 0 && V > 0, "sp_embed: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (table_dtype == kF32)
+    embed_kernel<float><<<T, 256, 0, s>>>((const float*)table, tokens, residual, H);
+  else if (table_dtype == kBF16)
+    embed_kernel<bf16_t><<<T, 256, 0, s>>>((const bf16_t*)table, tokens, residual, H);
+  else
+    SP_REQUIRE(false, "sp_embed: unsupported table dtype %d", table_dtype);
+  return check_launch("sp_embed");
+}
+
+extern "C" int sp_rmsnorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w,
+                          float eps, int out_dtype, void* out, int R, int H) {
+  SP_REQUIRE(R >= 0 && H > 0, "sp_rmsnorm: bad sizes R=%d H=%d", R, H);
+  if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = H >= 1024 ? 512 : 256;
+#define SP_NORM(TW, TO) \
+  rmsnorm_kernel<TW, TO><<<R, threads, 0, s>>>(x, rows, (const TW*)w, eps, (TO*)out, H)
+  if (w_dtype == kF32 && out_dtype == kF32) SP_NORM(float, float);
+  else if (w_dtype == kF32 && out_dtype == kBF16) SP_NORM(float, bf16_t);
+  else if (w_dtype == kBF16 && out_dtype == kF32) SP_NORM(bf16_t, float);
+  else if (w_dtype == kBF16 && out_dtype == kBF16) SP_NORM(bf16_t, bf16_t);
+  else SP_REQUIRE(false, "sp_rmsnorm: unsupported dtypes w=%d out=%d", w_dtype, out_dtype);
+#undef SP_NORM
+  return check_launch("sp_rmsnorm");
+}
+
+extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I) {
+  SP_REQUIRE(T >= 0 && I > 0, "sp_silu_mul: bad sizes T=%d I=%d", T, I);
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((I + 255) / 256, T);
+  if (dtype == kF32) silu_mul_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, (float*)out, I);
+  else if (dtype == kBF16) silu_mul_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, I);
+  else SP_REQUIRE(false, "sp_silu_mul: unsupported dtype %d", dtype);
+  return check_launch("sp_silu_mul");
+}
+
+extern "C" int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n) {
+  SP_REQUIRE(n >= 0, "sp_cast: bad size");
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int blocks = (int)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+  if (src_dtype == kF32 && dst_dtype == kBF16)
+    cast_kernel<float, bf16_t><<<blocks, 256, 0, s>>>((const float*)src, (bf16_t*)dst, n);
+  else if (src_dtype == kBF16 && dst_dtype == kF32)
+    cast_kernel<bf16_t, float><<<blocks, 256, 0, s>>>((const bf16_t*)src, (float*)dst, n);
+  else
+    SP_REQUIRE(false, "sp_cast: unsupported dtypes %d -> %d", src_dtype, dst_dtype);
+  return check_launch("sp_cast");
+}
+
+extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions,
+                             const float* inv_freq, int rotary_dim, const int32_t* slot_mapping, void* k_pool,
+                             void* v_pool, int T, int nq, int nkv, int hd, int page_size, int num_pages) {
+  SP_REQUIRE(T >= 0 && nq > 0 && nkv >= 0 && hd > 0, "sp_rope_cache: bad sizes");
+  SP_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
+             "sp_rope_cache: rotary_dim %d must be even and at most head size %d", rotary_dim, hd);
+  SP_REQUIRE(nkv == 0 || (slot_mapping && k_pool && v_pool && page_size > 0 && num_pages > 0),
+             "sp_rope_cache: cache arguments missing");
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == kF32)
+    rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim, slot_mapping,
+                                               (float*)k_pool, (float*)v_pool, nq, nkv, hd, page_size);
+  else if (dtype == kBF16)
+    rope_cache_kernel<bf16_t><<<T, 256, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim, slot_mapping,
+                                                (bf16_t*)k_pool, (bf16_t*)v_pool, nq, nkv, hd, page_size);
+  else
+    SP_REQUIRE(false, "sp_rope_cache: unsupported dtype %d", dtype);
+  return check_launch("sp_rope_cache");
+}

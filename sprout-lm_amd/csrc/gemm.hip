@@ -1,0 +1,31 @@
+// Entry point of the matrix products: checks the operands and picks a kernel.
+#include "common.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+int gemm_generic(hipStream_t s, int a_dtype, const void* a, int w_dtype, const void* w, int bias_dtype,
+                 const void* bias, int mode, int out_dtype, void* out, int T, int N, int K);
+int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode,
+              int out_dtype, void* out, int T, int N, int K, bool* handled);
+}  // namespace sprout
+
+using namespace sprout;
+
+extern "C" int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w, int bias_dtype,
+                       const void* bias, int mode, int out_dtype, void* out, int T, int N, int K) {
+  SP_REQUIRE(T >= 0 && N > 0 && K > 0, "sp_gemm: bad sizes T=%d N=%d K=%d", T, N, K);
+  SP_REQUIRE((a_dtype == kF32 || a_dtype == kBF16) && (w_dtype == kF32 || w_dtype == kBF16),
+             "sp_gemm: unsupported operand dtypes a=%d w=%d", a_dtype, w_dtype);
+  SP_REQUIRE(mode >= 0 && mode <= 2, "sp_gemm: unknown mode %d", mode);
+  SP_REQUIRE(mode != 0 || out_dtype == kF32 || out_dtype == kBF16, "sp_gemm: unsupported output dtype %d", out_dtype);
+  SP_REQUIRE(!bias || bias_dtype == kF32 || bias_dtype == kBF16, "sp_gemm: unsupported bias dtype %d", bias_dtype);
+  SP_REQUIRE(a && w && out, "sp_gemm: null operand");
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (a_dtype == kBF16 && w_dtype == kBF16) {
+    bool handled = false;
+    int rc = gemm_bf16(s, a, w, bias_dtype, bias, mode, out_dtype, out, T, N, K, &handled);
+    if (handled) return rc;
+  }
+  return gemm_generic(s, a_dtype, a, w_dtype, w, bias_dtype, bias, mode, out_dtype, out, T, N, K);
+}

@@ -1,0 +1,112 @@
+// Greedy and temperature sampling over float32 logits, two stages per row.
+// Greedy: lowest index among the maxima; a row with a non-finite logit yields -1
+// (reference: argmaxKernel, native/cuda-device.inc:97-115).
+// Temperature: argmax of logits / temperature + Gumbel noise.  The noise of a column comes from a
+// counter generator keyed by (seed, counter, column) only, so a request's draw does not depend on
+// what else is in the batch or on the row it lands in.
+#include "common.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+constexpr int SAMPLE_CHUNK = 8192;  // logits per first-stage block
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {  // splitmix64 finaliser
+  z += 0x9e3779b97f4a7c15ull;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ float gumbel(uint64_t seed, uint32_t counter, uint32_t column) {
+  const uint64_t h = mix64(mix64(seed ^ (uint64_t(counter) << 32)) + column);
+  const float u = (float(uint32_t(h >> 40)) + 0.5f) * (1.0f / 16777216.0f);  // (0, 1)
+  return -logf(-logf(u));
+}
+
+__device__ __forceinline__ void take_better(float& bv, int& bi, float v, int i) {
+  if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+}
+
+__global__ __launch_bounds__(256) void sample_stage1(const float* __restrict__ logits,
+                                                     const float* __restrict__ temperature,
+                                                     const int64_t* __restrict__ seed,
+                                                     const int32_t* __restrict__ counter,
+                                                     float* __restrict__ part_value, int* __restrict__ part_index,
+                                                     int V, int chunks) {
+  __shared__ float sv[256];
+  __shared__ int si[256];
+  __shared__ int sbad[256];
+  const int r = blockIdx.y, chunk = blockIdx.x;
+  const float* row = logits + size_t(r) * V;
+  const float temp = temperature ? temperature[r] : 0.f;
+  const float inv_temp = temp > 0.f ? 1.0f / temp : 1.0f;
+  const uint64_t sd = seed ? uint64_t(seed[r]) : 0;
+  const uint32_t ctr = counter ? uint32_t(counter[r]) : 0;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, bad = 0;
+  const int end = min(V, (chunk + 1) * SAMPLE_CHUNK);
+  for (int i = chunk * SAMPLE_CHUNK + threadIdx.x; i < end; i += 256) {
+    float v = row[i];
+    if (!isfinite(v)) bad = 1;
+    if (temp > 0.f) v = v * inv_temp + gumbel(sd, ctr, uint32_t(i));
+    take_better(bv, bi, v, i);
+  }
+  sv[threadIdx.x] = bv; si[threadIdx.x] = bi; sbad[threadIdx.x] = bad;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if (threadIdx.x < s) {
+      sbad[threadIdx.x] |= sbad[threadIdx.x + s];
+      take_better(sv[threadIdx.x], si[threadIdx.x], sv[threadIdx.x + s], si[threadIdx.x + s]);
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    part_value[size_t(r) * chunks + chunk] = sv[0];
+    part_index[size_t(r) * chunks + chunk] = sbad[0] ? -1 : si[0];
+  }
+}
+
+__global__ __launch_bounds__(64) void sample_stage2(const float* __restrict__ part_value,
+                                                    const int* __restrict__ part_index, int32_t* __restrict__ out,
+                                                    int chunks) {
+  const int r = blockIdx.x;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff, bad = 0;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const int i = part_index[size_t(r) * chunks + c];
+    if (i < 0) bad = 1;
+    else take_better(bv, bi, part_value[size_t(r) * chunks + c], i);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    bad |= __shfl_xor(bad, o, 64);
+    take_better(bv, bi, ov, oi);
+  }
+  if (threadIdx.x == 0) out[r] = (bad || bi == 0x7fffffff) ? -1 : bi;
+}
+
+}  // namespace sprout
+
+using namespace sprout;
+
+extern "C" int sp_sample_workspace_floats(int R, int V) {
+  const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  return R * chunks * 2;
+}
+
+extern "C" int sp_sample(void* stream, const float* logits, const float* temperature, const int64_t* seed,
+                         const int32_t* counter, int32_t* out, float* workspace, int R, int V) {
+  SP_REQUIRE(R >= 0 && V > 0, "sp_sample: bad sizes R=%d V=%d", R, V);
+  SP_REQUIRE(logits && out && workspace, "sp_sample: null argument");
+  if (R == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  float* part_value = workspace;
+  int* part_index = (int*)(workspace + size_t(R) * chunks);
+  sample_stage1<<<dim3(chunks, R), 256, 0, s>>>(logits, temperature, seed, counter, part_value, part_index, V, chunks);
+  sample_stage2<<<R, 64, 0, s>>>(part_value, part_index, out, chunks);
+  return check_launch("sp_sample");
+}

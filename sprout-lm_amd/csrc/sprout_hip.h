@@ -1,0 +1,58 @@
+// C interface of libsprout_hip.so.  Every function returns 0 on success; otherwise
+// sp_last_error() gives the reason.  Pointers are device pointers unless named host_*.
+// dtype codes: 0 = float32, 1 = bfloat16.  All launches go to `stream`.
+#pragma once
+#include <stdint.h>
+
+extern "C" {
+
+const char* sp_last_error();
+int sp_version();
+
+// residual[t, :] = table[tokens[t], :]            residual is float32 [T, H]
+int sp_embed(void* stream, int table_dtype, const void* table, const int32_t* tokens, float* residual,
+             int T, int H, int V);
+
+// out[r, :] = rmsnorm(x[rows ? rows[r] : r, :]) * w      x float32 [*, H]; out [R, H] of out_dtype
+int sp_rmsnorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, float eps,
+               int out_dtype, void* out, int R, int H);
+
+// out = a[T, K] . w[N, K]^T (+ bias[N])
+// mode 0: store as out_dtype [T, N];  mode 1: out (float32 [T, N]) += result;  mode 2: store float32
+int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w, int bias_dtype,
+            const void* bias, int mode, int out_dtype, void* out, int T, int N, int K);
+
+// Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
+// inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
+// (= page * page_size + offset; negative: not written).  nkv == 0: only q is rotated.
+// Pools are [pages][nkv][page_size][hd] of `dtype`.
+int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, const float* inv_freq,
+                  int rotary_dim, const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int nq,
+                  int nkv, int hd, int page_size, int num_pages);
+
+// Causal attention of a mixed batch over the paged pools.
+// q: [T, q_stride] (head h at column h * hd), out: [T, nq * hd].
+// Sequence s owns tokens q_start[s] .. q_start[s] + q_len[s]; their positions end at ctx_len[s] - 1.
+// tiles: [n_tiles][2] = (sequence, first query of the tile within the sequence's tokens).
+// window <= 0: all keys; else keys with position - key < window.
+int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
+                 const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
+                 const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
+                 int tile_q, void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
+                 float scale, int kernel_kind);
+int sp_attention_tile_q(int dtype, int hd, int max_q_len, int kernel_kind);
+
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i]
+int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I);
+
+// dst (dst_dtype) = src (src_dtype), n elements
+int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n);
+
+// Greedy / temperature sampling of R rows of float32 logits [R, V].
+// temperature[r] == 0: lowest index of the maximum.  Else argmax of logits / temperature + Gumbel noise
+// from a counter generator keyed by (seed[r], counter[r], column).
+// out[r] = token, or -1 if a logit of the row is not finite.  workspace: R * 2 * blocks_per_row floats.
+int sp_sample(void* stream, const float* logits, const float* temperature, const int64_t* seed,
+              const int32_t* counter, int32_t* out, float* workspace, int R, int V);
+int sp_sample_workspace_floats(int R, int V);
+}

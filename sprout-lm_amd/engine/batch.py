@@ -1,0 +1,178 @@
+"""The batch of one step: what parts see while they run.
+
+A step holds, for every request in it, the next tokens of that request (a portion of its prompt or
+one decoded token).  All tokens are laid out flat, request after request.  The integer arrays that
+the kernels need are packed into one host buffer and copied to the device in one transfer.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+TILE_SIZES = (16, 64, 128)   # query-tile sizes an attention kernel may ask for
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its cache, its next tokens, and where logits are wanted."""
+
+    seq: object                 # cache.SequenceCache
+    tokens: list
+    want: list                  # indices into `tokens`
+
+
+@dataclass
+class CacheSlotView:
+    """What a mixer gets for its cache slot in this step."""
+
+    writes: bool
+    k: torch.Tensor | None = None            # [pages, kv_heads, page_size, head_dim]
+    v: torch.Tensor | None = None
+    block_tables: torch.Tensor | None = None  # int32 [sequences, max_blocks]
+    slot_mapping: torch.Tensor | None = None  # int32 [tokens]: page * page_size + offset
+    state: torch.Tensor | None = None         # [max_sequences, *shape] for a fixed-size state slot
+    page_size: int = 0
+
+
+class Workspace:
+    """Named scratch tensors that live across steps and grow on demand."""
+
+    def __init__(self, device):
+        self.device = device
+        self._flat: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def get(self, name: str, shape, dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= s
+        key = (name, dtype)
+        flat = self._flat.get(key)
+        if flat is None or flat.numel() < n:
+            flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._flat[key] = flat
+        return flat[:n].view(shape)
+
+
+class StepContext:
+    def __init__(self, workspace: Workspace, act_dtype, attention_kind: int = 0):
+        self.workspace = workspace
+        self.act_dtype = act_dtype
+        self.attention_kind = attention_kind
+        self.n_tokens = self.n_seqs = self.n_logits = 0
+        self.max_q_len = 0
+        self.token_ids = self.positions = self.q_start = self.q_len = self.ctx_len = None
+        self.logit_rows = self.state_slots = self.seq_of_token = None
+        self._tiles: dict[int, tuple[torch.Tensor, int]] = {}
+        self.group_tables: list[torch.Tensor] = []
+        self.group_slots: list[torch.Tensor] = []
+        self.host = {}   # the same arrays on the host (numpy), for parts that plan on the CPU
+
+    def buffer(self, name: str, shape, dtype) -> torch.Tensor:
+        return self.workspace.get(name, shape, dtype)
+
+    def attention_tiles(self, dtype, head_dim: int):
+        from .. import ops
+        tile_q = ops.attention_tile_q(dtype, head_dim, self.max_q_len, self.attention_kind)
+        tiles, n = self._tiles[tile_q]
+        return tiles, n, tile_q
+
+
+def _tiles_for(q_lens, tile_q: int) -> np.ndarray:
+    out = []
+    for s, n in enumerate(q_lens):
+        for off in range(0, n, tile_q):
+            out.append((s, off))
+    return np.asarray(out, dtype=np.int32).reshape(-1, 2)
+
+
+class DescriptorStager:
+    """Pinned host buffers, used in turn, through which a step's integer arrays reach the device."""
+
+    def __init__(self, device, depth: int = 4):
+        self.device = device
+        self.depth = depth
+        self._host = [None] * depth
+        self._dev = [None] * depth
+        self._events = [None] * depth
+        self._turn = 0
+
+    def upload(self, arrays: list[np.ndarray]) -> list[torch.Tensor]:
+        """Copy the int32 arrays to the device in one transfer; returns a device view per array."""
+        sizes = [a.size for a in arrays]
+        offsets, total = [], 0
+        for n in sizes:
+            offsets.append(total)
+            total += (n + 3) // 4 * 4     # keep every array 16-byte aligned
+        i = self._turn
+        self._turn = (self._turn + 1) % self.depth
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        if self._host[i] is None or self._host[i].numel() < total:
+            cap = max(4096, 1 << (max(total, 1) - 1).bit_length())
+            self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._dev[i] = torch.empty(cap, dtype=torch.int32, device=self.device)
+        host = self._host[i].numpy()
+        for a, off, n in zip(arrays, offsets, sizes):
+            host[off:off + n] = a.reshape(-1)
+        self._dev[i][:total].copy_(self._host[i][:total], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._events[i] = event
+        return [self._dev[i][off:off + n].view(a.shape) for a, off, n in zip(arrays, offsets, sizes)]
+
+
+def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, workspace: Workspace, act_dtype,
+                  attention_kind: int = 0) -> StepContext:
+    """Lay the entries out flat and stage every array the kernels need.
+
+    Each entry's sequence must already hold pages for its new tokens (CacheManager.reserve).
+    """
+    ctx = StepContext(workspace, act_dtype, attention_kind)
+    bs = cache.block_size
+    q_lens = [len(e.tokens) for e in entries]
+    starts = np.zeros(len(entries), dtype=np.int32)
+    if entries:
+        starts[1:] = np.cumsum(q_lens[:-1])
+    T = int(sum(q_lens))
+    first_pos = np.asarray([e.seq.length for e in entries], dtype=np.int32)
+    q_len = np.asarray(q_lens, dtype=np.int32)
+    ctx_len = first_pos + q_len
+    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries]) if T else np.zeros(0, np.int32)
+    seq_of_token = np.repeat(np.arange(len(entries), dtype=np.int32), q_len)
+    positions = (np.arange(T, dtype=np.int32) - starts[seq_of_token] + first_pos[seq_of_token]).astype(np.int32)
+    rows = [starts[s] + w for s, e in enumerate(entries) for w in e.want]
+    logit_rows = np.asarray(rows, dtype=np.int32)
+    state_slots = np.asarray([e.seq.state_slot for e in entries], dtype=np.int32)
+
+    arrays = [token_ids, positions, starts, q_len, ctx_len, logit_rows, state_slots, seq_of_token]
+    tile_arrays = [_tiles_for(q_lens, t) for t in TILE_SIZES]
+    arrays += tile_arrays
+    for gi, group in enumerate(cache.groups):
+        width = max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
+        tables = np.full((len(entries), width), -1, dtype=np.int32)
+        slots = np.full(T, -1, dtype=np.int32)
+        for s, e in enumerate(entries):
+            blocks = e.seq.blocks[gi]
+            tables[s, :len(blocks)] = blocks
+            if q_lens[s]:
+                pos = np.arange(first_pos[s], ctx_len[s])
+                pages = np.asarray(blocks, dtype=np.int64)[pos // bs]
+                slots[starts[s]:starts[s] + q_lens[s]] = pages * bs + pos % bs
+        arrays += [tables, slots]
+
+    dev = stager.upload(arrays)
+    (ctx.token_ids, ctx.positions, ctx.q_start, ctx.q_len, ctx.ctx_len, ctx.logit_rows, ctx.state_slots,
+     ctx.seq_of_token) = dev[:8]
+    for t, arr, d in zip(TILE_SIZES, tile_arrays, dev[8:8 + len(TILE_SIZES)]):
+        ctx._tiles[t] = (d, arr.shape[0])
+    rest = dev[8 + len(TILE_SIZES):]
+    ctx.group_tables = rest[0::2]
+    ctx.group_slots = rest[1::2]
+    ctx.n_tokens, ctx.n_seqs, ctx.n_logits = T, len(entries), len(rows)
+    ctx.max_q_len = max(q_lens, default=0)
+    ctx.host = {"q_start": starts, "q_len": q_len, "ctx_len": ctx_len, "positions": positions,
+                "token_ids": token_ids, "state_slots": state_slots, "seq_of_token": seq_of_token,
+                "first_pos": first_pos}
+    return ctx

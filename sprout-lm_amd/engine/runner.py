@@ -1,0 +1,151 @@
+"""The model on the device and its one step function."""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.spec import PagedKVSpec
+from ..config.base import token_id_list
+from ..models.plan import ModelPlan
+from ..registry import build_model_plan, load_config
+from ..weights.loader import load_named_tensors
+from ..weights.random_init import random_tensors
+from .batch import CacheSlotView, DescriptorStager, StepEntry, Workspace, build_context
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"Unsupported dtype {name}; the engine computes in bfloat16 or float32.")
+        return name
+    try:
+        return DTYPES[name]
+    except KeyError:
+        raise ValueError(f"Unknown dtype {name!r}; choose bfloat16 or float32.") from None
+
+
+def require_gpu() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("No GPU is visible: the engine runs its HIP kernels on an AMD GPU and has no CPU path.")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+class ModelRunner:
+    """Weights, cache pools and workspace of one model, and `step`.
+
+    `step` runs exactly the tokens it is given, as one batch, reading earlier tokens from the
+    cache, and returns float32 logits at the wanted places.
+    """
+
+    def __init__(self, plan: ModelPlan, tensors: dict, dtype: torch.dtype, device, block_size: int, num_blocks: int,
+                 max_sequences: int, prefix_caching: bool = False, stop_token_ids=None):
+        self.plan, self.dtype, self.device = plan, dtype, device
+        self.parts = plan.instantiate()
+        self.parts.bind(tensors, device, dtype)
+        self.cache = CacheManager(self.parts.cache_slot_specs, block_size, num_blocks, max_sequences, prefix_caching)
+        self.cache.attach_storage(dtype, device)
+        self.workspace = Workspace(device)
+        self.stager = DescriptorStager(device)
+        self.stop_token_ids = tuple(stop_token_ids if stop_token_ids is not None else plan.eos_token_ids)
+        self.attention_kind = 1 if dtype == torch.float32 else 0
+        self.vocab_size, self.hidden_size, self.max_positions = plan.vocab_size, plan.hidden_size, plan.max_positions
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", **cache_options) -> "ModelRunner":
+        device = require_gpu()
+        dtype = parse_dtype(dtype)
+        config = load_config(folder)
+        plan = build_model_plan(config)
+        tensors = load_named_tensors(folder, plan.expected_tensors(), set(plan.ignorable_tensors), dtype, device)
+        return cls(plan, tensors, dtype, device, stop_token_ids=stop_ids_of_folder(folder, plan), **cache_options)
+
+    @classmethod
+    def from_config(cls, config, seed: int, dtype="bfloat16", **cache_options) -> "ModelRunner":
+        """Random weights drawn on the device (for benchmarks; a model folder is not written)."""
+        device = require_gpu()
+        dtype = parse_dtype(dtype)
+        plan = build_model_plan(config)
+        tensors = random_tensors(plan.expected_tensors(), seed, dtype=dtype, device=device)
+        return cls(plan, tensors, dtype, device, **cache_options)
+
+    # ------------------------------------------------------------------ the step
+    def _slot_view(self, ctx, call) -> CacheSlotView | None:
+        if call.cache_slot is None:
+            return None
+        kind, g, index = self.cache.slot_location[call.cache_slot]
+        if kind == "paged":
+            group = self.cache.groups[g]
+            return CacheSlotView(call.writes, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
+                                 slot_mapping=ctx.group_slots[g], page_size=self.cache.block_size)
+        group = self.cache.state_groups[g]
+        return CacheSlotView(call.writes, state=group.data[index])
+
+    def validate(self, entries: list[StepEntry]) -> None:
+        seen = set()
+        for e in entries:
+            if id(e.seq) in seen:
+                raise ValueError("A request appears twice in one step.")
+            seen.add(id(e.seq))
+            if e.seq.released:
+                raise ValueError("A request's cache was released before the step.")
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError("A step entry brings no tokens.")
+            if any(not isinstance(t, int) or isinstance(t, bool) or t < 0 or t >= self.vocab_size for t in e.tokens):
+                raise ValueError(f"Token ids must be integers in [0, {self.vocab_size}).")
+            if e.seq.length + n > self.max_positions:
+                raise ValueError(f"Position {e.seq.length + n - 1} is beyond the model's {self.max_positions} positions.")
+            if any(not isinstance(w, int) or w < 0 or w >= n for w in e.want):
+                raise ValueError("Wanted logit places must index the entry's own tokens.")
+            for gi, needed in enumerate(self.cache.pages_needed(e.seq, e.seq.length + n)):
+                if needed:
+                    raise ValueError("Pages for the entry's tokens were not reserved before the step.")
+
+    def step(self, entries: list[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns float32 logits [number of wanted places, vocab] on the device.
+
+        The sequences' lengths are advanced (and pages that a window has passed are given back)
+        before the call returns; the kernels may still be running on the stream.
+        """
+        self.validate(entries)
+        ctx = build_context(entries, self.cache, self.stager, self.workspace, self.dtype, self.attention_kind)
+        logits = self.forward(ctx)
+        for e in entries:
+            self.cache.commit(e.seq, e.seq.length + len(e.tokens))
+        return logits
+
+    def forward(self, ctx) -> torch.Tensor:
+        T, H = ctx.n_tokens, self.hidden_size
+        residual = ctx.buffer("residual", (T, H), torch.float32)
+        self.parts.embedding.forward(ctx, ctx.token_ids, residual)
+        for call in self.plan.schedule:
+            self.parts.blocks[call.layer].forward(ctx, residual, self._slot_view(ctx, call))
+        n = ctx.n_logits
+        logits = ctx.buffer("logits", (n, self.vocab_size), torch.float32)
+        if n:
+            normed = ctx.buffer("final_normed", (n, H), self.dtype)
+            self.parts.final_norm.forward(ctx, residual, normed, rows=ctx.logit_rows)
+            self.parts.head.forward(ctx, normed, logits)
+        return logits
+
+    # ------------------------------------------------------------------ sizes
+    def kv_bytes_per_token(self) -> int:
+        size = torch.empty((), dtype=self.dtype).element_size()
+        return sum(2 * s.kv_heads * s.head_dim * size for s in self.parts.cache_slot_specs if isinstance(s, PagedKVSpec))
+
+
+def stop_ids_of_folder(folder: str, plan: ModelPlan) -> tuple[int, ...]:
+    """generation_config.json's eos_token_id replaces the configuration's (reference: src/qwen.ts:124-128)."""
+    path = os.path.join(folder, "generation_config.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            generation = json.load(f)
+        if isinstance(generation, dict) and generation.get("eos_token_id") is not None:
+            return token_id_list(generation["eos_token_id"], plan.vocab_size, "generation_config eos_token_id")
+    return tuple(plan.eos_token_ids)

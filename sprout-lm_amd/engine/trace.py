@@ -1,0 +1,88 @@
+"""Trace replay: feeds given token ids through the model step by step and writes logits.
+
+It samples nothing and decides nothing: every step of the trace becomes one call of the engine's
+own step function, on the engine's own cache manager and kernels.
+
+    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+
+Steps are read from standard input, one JSON object a line:
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+For a step in which logits are wanted, `<out>/<step>.f32` holds them as little-endian float32
+[wanted, vocab], in the order of the entries and of `want`.  After every step the line
+`done <step>` is printed.  The analogue in the reference is scripts/reference.py:20-44, which
+writes last-position logits of whole sequences.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+
+PAGE_TOKENS = 16
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
+    parser.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    parser.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    parser.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    parser.add_argument("--max-tokens", type=int, required=True,
+                        help="most tokens live requests hold at a time (each rounded up to 64)")
+    parser.add_argument("--block-size", type=int, default=PAGE_TOKENS, help="tokens per cache page (divides 64)")
+    parser.add_argument("--max-sequences", type=int, default=16)
+    args = parser.parse_args(argv)
+    if args.max_tokens <= 0 or args.block_size <= 0 or 64 % args.block_size:
+        parser.error("--max-tokens must be positive and --block-size must divide 64")
+
+    print("[trace_run] loading the engine (kernels are compiled at the first call) ...", file=sys.stderr, flush=True)
+    import numpy as np
+    import torch
+    from .batch import StepEntry
+    from .runner import ModelRunner
+    from ..ops import library
+    library()
+    num_blocks = -(-args.max_tokens // args.block_size)
+    runner = ModelRunner.from_folder(args.model, args.dtype, block_size=args.block_size, num_blocks=num_blocks,
+                                     max_sequences=args.max_sequences, prefix_caching=False)
+    os.makedirs(args.out, exist_ok=True)
+    print(f"[trace_run] ready: {runner.plan.architecture}, {args.dtype}, {num_blocks} pages of {args.block_size}",
+          file=sys.stderr, flush=True)
+
+    live = {}
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        record = json.loads(line)
+        step = record["step"]
+        entries = []
+        for item in record.get("entries", []):
+            seq = live.get(item["id"])
+            if seq is None:
+                seq = live[item["id"]] = runner.cache.create()
+            tokens = [int(t) for t in item["tokens"]]
+            if not runner.cache.reserve(seq, seq.length + len(tokens)):
+                print(f"[trace_run] step {step}: the cache pool of {args.max_tokens} tokens is too small for "
+                      f"request {item['id']!r}", file=sys.stderr, flush=True)
+                return 1
+            entries.append(StepEntry(seq, tokens, [int(w) for w in item.get("want", [])]))
+        if entries:
+            logits = runner.step(entries)
+            if logits.shape[0]:
+                host = logits.to("cpu", copy=True).numpy().astype("<f4", copy=False)
+                host.tofile(os.path.join(args.out, f"{step}.f32"))
+            else:
+                torch.cuda.current_stream().synchronize()
+        for name in record.get("end", []):
+            seq = live.pop(name, None)
+            if seq is not None:
+                seq.release()
+        print(f"done {step}", flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,185 @@
+"""One function per kernel entry point.  Host-side shape checks stand before every launch, because a
+kernel that reads past a buffer can take the whole GPU down."""
+from __future__ import annotations
+
+import torch
+
+from .library import KernelError, check, library
+
+_CODES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODES[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: unsupported dtype {t.dtype}") from None
+
+
+def _gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{what} must live on the GPU; the engine has no CPU path.")
+    if not t.is_contiguous():
+        raise KernelError(f"{what} must be contiguous.")
+
+
+def _ints(t: torch.Tensor, n: int, what: str) -> None:
+    _gpu(t, what)
+    if t.dtype != torch.int32 or t.numel() < n:
+        raise KernelError(f"{what}: expected at least {n} int32 values, got {t.numel()} of {t.dtype}.")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def embed(table: torch.Tensor, tokens: torch.Tensor, residual: torch.Tensor) -> None:
+    """residual[t] = table[tokens[t]] as float32."""
+    _gpu(table, "embedding table"); _gpu(residual, "residual")
+    T = residual.shape[0]
+    V, H = table.shape
+    _ints(tokens, T, "tokens")
+    if residual.dtype != torch.float32 or residual.shape[1] != H:
+        raise KernelError(f"embed: residual must be float32 [T, {H}], got {residual.dtype} {tuple(residual.shape)}")
+    check(library().sp_embed(_stream(), _code(table, "embedding table"), table.data_ptr(), tokens.data_ptr(),
+                             residual.data_ptr(), T, H, V))
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """out[r] = rmsnorm(x[rows[r]] or x[r]) * weight; x is float32."""
+    _gpu(x, "norm input"); _gpu(weight, "norm weight"); _gpu(out, "norm output")
+    R, H = out.shape
+    if x.dtype != torch.float32 or x.shape[1] != H or weight.numel() != H:
+        raise KernelError(f"rmsnorm: shapes do not fit: x {tuple(x.shape)} {x.dtype}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    if rows is not None:
+        _ints(rows, R, "norm rows")
+    elif x.shape[0] < R:
+        raise KernelError("rmsnorm: fewer input rows than output rows")
+    check(library().sp_rmsnorm(_stream(), x.data_ptr(), _ptr(rows), _code(weight, "norm weight"), weight.data_ptr(),
+                               float(eps), _code(out, "norm output"), out.data_ptr(), R, H))
+
+
+STORE, ACCUMULATE, STORE_F32 = 0, 1, 2
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: torch.Tensor | None = None,
+         accumulate: bool = False) -> None:
+    """out = a @ w.T (+ bias); with accumulate, out (float32) += a @ w.T (+ bias)."""
+    _gpu(a, "gemm input"); _gpu(w, "gemm weight"); _gpu(out, "gemm output")
+    T, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(out.shape) != (T, N):
+        raise KernelError(f"gemm: shapes do not fit: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if bias is not None:
+        _gpu(bias, "gemm bias")
+        if bias.numel() != N:
+            raise KernelError(f"gemm: bias has {bias.numel()} values for {N} columns")
+    if accumulate:
+        if out.dtype != torch.float32:
+            raise KernelError("gemm: accumulation needs a float32 output")
+        mode = ACCUMULATE
+    else:
+        mode = STORE
+    check(library().sp_gemm(_stream(), _code(a, "gemm input"), a.data_ptr(), _code(w, "gemm weight"), w.data_ptr(),
+                            _code(bias, "gemm bias") if bias is not None else 0, _ptr(bias), mode,
+                            _code(out, "gemm output"), out.data_ptr(), T, N, K))
+
+
+def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int, nq: int, nkv: int,
+               hd: int, slot_mapping: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
+               v_pool: torch.Tensor | None = None) -> None:
+    """Rotate q and k heads of qkv in place and write k, v into the pools ([pages, nkv, page, hd])."""
+    _gpu(qkv, "qkv")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (nq + 2 * nkv) * hd:
+        raise KernelError(f"rope_cache: qkv has {qkv.shape[1]} columns, expected {(nq + 2 * nkv) * hd}")
+    _ints(positions, T, "positions")
+    _gpu(inv_freq, "inv_freq")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(rotary_dim // 2, 0):
+        raise KernelError("rope_cache: inv_freq must hold rotary_dim / 2 float32 values")
+    page_size = num_pages = 0
+    if nkv:
+        _ints(slot_mapping, T, "slot_mapping")
+        for pool in (k_pool, v_pool):
+            _gpu(pool, "cache pool")
+            if pool.dtype != qkv.dtype or pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[3] != hd:
+                raise KernelError(f"rope_cache: pool {tuple(pool.shape)} {pool.dtype} does not fit nkv={nkv} hd={hd} {qkv.dtype}")
+        num_pages, _, page_size, _ = k_pool.shape
+        if tuple(v_pool.shape) != tuple(k_pool.shape):
+            raise KernelError("rope_cache: key and value pools differ in shape")
+    check(library().sp_rope_cache(_stream(), _code(qkv, "qkv"), qkv.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(),
+                                  rotary_dim, _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), T, nq, nkv, hd, page_size,
+                                  num_pages))
+
+
+def attention_tile_q(dtype: torch.dtype, hd: int, max_q_len: int, kind: int = 0) -> int:
+    return library().sp_attention_tile_q(_CODES[dtype], hd, max_q_len, kind)
+
+
+def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
+              q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, tiles: torch.Tensor, n_tiles: int,
+              tile_q: int, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
+              n_seqs: int, kind: int = 0) -> None:
+    """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h)."""
+    for t, what in ((q, "q"), (k_pool, "key pool"), (v_pool, "value pool"), (out, "attention output")):
+        _gpu(t, what)
+    T = out.shape[0]
+    if out.shape[1] != nq * hd or q.shape[0] < T or q.dtype != out.dtype or k_pool.dtype != q.dtype:
+        raise KernelError(f"attention: shapes or dtypes do not fit: q {tuple(q.shape)} {q.dtype}, out {tuple(out.shape)} {out.dtype}, pool {k_pool.dtype}")
+    if q_stride > q.shape[1] or q_stride < nq * hd:
+        raise KernelError("attention: bad q row stride")
+    if k_pool.dim() != 4 or k_pool.shape[1] != nkv or k_pool.shape[3] != hd or tuple(k_pool.shape) != tuple(v_pool.shape):
+        raise KernelError(f"attention: pool {tuple(k_pool.shape)} does not fit nkv={nkv} hd={hd}")
+    num_pages, _, page_size, _ = k_pool.shape
+    _gpu(block_tables, "block tables")
+    if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] < n_seqs:
+        raise KernelError("attention: block tables must be int32 [sequences, max_blocks]")
+    for t, what in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+        _ints(t, n_seqs, what)
+    _ints(tiles, 2 * n_tiles, "tiles")
+    check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
+                                 block_tables.data_ptr(), block_tables.shape[1], q_start.data_ptr(), q_len.data_ptr(),
+                                 ctx_len.data_ptr(), tiles.data_ptr(), n_tiles, tile_q, out.data_ptr(), nq, nkv, hd,
+                                 page_size, num_pages, int(window) if window else 0, float(scale), kind))
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = silu(gu[t, i]) * gu[t, I + i]."""
+    _gpu(gu, "gate/up"); _gpu(out, "gated output")
+    T, I = out.shape
+    if tuple(gu.shape) != (T, 2 * I) or gu.dtype != out.dtype:
+        raise KernelError(f"silu_mul: shapes do not fit: gu {tuple(gu.shape)}, out {tuple(out.shape)}")
+    check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I))
+
+
+def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
+    _gpu(src, "cast source"); _gpu(dst, "cast destination")
+    if src.numel() != dst.numel():
+        raise KernelError("cast: sizes differ")
+    check(library().sp_cast(_stream(), _code(src, "cast source"), src.data_ptr(), _code(dst, "cast destination"),
+                            dst.data_ptr(), src.numel()))
+
+
+def sample_workspace_floats(rows: int, vocab: int) -> int:
+    return library().sp_sample_workspace_floats(rows, vocab)
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, temperature: torch.Tensor | None = None,
+           seed: torch.Tensor | None = None, counter: torch.Tensor | None = None) -> None:
+    """out[r] = sampled token of row r (greedy where temperature is 0 or absent), -1 for a non-finite row."""
+    _gpu(logits, "logits"); _gpu(out, "sampled tokens"); _gpu(workspace, "sampling workspace")
+    R, V = logits.shape
+    if logits.dtype != torch.float32 or out.dtype != torch.int32 or out.numel() < R:
+        raise KernelError("sample: logits must be float32 and the output int32 with one entry per row")
+    if workspace.dtype != torch.float32 or workspace.numel() < sample_workspace_floats(R, V):
+        raise KernelError("sample: workspace too small")
+    if temperature is not None:
+        _gpu(temperature, "temperature"); _gpu(seed, "seed"); _ints(counter, R, "counter")
+        if temperature.dtype != torch.float32 or temperature.numel() < R or seed.dtype != torch.int64 or seed.numel() < R:
+            raise KernelError("sample: temperature must be float32 and seed int64, one per row")
+    check(library().sp_sample(_stream(), logits.data_ptr(), _ptr(temperature), _ptr(seed), _ptr(counter), out.data_ptr(),
+                              workspace.data_ptr(), R, V))

@@ -1,0 +1,58 @@
+"""Loads libsprout_hip.so (building it at the first call) and declares its C interface."""
+from __future__ import annotations
+
+import ctypes
+import threading
+
+_lock = threading.Lock()
+_lib = None
+
+
+class KernelError(RuntimeError):
+    """A kernel entry point refused its arguments or a launch failed."""
+
+
+def _declare(lib):
+    c_int, c_void, c_float, c_i64 = ctypes.c_int, ctypes.c_void_p, ctypes.c_float, ctypes.c_int64
+    lib.sp_last_error.restype = ctypes.c_char_p
+    lib.sp_version.restype = c_int
+    sig = {
+        "sp_embed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int],
+        "sp_rmsnorm": [c_void, c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int],
+        "sp_gemm": [c_void, c_int, c_void, c_int, c_void, c_int, c_void, c_int, c_int, c_void, c_int, c_int, c_int],
+        "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
+                          c_int, c_int, c_int],
+        "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
+                         c_int, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
+        "sp_attention_tile_q": [c_int, c_int, c_int, c_int],
+        "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int],
+        "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
+        "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_sample_workspace_floats": [c_int, c_int],
+    }
+    for name, argtypes in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+
+
+def library():
+    """The loaded library.  There is no fallback: without it the engine cannot run."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                from ..csrc.build import ensure_built
+                path = ensure_built()
+                try:
+                    lib = ctypes.CDLL(path)
+                except OSError as e:
+                    raise KernelError(f"Cannot load the HIP kernel library {path}: {e}") from None
+                _declare(lib)
+                _lib = lib
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(library().sp_last_error().decode(errors="replace"))

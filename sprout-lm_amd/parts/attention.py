@@ -1,0 +1,81 @@
+"""Grouped-query causal attention over the paged cache (reference: src/qwen.ts:167-195)."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import ops
+from ..cache.spec import PagedKVSpec
+from ..weights.loader import TensorSpec
+from .base import Mixer, register_part
+
+
+@register_part("mixer", "attention")
+class Attention(Mixer):
+    """q, k, v projections, position encoding of q and k, cache write, attention, output projection.
+
+    hidden, heads, kv_heads, head_dim: sizes.  qkv_bias / out_bias: whether the projections carry
+    biases.  position: a PositionEncoding part.  window: None for all earlier keys, else how many
+    of the latest keys a query sees.  own_kv False: the layer has no k/v projections and reads the
+    cache slot that another layer writes.
+
+    The three input projections are kept as one matrix [(heads + 2 kv_heads) * head_dim, hidden]
+    (rows of q, then k, then v), concatenated when the tensors are bound.
+    """
+
+    def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
+                 out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None):
+        if heads % kv_heads:
+            raise ValueError(f"{heads} query heads do not divide into {kv_heads} key/value heads.")
+        self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
+        self.position, self.qkv_bias, self.out_bias = position, qkv_bias, out_bias
+        self.window, self.own_kv = window, own_kv
+        self.scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
+
+    def cache_spec(self):
+        return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
+
+    def tensors(self):
+        q, kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
+        names = [("q_proj", q)] + ([("k_proj", kv), ("v_proj", kv)] if self.own_kv else [])
+        out = {}
+        for name, rows in names:
+            out[f"{name}.weight"] = TensorSpec((rows, self.hidden))
+            if self.qkv_bias:
+                out[f"{name}.bias"] = TensorSpec((rows,), "vector")
+        out["o_proj.weight"] = TensorSpec((self.hidden, q))
+        if self.out_bias:
+            out["o_proj.bias"] = TensorSpec((self.hidden,), "vector")
+        return out
+
+    def bind(self, tensors):
+        names = ["q_proj"] + (["k_proj", "v_proj"] if self.own_kv else [])
+        self.w_qkv = torch.cat([tensors[f"{n}.weight"] for n in names], dim=0).contiguous()
+        self.b_qkv = torch.cat([tensors[f"{n}.bias"] for n in names], dim=0).contiguous() if self.qkv_bias else None
+        self.w_o = tensors["o_proj.weight"]
+        self.b_o = tensors.get("o_proj.bias")
+        self.w = {}
+
+    def prepare(self, device, dtype):
+        self.position.prepare(device, dtype)
+
+    def forward(self, ctx, h, residual, cache):
+        T = h.shape[0]
+        nkv = self.kv_heads if (self.own_kv and cache.writes) else 0
+        width = (self.heads + 2 * nkv) * self.head_dim
+        qkv = ctx.buffer("qkv", (T, width), ctx.act_dtype)
+        w, b = self.w_qkv, self.b_qkv
+        if nkv == 0 and self.own_kv:   # a second call of the layer that only reads: q rows only
+            w = w[: self.heads * self.head_dim]
+            b = None if b is None else b[: self.heads * self.head_dim]
+        ops.gemm(h, w, qkv, bias=b)
+        ops.rope_cache(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim, self.heads, nkv,
+                       self.head_dim, cache.slot_mapping if nkv else None, cache.k if nkv else None,
+                       cache.v if nkv else None)
+        attn = ctx.buffer("attn", (T, self.heads * self.head_dim), ctx.act_dtype)
+        tiles, n_tiles, tile_q = ctx.attention_tiles(ctx.act_dtype, self.head_dim)
+        ops.attention(qkv, width, cache.k, cache.v, cache.block_tables, ctx.q_start, ctx.q_len, ctx.ctx_len, tiles,
+                      n_tiles, tile_q, attn, self.heads, self.kv_heads, self.head_dim, self.window, self.scale,
+                      ctx.n_seqs, kind=ctx.attention_kind)
+        ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)

@@ -1,0 +1,96 @@
+"""Interfaces of the parts a model is put together from, and the registries that name them.
+
+A part knows its own sizes and constants (constructor parameters), the tensors it needs (local
+names, `tensors()`), and how to run on a step's batch (`forward`).  It does not know which model
+it is in, which layer it is, or what its tensors are called in a checkpoint: the model plan gives
+every part a name prefix, and the runner hands it its tensors under their local names.
+"""
+from __future__ import annotations
+
+from typing import Callable
+
+from ..weights.loader import TensorSpec
+
+_REGISTRIES: dict[str, dict[str, type]] = {
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def register_part(category: str, name: str) -> Callable[[type], type]:
+    """Class decorator: make `cls` available to model plans as part `name` of `category`."""
+    if category not in _REGISTRIES:
+        raise KeyError(f"Unknown part category {category!r}; categories are {sorted(_REGISTRIES)}.")
+
+    def wrap(cls: type) -> type:
+        _REGISTRIES[category][name] = cls
+        cls.kind = name
+        return cls
+
+    return wrap
+
+
+def make_part(category: str, name: str, **params):
+    try:
+        cls = _REGISTRIES[category][name]
+    except KeyError:
+        raise KeyError(f"No {category} part named {name!r}; registered: {sorted(_REGISTRIES[category])}.") from None
+    return cls(**params)
+
+
+def registered_parts(category: str) -> list[str]:
+    return sorted(_REGISTRIES[category])
+
+
+class Part:
+    """Base of every part."""
+
+    kind = ""
+
+    def tensors(self) -> dict[str, TensorSpec]:
+        """Local tensor name -> what is expected of it."""
+        return {}
+
+    def bind(self, tensors: dict) -> None:
+        """Receive the device tensors named in `tensors()`.  Called once after loading."""
+        self.w = tensors
+
+    def prepare(self, device, dtype) -> None:
+        """Build device-side constants (tables of frequencies and the like).  Called once."""
+
+
+class Norm(Part):
+    def forward(self, ctx, x, out, rows=None):
+        """out = norm(x[rows] or x).  x is the float32 residual stream, out has the activation dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Turns positions into something a mixer applies to its queries and keys."""
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a sequence (attention, or anything with state)."""
+
+    def cache_spec(self):
+        """A PagedKVSpec, a StateSpec, or None if the mixer keeps nothing between steps."""
+        return None
+
+    def forward(self, ctx, h, residual, cache):
+        """residual += mixer(h).  `cache` is this call's cache slot (`ctx.cache_slot(...)` view) or None."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h, residual):
+        """residual += feed_forward(h), token by token."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arranges a mixer, a feed-forward and their norms around the residual stream."""
+
+    def parts(self) -> dict[str, Part]:
+        raise NotImplementedError
+
+    def forward(self, ctx, residual, cache):
+        raise NotImplementedError

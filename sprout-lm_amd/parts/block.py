@@ -1,0 +1,23 @@
+"""Arrangement of parts in a layer (reference: src/qwen.ts:164-202)."""
+from __future__ import annotations
+
+from .base import Block, register_part
+
+
+@register_part("block", "pre_norm")
+class PreNormBlock(Block):
+    """x += mixer(norm(x)); x += feed_forward(norm(x)).  The residual stream x is float32."""
+
+    def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def parts(self):
+        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ffn_norm": self.ffn_norm, "ffn": self.ffn}
+
+    def forward(self, ctx, residual, cache):
+        T, H = residual.shape
+        h = ctx.buffer("normed", (T, H), ctx.act_dtype)
+        self.mixer_norm.forward(ctx, residual, h)
+        self.mixer.forward(ctx, h, residual, cache)
+        self.ffn_norm.forward(ctx, residual, h)
+        self.ffn.forward(ctx, h, residual)

@@ -1,0 +1,36 @@
+"""Dense gated feed-forward (reference: src/qwen.ts:196-200)."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from ..weights.loader import TensorSpec
+from .base import FeedForward, register_part
+
+
+@register_part("feed_forward", "gated_mlp")
+class GatedMLP(FeedForward):
+    """down(act(gate(x)) * up(x)), no biases.  gate and up are kept as one matrix [2 * inner, hidden]."""
+
+    def __init__(self, hidden: int, inner: int, activation: str = "silu"):
+        if activation != "silu":
+            raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; only 'silu'.")
+        self.hidden, self.inner, self.activation = hidden, inner, activation
+
+    def tensors(self):
+        return {"gate_proj.weight": TensorSpec((self.inner, self.hidden)),
+                "up_proj.weight": TensorSpec((self.inner, self.hidden)),
+                "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+
+    def bind(self, tensors):
+        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        self.w_down = tensors["down_proj.weight"]
+        self.w = {}
+
+    def forward(self, ctx, h, residual):
+        T = h.shape[0]
+        gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
+        ops.gemm(h, self.w_gate_up, gu)
+        act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
+        ops.silu_mul(gu, act)
+        ops.gemm(act, self.w_down, residual, accumulate=True)

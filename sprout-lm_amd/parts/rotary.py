@@ -1,0 +1,40 @@
+"""Rotary position encoding, half-split ("neox") pairing (reference: rope, src/qwen.ts:81-92)."""
+from __future__ import annotations
+
+import torch
+
+from .base import PositionEncoding, register_part
+
+
+@register_part("position", "rotary_neox")
+class NeoxRotary(PositionEncoding):
+    """Pair (d, d + rotary_dim/2) of a head turns by position * theta^(-2d / rotary_dim).
+
+    The table of inverse frequencies is computed in float64 and kept in float32; angles, sines
+    and cosines are float32 in the kernel.
+    """
+
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
+        self.head_dim, self.theta = head_dim, theta
+        self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {head_dim}.")
+        self.inv_freq = None
+
+    def prepare(self, device, dtype):
+        d = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
+        self.inv_freq = (float(self.theta) ** (-d / self.rotary_dim)).to(torch.float32).to(device)
+
+
+@register_part("position", "none")
+class NoPosition(PositionEncoding):
+    """No position encoding: queries and keys are used as projected."""
+
+    rotary_dim = 0
+
+    def __init__(self, head_dim: int = 0):
+        self.head_dim = head_dim
+        self.inv_freq = None
+
+    def prepare(self, device, dtype):
+        self.inv_freq = torch.zeros(1, dtype=torch.float32, device=device)

@@ -1,0 +1,71 @@
+"""Engine against the plain implementation: each request alone and whole."""
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("models"))
+    return {name: H.make_model_folder(root, name) for name in H.CONFIGS}
+
+
+def make_runner(folder, name, dtype, num_blocks=64, max_sequences=8):
+    from sprout_lm_amd.engine import ModelRunner
+    return ModelRunner.from_folder(folder, dtype, block_size=H.PAGE_SIZE[name], num_blocks=num_blocks,
+                                   max_sequences=max_sequences)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_prompts_match_plain(folders, name, dtype):
+    from sprout_lm_amd.engine import StepEntry
+    runner = make_runner(folders[name], name, dtype)
+    vocab = H.CONFIGS[name]["vocab_size"]
+    for n, seed in ((1, 1), (5, 2), (17, 3), (33, 4), (70, 5)):
+        tokens = H.random_tokens(vocab, n, seed)
+        seq = runner.cache.create()
+        assert runner.cache.reserve(seq, n)
+        got = runner.step([StepEntry(seq, tokens, list(range(n)))]).cpu().numpy()
+        seq.release()
+        want = H.plain_logits(folders[name], dtype, tokens)
+        err = np.abs(got - want).max()
+        print(f"{name} {dtype} n={n}: max err {err:.3e} (scale {np.abs(want).max():.2f})")
+        assert err <= H.tolerance(dtype, want)
+    assert runner.cache.free_pages() == [64]
+
+
+def test_reference_fixture_logits_fp32(reference_fixture):
+    """The reference's own fixture: logits computed by an independent library (test/qwen.test.ts:15-46).
+
+    Head size 4 is outside what the bfloat16 kernels take; the float32 path takes any even head size.
+    """
+    import json, os
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    runner = ModelRunner.from_folder(reference_fixture, "float32", block_size=2, num_blocks=12, max_sequences=4)
+    ref = json.load(open(os.path.join(reference_fixture, "reference.json")))
+    for case in ref["cases"]:
+        # a blocker takes physical page 0 first, so the request's pages are not in order
+        blocker = runner.cache.create()
+        assert runner.cache.reserve(blocker, 1)
+        seq = runner.cache.create()
+        history = list(case["tokens"])
+        assert runner.cache.reserve(seq, 2)
+        runner.step([StepEntry(seq, history[:2], [])])
+        blocker.release()
+        assert runner.cache.reserve(seq, len(history))
+        logits = runner.step([StepEntry(seq, history[2:], [len(history) - 3])]).cpu().numpy()[0]
+        assert seq.blocks[0][:2] == [1, 0]
+        for step, name in enumerate(case["logits"]):
+            want = np.fromfile(os.path.join(reference_fixture, name), dtype="<f4")
+            assert np.abs(logits - want).max() < 1e-5      # the reference's GPU bound (test/cuda-device.integration.ts:38)
+            assert int(np.argmax(logits)) == case["output"][step]
+            if step + 1 < len(case["logits"]):
+                assert runner.cache.reserve(seq, seq.length + 1)
+                logits = runner.step([StepEntry(seq, [case["output"][step]], [0])]).cpu().numpy()[0]
+        seq.release()
+        assert runner.cache.free_pages() == [12]
