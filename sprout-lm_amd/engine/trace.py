@@ -24,6 +24,38 @@ import sys
 PAGE_TOKENS = 16
 
 
+class PoolTooSmall(RuntimeError):
+    pass
+
+
+class TraceSession:
+    """Live requests of a replay and the translation of one trace step into one engine step."""
+
+    def __init__(self, runner):
+        self.runner = runner
+        self.live = {}
+
+    def run_step(self, record):
+        """Run the step's entries as one batch, free what `end` names; returns the logits or None."""
+        from .batch import StepEntry
+        cache = self.runner.cache
+        entries = []
+        for item in record.get("entries", []):
+            seq = self.live.get(item["id"])
+            if seq is None:
+                seq = self.live[item["id"]] = cache.create()
+            tokens = [int(t) for t in item["tokens"]]
+            if not cache.reserve(seq, seq.length + len(tokens)):
+                raise PoolTooSmall(item["id"])
+            entries.append(StepEntry(seq, tokens, [int(w) for w in item.get("want", [])]))
+        logits = self.runner.step(entries) if entries else None
+        for name in record.get("end", []):
+            seq = self.live.pop(name, None)
+            if seq is not None:
+                seq.release()
+        return logits
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
     parser.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
@@ -40,7 +72,6 @@ def main(argv=None) -> int:
     print("[trace_run] loading the engine (kernels are compiled at the first call) ...", file=sys.stderr, flush=True)
     import numpy as np
     import torch
-    from .batch import StepEntry
     from .runner import ModelRunner
     from ..ops import library
     library()
@@ -51,36 +82,27 @@ def main(argv=None) -> int:
     print(f"[trace_run] ready: {runner.plan.architecture}, {args.dtype}, {num_blocks} pages of {args.block_size}",
           file=sys.stderr, flush=True)
 
-    live = {}
-    for line in sys.stdin:
+    session = TraceSession(runner)
+    while True:
+        line = sys.stdin.readline()   # one line at a time: the next step comes only after `done`
+        if not line:
+            break
         line = line.strip()
         if not line:
             continue
         record = json.loads(line)
-        step = record["step"]
-        entries = []
-        for item in record.get("entries", []):
-            seq = live.get(item["id"])
-            if seq is None:
-                seq = live[item["id"]] = runner.cache.create()
-            tokens = [int(t) for t in item["tokens"]]
-            if not runner.cache.reserve(seq, seq.length + len(tokens)):
-                print(f"[trace_run] step {step}: the cache pool of {args.max_tokens} tokens is too small for "
-                      f"request {item['id']!r}", file=sys.stderr, flush=True)
-                return 1
-            entries.append(StepEntry(seq, tokens, [int(w) for w in item.get("want", [])]))
-        if entries:
-            logits = runner.step(entries)
-            if logits.shape[0]:
-                host = logits.to("cpu", copy=True).numpy().astype("<f4", copy=False)
-                host.tofile(os.path.join(args.out, f"{step}.f32"))
-            else:
-                torch.cuda.current_stream().synchronize()
-        for name in record.get("end", []):
-            seq = live.pop(name, None)
-            if seq is not None:
-                seq.release()
-        print(f"done {step}", flush=True)
+        try:
+            logits = session.run_step(record)
+        except PoolTooSmall as e:
+            print(f"[trace_run] step {record['step']}: the cache pool of {args.max_tokens} tokens is too small "
+                  f"for request {e.args[0]!r}", file=sys.stderr, flush=True)
+            return 1
+        if logits is not None and logits.shape[0]:
+            host = logits.to("cpu", copy=True).numpy().astype("<f4", copy=False)
+            host.tofile(os.path.join(args.out, f"{record['step']}.f32"))
+        else:
+            torch.cuda.current_stream().synchronize()
+        print(f"done {record['step']}", flush=True)
     return 0
 
 
