@@ -157,14 +157,19 @@ class CacheManager:
             end += bs
         return seq
 
-    def publish(self, tokens, seq: SequenceCache) -> None:
-        """Offer the last full page of `seq` (whose tokens are `tokens`) for reuse; the first publisher wins."""
-        if not self.prefix_caching or seq.released or seq.length == 0 or seq.length % self.block_size:
+    def publish(self, tokens, seq: SequenceCache, length: int | None = None) -> None:
+        """Offer the full page of `seq` that ends at `length` (default: its computed length) for reuse.
+
+        `tokens[:length]` are the tokens computed so far; the first publisher of a prefix wins
+        (reference: src/kv-cache.ts:114-123).
+        """
+        length = seq.length if length is None else length
+        if not self.prefix_caching or seq.released or length == 0 or length % self.block_size:
             return
-        if len(tokens) != seq.length:
-            raise ValueError("Prefix tokens must match the computed length.")
+        if len(tokens) < length or length > seq.length:
+            raise ValueError("Prefix tokens must cover the published length, which must be computed.")
         bs = self.block_size
-        n_pages = seq.length // bs
+        n_pages = length // bs
         while len(seq.prefix_keys) < n_pages:
             i = len(seq.prefix_keys)
             parent = seq.prefix_keys[-1] if seq.prefix_keys else b""

@@ -1,0 +1,303 @@
+"""Each kernel alone against a plain float64 computation, at other sizes than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def t(x, dtype=torch.float32):
+    return torch.as_tensor(np.asarray(x)).to(DEV).to(dtype).contiguous()
+
+
+def bf16(x):
+    return torch.as_tensor(np.asarray(x, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+
+
+@pytest.mark.parametrize("T,N,K", [(1, 1, 1), (1, 37, 33), (3, 130, 31), (5, 64, 1025), (17, 151, 96), (64, 100, 70),
+                                   (77, 300, 129), (200, 96, 224), (130, 257, 511)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T * 1000 + N + K)
+    a, w, b = rng.standard_normal((T, K)), rng.standard_normal((N, K)) / math.sqrt(K), rng.standard_normal(N)
+    if dtype == torch.bfloat16:
+        a, w, b = bf16(a), bf16(w), bf16(b)
+    want = a.astype(np.float64) @ w.astype(np.float64).T
+    tol = 1e-5 * max(1, math.sqrt(K) / 8) if dtype == torch.float32 else 2e-2
+    A, W, B = t(a, dtype), t(w, dtype), t(b, dtype)
+    out = torch.empty(T, N, dtype=dtype, device=DEV)
+    ops.gemm(A, W, out, bias=B)
+    assert np.abs(out.float().cpu().numpy() - (want + b)).max() <= tol * (1 + np.abs(want).max())
+    out32 = torch.empty(T, N, dtype=torch.float32, device=DEV)
+    ops.gemm(A, W, out32)                                   # float32 result of bfloat16 operands is not rounded
+    assert np.abs(out32.cpu().numpy() - want).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
+    base = rng.standard_normal((T, N)).astype(np.float32)
+    acc = t(base)
+    ops.gemm(A, W, acc, accumulate=True)                    # the residual sum is float32
+    assert np.abs(acc.cpu().numpy() - (base + want)).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
+
+
+def test_gemm_mixed_operand_dtypes_and_refusals():
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(0)
+    a, w = bf16(rng.standard_normal((9, 40))), rng.standard_normal((21, 40)).astype(np.float32)
+    out = torch.empty(9, 21, dtype=torch.float32, device=DEV)
+    ops.gemm(t(a, torch.bfloat16), t(w), out)               # a weight stored in 32-bit stays so
+    assert np.abs(out.cpu().numpy() - a.astype(np.float64) @ w.astype(np.float64).T).max() < 1e-4
+    with pytest.raises(ops.KernelError):
+        ops.gemm(t(a, torch.bfloat16), t(w[:, :39]), out)
+    with pytest.raises(ops.KernelError):
+        ops.gemm(t(a, torch.bfloat16).cpu(), t(w), out)     # no CPU path
+    with pytest.raises(ops.KernelError):
+        ops.gemm(t(a, torch.bfloat16), t(w), torch.empty(9, 21, dtype=torch.bfloat16, device=DEV), accumulate=True)
+
+
+@pytest.mark.parametrize("H", [1, 24, 96, 896, 1000, 5120])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(H, out_dtype):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(H)
+    x = (rng.standard_normal((7, H)) * 3).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, H).astype(np.float32)
+    for eps in (1e-6, 1e-2):
+        want = x / np.sqrt((x.astype(np.float64) ** 2).mean(-1, keepdims=True) + eps) * w
+        out = torch.empty(7, H, dtype=out_dtype, device=DEV)
+        ops.rmsnorm(t(x), t(w), eps, out)
+        tol = 2e-6 if out_dtype == torch.float32 else 2 ** -8
+        assert np.abs(out.float().cpu().numpy() - want).max() <= tol * (1 + np.abs(want).max())
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    out = torch.empty(3, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(t(x), t(w), 1e-6, out, rows=rows)
+    full = torch.empty(7, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(t(x), t(w), 1e-6, full)
+    assert torch.equal(out, full[[5, 0, 5]])
+    zero = torch.empty(2, H, dtype=torch.float32, device=DEV)
+    ops.rmsnorm(torch.zeros(2, H, device=DEV), t(w), 1e-6, zero)
+    assert torch.all(zero == 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_and_silu_mul_and_cast(dtype):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(1)
+    table = rng.standard_normal((331, 70)).astype(np.float32)
+    tokens = torch.tensor([330, 0, 7, 7, 128], dtype=torch.int32, device=DEV)
+    res = torch.empty(5, 70, dtype=torch.float32, device=DEV)
+    ops.embed(t(table, dtype), tokens, res)
+    assert torch.equal(res, t(table, dtype).float()[tokens.long()])
+    gu = rng.standard_normal((6, 2 * 333)).astype(np.float32) * 4
+    if dtype == torch.bfloat16:
+        gu = bf16(gu)
+    g, u = gu[:, :333].astype(np.float64), gu[:, 333:].astype(np.float64)
+    out = torch.empty(6, 333, dtype=dtype, device=DEV)
+    ops.silu_mul(t(gu, dtype), out)
+    want = g / (1 + np.exp(-g)) * u
+    tol = 1e-6 if dtype == torch.float32 else 2 ** -8
+    assert np.abs(out.float().cpu().numpy() - want).max() <= tol * (1 + np.abs(want).max())
+    src = t(rng.standard_normal(1001).astype(np.float32))
+    dst = torch.empty(1001, dtype=torch.bfloat16, device=DEV)
+    ops.cast(src, dst)
+    assert torch.equal(dst, src.to(torch.bfloat16))
+
+
+def plain_rope(x, pos, hd, rotary, theta):
+    x = x.astype(np.float64).copy()
+    half = rotary // 2
+    heads = x.shape[1] // hd
+    d = np.arange(half)
+    ang = pos[:, None] * theta ** (-2.0 * d / rotary)
+    for h in range(heads):
+        a, b = x[:, h * hd:h * hd + half].copy(), x[:, h * hd + half:h * hd + rotary].copy()
+        x[:, h * hd:h * hd + half] = a * np.cos(ang) - b * np.sin(ang)
+        x[:, h * hd + half:h * hd + rotary] = b * np.cos(ang) + a * np.sin(ang)
+    return x
+
+
+@pytest.mark.parametrize("nq,nkv,hd,rotary,page", [(4, 2, 16, 16, 16), (3, 1, 32, 32, 8), (5, 5, 48, 48, 4), (7, 1, 64, 32, 32),
+                                                   (2, 2, 128, 128, 16), (1, 1, 6, 6, 2)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_and_cache_write(nq, nkv, hd, rotary, page, dtype):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(nq * 100 + hd)
+    T, pages, theta = 11, 9, 10000.0
+    qkv = rng.standard_normal((T, (nq + 2 * nkv) * hd)).astype(np.float32)
+    if dtype == torch.bfloat16:
+        qkv = bf16(qkv)
+    pos = rng.integers(0, 500, T)
+    slots = rng.permutation(pages * page)[:T].astype(np.int32)
+    slots[3] = -1                                           # a token whose keys are not written
+    inv = torch.tensor(theta ** (-2.0 * np.arange(rotary // 2) / rotary), dtype=torch.float32, device=DEV)
+    Q = t(qkv, dtype)
+    kp = torch.zeros(pages, nkv, page, hd, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    ops.rope_cache(Q, torch.tensor(pos, dtype=torch.int32, device=DEV), inv, rotary, nq, nkv, hd,
+                   torch.tensor(slots, device=DEV), kp, vp)
+    want_qk = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, rotary, theta)
+    tol = 2e-4 if dtype == torch.float32 else 2 ** -7       # float32 angles of positions up to 500
+    got = Q.float().cpu().numpy()
+    assert np.abs(got[:, :(nq + nkv) * hd] - want_qk).max() <= tol * 4
+    assert np.array_equal(got[:, (nq + nkv) * hd:], qkv[:, (nq + nkv) * hd:])
+    kp, vp = kp.float().cpu().numpy(), vp.float().cpu().numpy()
+    written = np.zeros((pages, page), bool)
+    for i in range(T):
+        if slots[i] < 0:
+            continue
+        pg, off = divmod(int(slots[i]), page)
+        written[pg, off] = True
+        for g in range(nkv):
+            assert np.array_equal(kp[pg, g, off], got[i, (nq + g) * hd:(nq + g + 1) * hd])
+            assert np.array_equal(vp[pg, g, off], qkv[i, (nq + nkv + g) * hd:(nq + nkv + g + 1) * hd])
+    unwritten = ~written[:, None, :, None]                   # pools are [pages, groups, page, head size]
+    assert np.all((kp == 0) | ~unwritten) and np.all((vp == 0) | ~unwritten)
+
+
+def plain_attention(q, keys, values, nq, nkv, hd, first_pos, window, scale):
+    """q [n, nq*hd] at positions first_pos..; keys/values [ctx, nkv*hd]."""
+    out = np.zeros_like(q, dtype=np.float64)
+    for i in range(q.shape[0]):
+        p = first_pos + i
+        lo = 0 if not window else max(0, p - window + 1)
+        for h in range(nq):
+            g = h // (nq // nkv)
+            s = keys[lo:p + 1, g * hd:(g + 1) * hd] @ q[i, h * hd:(h + 1) * hd] * scale
+            e = np.exp(s - s.max())
+            out[i, h * hd:(h + 1) * hd] = (e / e.sum()) @ values[lo:p + 1, g * hd:(g + 1) * hd]
+    return out
+
+
+def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=None, seed=0):
+    """seqs: list of (ctx_len, q_len).  Pages are scattered over the pool in random order."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(seed)
+    n_pages = sum(-(-c // page) for c, _ in seqs) + 3
+    order = list(rng.permutation(n_pages))
+    kp = rng.standard_normal((n_pages, nkv, page, hd)).astype(np.float32)     # unused slots hold noise, not zeros
+    vp = rng.standard_normal((n_pages, nkv, page, hd)).astype(np.float32)
+    if dtype == torch.bfloat16:
+        kp, vp = bf16(kp), bf16(vp)
+    T = sum(q for _, q in seqs)
+    q = rng.standard_normal((T, nq * hd)).astype(np.float32)
+    max_blocks = max(-(-c // page) for c, _ in seqs) + 1
+    tables = np.full((len(seqs), max_blocks), -1, np.int32)
+    keys, values, starts = [], [], []
+    t0 = 0
+    for s, (ctx, qlen) in enumerate(seqs):
+        blocks = [order.pop() for _ in range(-(-ctx // page))]
+        tables[s, :len(blocks)] = blocks
+        k = np.concatenate([kp[b].transpose(1, 0, 2).reshape(page, nkv * hd) for b in blocks])[:ctx]
+        v = np.concatenate([vp[b].transpose(1, 0, 2).reshape(page, nkv * hd) for b in blocks])[:ctx]
+        if spike is not None and s == spike[0]:
+            # one far key stands out for the last query: its score dominates, so missing it shows
+            _, far = spike
+            k[far] *= 0.0
+            k[far, :hd] = 6.0
+            q[t0 + qlen - 1, :] = 0.0
+            for h in range(nq):
+                q[t0 + qlen - 1, h * hd:h * hd + hd] = 3.0 if h // (nq // nkv) == 0 else 0.1
+            pg, off = divmod(far, page)
+            kp[blocks[pg], :, off, :] = k[far].reshape(nkv, hd)
+        if dtype == torch.bfloat16:
+            k, v = bf16(k), bf16(v)
+        keys.append(k); values.append(v); starts.append(t0)
+        t0 += qlen
+    if dtype == torch.bfloat16:
+        q, kp = bf16(q), bf16(kp)
+    tile_q = ops.attention_tile_q(dtype, hd, max(ql for _, ql in seqs), kind)
+    tiles = np.asarray([(s, off) for s, (_, ql) in enumerate(seqs) for off in range(0, ql, tile_q)], np.int32)
+    out = torch.full((T, nq * hd), float("nan"), dtype=dtype, device=DEV)
+    scale = 1 / math.sqrt(hd)
+    ops.attention(t(q, dtype), nq * hd, t(kp, dtype), t(vp, dtype), t(tables, torch.int32), t(starts, torch.int32),
+                  t([ql for _, ql in seqs], torch.int32), t([c for c, _ in seqs], torch.int32), t(tiles, torch.int32),
+                  len(tiles), tile_q, out, nq, nkv, hd, window, scale, len(seqs), kind=kind)
+    got = out.float().cpu().numpy()
+    want = np.concatenate([plain_attention(q[starts[s]:starts[s] + ql].astype(np.float64), keys[s].astype(np.float64),
+                                           values[s].astype(np.float64), nq, nkv, hd, c - ql, window, scale)
+                           for s, (c, ql) in enumerate(seqs)])
+    return got, want
+
+
+ATT_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 8), (5, 5, 48, 16), (14, 2, 64, 16), (8, 2, 128, 32), (6, 3, 80, 4), (2, 1, 256, 16)]
+ATT_BATCHES = [[(1, 1)], [(17, 17)], [(70, 1), (33, 33), (9, 2), (130, 5)], [(300, 300)], [(513, 1), (64, 64), (257, 2)]]
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page", ATT_SHAPES)
+@pytest.mark.parametrize("batch", range(len(ATT_BATCHES)))
+@pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
+def test_attention_mixed_batches(nq, nkv, hd, page, batch, dtype, kind):
+    got, want = run_attention(dtype, nq, nkv, hd, page, ATT_BATCHES[batch], kind=kind, seed=batch)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
+@pytest.mark.parametrize("window", [1, 5, 16, 33, 100])
+def test_attention_window_edges(dtype, kind, window):
+    got, want = run_attention(dtype, 4, 2, 32, 8, [(90, 1), (90, 40), (7, 7), (200, 3)], window=window, kind=kind, seed=window)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
+@pytest.mark.parametrize("far", [0, 15, 16, 255, 256, 640, 699])
+def test_attention_finds_one_far_key_among_hundreds(dtype, kind, far):
+    """One key's score dominates; the output of the last query is that key's value row."""
+    got, want = run_attention(dtype, 4, 2, 64, 16, [(700, 1), (700, 9)], kind=kind, spike=(1, far), seed=far)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+def test_attention_refuses_what_it_cannot_take():
+    from sprout_lm_amd import ops
+    q = torch.zeros(1, 4 * 16, device=DEV)
+    pool = torch.zeros(2, 3, 16, 16, device=DEV)
+    ints = torch.zeros(4, dtype=torch.int32, device=DEV)
+    table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    with pytest.raises(ops.KernelError, match="groups"):
+        ops.attention(q, 64, pool, pool, table, ints, ints, ints, ints, 1, 16, torch.empty_like(q), 4, 3, 16, None, 0.25, 1, kind=1)
+    big = torch.zeros(1, 512, device=DEV)
+    pool = torch.zeros(2, 1, 16, 512, device=DEV)
+    with pytest.raises(ops.KernelError, match="head size"):
+        ops.attention(big, 512, pool, pool, table, ints, ints, ints, ints, 1, 16, torch.empty_like(big), 1, 1, 512, None, 0.1, 1, kind=1)
+
+
+def test_sampling_greedy_ties_nonfinite_and_temperature():
+    from sprout_lm_amd import ops
+    V = 151936 // 8 + 13
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((5, V)).astype(np.float32)
+    logits[1, [70, 9000, 18000]] = 9.0                      # ties: the lowest index wins
+    logits[2, 555] = np.nan
+    logits[3, V - 1] = 50.0
+    logits[4, 17] = np.inf
+    L = t(logits)
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ws = torch.empty(ops.sample_workspace_floats(5, V), device=DEV)
+    ops.sample(L, out, ws)
+    assert out.tolist() == [int(np.argmax(logits[0])), 70, -1, V - 1, -1]
+    # temperature: reproducible, keyed by (seed, counter), and distributed as softmax(logits / T)
+    small = np.log(np.array([[0.5, 0.25, 0.125, 0.125]], np.float32)).repeat(4000, 0)
+    S = t(small)
+    temp = torch.full((4000,), 1.0, device=DEV)
+    seed = torch.full((4000,), 42, dtype=torch.int64, device=DEV)
+    counter = torch.arange(4000, dtype=torch.int32, device=DEV)
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    ws = torch.empty(ops.sample_workspace_floats(4000, 4), device=DEV)
+    ops.sample(S, out, ws, temp, seed, counter)
+    first = out.clone()
+    ops.sample(S, out, ws, temp, seed, counter)
+    assert torch.equal(first, out)
+    freq = np.bincount(first.cpu().numpy(), minlength=4) / 4000
+    assert np.abs(freq - [0.5, 0.25, 0.125, 0.125]).max() < 0.03
+    ops.sample(S, out, ws, temp, seed + 1, counter)
+    assert not torch.equal(first, out)
+    # row r of a batch draws what it would draw alone
+    ops.sample(S[10:11].contiguous(), out[:1], ws, temp[:1], seed[:1], counter[10:11].contiguous())
+    assert out[0].item() == first[10].item()
+    cold = torch.full((4000,), 0.05, device=DEV)
+    ops.sample(S, out, ws, cold, seed, counter)
+    assert (out == 0).float().mean().item() > 0.99

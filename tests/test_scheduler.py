@@ -1,0 +1,191 @@
+"""The scheduler's decisions, on the CPU with a stand-in model (reference: test/engine.test.ts, test/qwen.test.ts:48-117)."""
+import pytest
+
+from sprout_lm_amd.engine import Engine
+from tests.fake_model import ArgmaxSampler, FakeRunner
+
+
+def make(block_size=4, num_blocks=64, max_sequences=4, prefix_caching=True, eos=(), **options):
+    runner = FakeRunner(block_size, num_blocks, max_sequences, prefix_caching, eos)
+    options.setdefault("max_batch_tokens", 8)
+    options.setdefault("prefill_chunk_size", 4)
+    options.setdefault("record_trace", True)
+    return Engine(runner, sampler=ArgmaxSampler(), prefix_caching=prefix_caching, **options)
+
+
+def drain(engine, limit=2000):
+    reports = []
+    while engine.pending:
+        assert len(reports) < limit, "scheduler must make progress"
+        report = engine.step()
+        assert sum(w["tokens"] for w in report.work) <= engine.options.max_batch_tokens
+        assert all(p["refs"] >= 0 and p["active_refs"] >= 0 for p in report.memory["pages"])
+        reports.append(report)
+    return reports
+
+
+def prompt(text):
+    return [ord(c) % 50 for c in text]
+
+
+def test_late_request_joins_and_decode_mixes_with_chunked_prefill():
+    engine = make(max_batch_tokens=6, prefill_chunk_size=3, max_sequences=3)
+    prompts = [prompt("a"), prompt("longer prompt"), prompt("late")]
+    engine.add("A", prompts[0], 6)
+    engine.add("B", prompts[1], 3)
+    engine.step()
+    engine.add("C", prompts[2], 2)
+    reports = drain(engine)
+    assert any({w["phase"] for w in r.work} >= {"decode", "prefill"} for r in reports)
+    for rid, p, n in zip("ABC", prompts, (6, 3, 2)):
+        result = engine.result(rid)
+        assert result["status"] == "finished" and result["finish_reason"] == "length"
+        assert result["output"] == engine.model.greedy(p, n)
+    kinds = [(e["id"], e["type"]) for e in engine.trace]
+    assert kinds.index(("C", "admitted")) < kinds.index(("B", "finished"))
+    assert max(engine.model.steps) <= 6
+
+
+def test_decode_goes_first_and_budget_cuts_prompts():
+    engine = make(max_batch_tokens=5, prefill_chunk_size=4, max_sequences=3)
+    engine.add("A", prompt("ab"), 4)
+    engine.step()                                  # A prefilled (2 tokens) and sampled
+    engine.add("B", prompt("0123456789"), 1)
+    report = engine.step()
+    assert [(w["id"], w["phase"], w["from"], w["tokens"]) for w in report.work] == [("A", "decode", 2, 1), ("B", "prefill", 0, 4)]
+    report = engine.step()
+    assert [(w["id"], w["from"], w["tokens"]) for w in report.work] == [("A", 3, 1), ("B", 4, 4)]
+    drain(engine)
+
+
+def test_prefix_sharing_reuses_pages_and_recomputes_the_last_prompt_token():
+    engine = make(block_size=2, prefill_chunk_size=8)
+    p = prompt("abcd")                             # exactly two full pages
+    engine.add("A", p, 4)
+    engine.step()
+    a_pages = engine.result("A")["block_table"]
+    engine.add("B", p, 4)
+    report = engine.step()
+    assert engine.result("B")["prefix_hits"] == 2
+    assert engine.result("B")["block_table"][0] == a_pages[0]
+    assert report.memory["pages"][a_pages[0]]["active_refs"] == 2
+    drain(engine)
+    assert engine.result("A")["output"] == engine.result("B")["output"] == engine.model.greedy(p, 4)
+    assert all(page["active_refs"] == 0 for page in engine.cache.snapshot()["pages"])
+    engine.cache.clear_prefixes()
+    assert engine.cache.free_pages() == [engine.options.num_blocks]
+
+
+def test_same_suffix_under_another_context_does_not_hit():
+    engine = make(block_size=2, prefill_chunk_size=8)
+    engine.add("A", [1, 2, 3, 4, 5], 1)
+    drain(engine)
+    engine.add("B", [9, 8, 3, 4, 5], 1)
+    drain(engine)
+    assert engine.result("B")["prefix_hits"] == 0
+    assert engine.result("B")["output"] == engine.model.greedy([9, 8, 3, 4, 5], 1)
+
+
+@pytest.mark.parametrize("prefix_caching", [False, True])
+def test_pressure_preempts_and_recomputes_without_changing_outputs(prefix_caching):
+    engine = make(block_size=2, num_blocks=5, max_batch_tokens=6, prefill_chunk_size=2, prefix_caching=prefix_caching)
+    prompts = [prompt("aa"), prompt("bb"), prompt("cc")]
+    for i, p in enumerate(prompts):
+        engine.add(str(i), p, 7)
+    reports = drain(engine)
+    assert any(e["type"] == "preempted" for e in engine.trace)
+    assert any(w["phase"] == "recompute" for r in reports for w in r.work)
+    for i, p in enumerate(prompts):
+        assert engine.result(str(i))["output"] == engine.model.greedy(p, 7)
+    assert engine.stats()["preemptions"] > 0 and engine.stats()["recomputed_tokens"] > 0
+    engine.cache.clear_prefixes()
+    assert engine.cache.free_pages() == [5]
+
+
+def test_when_pages_run_out_the_youngest_steps_back_and_the_oldest_never_does():
+    engine = make(block_size=2, num_blocks=4, max_batch_tokens=8, prefill_chunk_size=4, prefix_caching=False)
+    engine.add("old", prompt("abcd"), 4)
+    engine.add("young", prompt("efgh"), 4)
+    drain(engine)
+    preempted = [e["id"] for e in engine.trace if e["type"] == "preempted"]
+    assert preempted and set(preempted) == {"young"}
+    assert engine.result("old")["preemptions"] == 0
+    # a request preempted while the step was planned brought no tokens to that step
+    for e in engine.trace:
+        if e["type"] == "preempted":
+            tick_tokens = [t for t in engine.trace if t["tick"] == e["tick"] and t["id"] == e["id"] and t["type"] == "token"]
+            assert not tick_tokens
+    assert engine.result("young")["output"] == engine.model.greedy(prompt("efgh"), 4)
+
+
+def test_cancel_running_and_queued_requests_without_hurting_a_sibling():
+    engine = make(block_size=2, max_sequences=2)
+    p = prompt("abc")
+    engine.add("A", p, 5)
+    engine.step()
+    engine.add("B", p, 5)
+    engine.step()
+    engine.add("queued", p, 1)
+    assert engine.cancel("A") and engine.cancel("queued") and not engine.cancel("A")
+    drain(engine)
+    assert engine.result("A")["status"] == "cancelled" and engine.result("queued")["status"] == "cancelled"
+    assert engine.result("B")["output"] == engine.model.greedy(p, 5)
+    assert engine.forget("A") and not engine.forget("A")
+    engine.cache.clear_prefixes()
+    assert engine.cache.free_pages() == [engine.options.num_blocks]
+
+
+def test_eos_is_emitted_once_counted_and_frees_pages_before_the_limit():
+    probe = make()
+    first = probe.model.greedy([1, 2], 1)[0]
+    engine = make(block_size=2, num_blocks=4, eos=(first,))
+    events = list(engine.stream([1, 2], max_new_tokens=5))
+    assert [e["token"] for e in events if e["type"] == "token"] == [first]
+    assert events[-1] == {"id": events[0]["id"], "type": "finished", "finish_reason": "eos",
+                          "usage": {"prompt_tokens": 2, "completion_tokens": 1}}
+    assert all(page["active_refs"] == 0 for page in engine.cache.snapshot()["pages"])
+    # ignore_eos runs to the length limit
+    engine.add("x", [1, 2], 3, ignore_eos=True)
+    drain(engine)
+    assert engine.result("x")["finish_reason"] == "length" and len(engine.result("x")["output"]) == 3
+
+
+def test_invalid_inputs_and_requests_that_cannot_fit():
+    with pytest.raises(Exception, match="positive integer"):
+        make(max_batch_tokens=0)
+    engine = make(block_size=2, num_blocks=1, max_sequences=1)
+    for bad, pattern in (([], "valid token"), ([-1], "valid token"), ([50], "valid token")):
+        with pytest.raises(ValueError, match=pattern):
+            engine.add("x", bad, 1)
+    with pytest.raises(ValueError, match="positive integer"):
+        engine.add("x", [1], 0)
+    with pytest.raises(ValueError, match="cannot fit"):
+        engine.add("x", [1, 2], 2)
+    with pytest.raises(ValueError, match="context limit"):
+        make(num_blocks=64).add("x", [1], 65)
+    engine.add("x", [1, 2], 1)
+    with pytest.raises(ValueError, match="unique"):
+        engine.add("x", [1], 1)
+    drain(engine)
+
+
+def test_a_failing_step_ends_every_request_and_returns_every_page():
+    engine = make(block_size=2, num_blocks=8)
+    engine.add("A", prompt("abcd"), 4)
+    engine.add("B", prompt("abcd"), 4)
+    engine.step()
+
+    def broken(entries):
+        raise RuntimeError("device lost")
+    engine.model.step = broken
+    with pytest.raises(RuntimeError, match="device lost"):
+        engine.step()
+    assert not engine.pending
+    assert engine.result("A")["status"] == engine.result("B")["status"] == "cancelled"
+    assert engine.cache.free_pages() == [8]
+
+
+def test_generate_returns_outputs_in_order():
+    engine = make(max_sequences=2)
+    prompts = [prompt("one"), prompt("second"), prompt("3")]
+    assert engine.generate(prompts, max_new_tokens=3) == [engine.model.greedy(p, 3) for p in prompts]
