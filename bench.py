@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Default: Qwen2.5-0.5B layer sizes (BASELINE.json configs[2]) with random weights, bfloat16, a batch
+of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
+(scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
+MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
+
+
+def weight_bytes_per_step(cfg, element: int) -> int:
+    """Every weight a decode step uses, read once (the embedding rows it gathers are negligible)."""
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    layer = H * (Q + 2 * KV) + (Q + 2 * KV) + Q * H + 3 * H * I + 2 * H
+    return (L * layer + V * H + H) * element
+
+
+def kv_bytes(cfg, batch: int, context: int, element: int) -> int:
+    KV = cfg.num_key_value_heads * cfg.head_dim
+    return batch * context * 2 * cfg.num_hidden_layers * KV * element
+
+
+def prefill_flops(cfg, T: int) -> float:
+    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
+    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    linear = 2.0 * T * L * (H * (Q + 2 * KV) + Q * H + 3 * H * I)
+    attention = 2.0 * L * Q * T * T          # causal: half of 4 Q T^2
+    return linear + attention + 2.0 * V * H  # logits of the last position only
+
+
+def make_engine(cfg, dtype, batch, context, layers_note):
+    from sprout_lm_amd.engine import Engine
+    pages_per_request = -(-context // 16)
+    return Engine.from_config(cfg, seed=0, dtype=dtype, block_size=16, num_blocks=batch * (pages_per_request + 1),
+                              max_sequences=batch, max_batch_tokens=max(2048, batch), prefill_chunk_size=2048,
+                              prefix_caching=False, record_trace=False)
+
+
+def measure_decode(engine, cfg, batch, context, steps, warmup):
+    """`batch` requests decode together; the timed steps end exactly at `context` tokens."""
+    import random
+    import torch
+    rng = random.Random(batch)
+    # requests that finish their prompt early decode while the others still prefill: leave them room
+    slack = -(-batch * context // engine.options.max_batch_tokens) + 2
+    prompt_len = context - (steps + warmup) - slack
+    for i in range(batch):
+        prompt = [rng.randrange(cfg.vocab_size) for _ in range(prompt_len)]
+        engine.add(f"b{batch}-{i}", prompt, steps + warmup + slack + 1, ignore_eos=True)
+    # prefill everything (the last prompt token's step samples the first output)
+    while any(not r.output for r in engine.scheduler.requests.values()):
+        engine.step()
+    for _ in range(warmup - 1):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        report = engine.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert len(report.work) == batch and all(w["phase"] == "decode" for w in report.work), "timed steps must decode"
+    for rid in list(engine.scheduler.requests):
+        engine.cancel(rid)
+        engine.forget(rid)
+    return elapsed / steps
+
+
+def measure_prefill(engine, cfg, tokens, repeats=3):
+    import random
+    import torch
+    rng = random.Random(1)
+    best = None
+    for r in range(repeats + 1):
+        prompt = [rng.randrange(cfg.vocab_size) for _ in range(tokens)]
+        engine.add(f"p{r}", prompt, 1, ignore_eos=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while engine.pending:
+            engine.step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        engine.forget(f"p{r}")
+        if r > 0:
+            best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=4096)
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (named in config)")
+    parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    parser.add_argument("--preset", default="qwen2.5-0.5b")
+    parser.add_argument("--prefill-tokens", type=int, default=2048)
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs.")
+        return 2
+
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.registry import config_from_dict
+    raw = dict(PRESETS[args.preset])
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(raw)
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+    element = 2 if args.dtype == "bf16" else 4
+
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    engine = make_engine(cfg, dtype, biggest, args.context, None)
+    warmup = max(args.warmup, 1)
+
+    step_s = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
+            points[f"decode_b{b}"] = round(b / s, 1)
+    prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
+
+    read = weight_bytes_per_step(cfg, element) + kv_bytes(cfg, args.batch, args.context, element)
+    achieved = read / step_s / 1e9
+    flops = prefill_flops(cfg, args.prefill_tokens)
+    value = args.batch / step_s
+    line = {
+        "metric": "decode tok/s at batch 8 (Qwen2.5-0.5B sizes, context 4096); prefill tok/s at 2,048 tokens; % roofline",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": warmup,
+        "ms_per_step": round(step_s * 1000, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
+        "config": {"model": f"{args.preset} sizes, random weights", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": cfg.num_hidden_layers, "layers_of_configuration": full_layers,
+                   "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+                   "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "vocab_size": cfg.vocab_size, "tied_embeddings": cfg.tie_word_embeddings, "page_size": 16,
+                   "prefill_tokens": args.prefill_tokens, "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps},
+        "prefill": {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
+                    "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / MFMA_PEAK[args.dtype], 5)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 5)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

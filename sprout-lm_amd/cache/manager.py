@@ -23,7 +23,7 @@ class PagedGroup:
     slots: list[int]              # cache slot ids that live in this group, in pool order
     pool: PagePool
     k: object = None              # device tensor [len(slots), pages, kv_heads, page_size, head_dim]
-    v: object = None
+    v: object = None              # device tensor [len(slots), pages, kv_heads, head_dim, page_size]
 
 
 @dataclass
@@ -101,9 +101,11 @@ class CacheManager:
         """Allocate the pools on the device.  Host-only users (tests, planning) never call this."""
         import torch
         for g in self.groups:
-            shape = (len(g.slots), self.num_blocks, g.spec.kv_heads, self.block_size, g.spec.head_dim)
-            g.k = torch.zeros(shape, dtype=dtype, device=device)
-            g.v = torch.zeros(shape, dtype=dtype, device=device)
+            # keys [slot, page, head, token, dim]; values [slot, page, head, dim, token]: the keys of one
+            # dimension lie together, which is how the P.V matrix product reads them
+            n, kv, hd = len(g.slots), g.spec.kv_heads, g.spec.head_dim
+            g.k = torch.zeros((n, self.num_blocks, kv, self.block_size, hd), dtype=dtype, device=device)
+            g.v = torch.zeros((n, self.num_blocks, kv, hd, self.block_size), dtype=dtype, device=device)
         for g in self.state_groups:
             g.data = torch.zeros((len(g.slots), self.max_sequences, *g.spec.shape),
                                  dtype=getattr(torch, g.spec.dtype), device=device)

@@ -7,26 +7,75 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale);
+bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
+bool attention_mfma_decode_supports(int nq, int nkv);
+int attention_mfma_tile_q(int hd);
+size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx);
+int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                   const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                   const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
+                   int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int hd, int page_size,
+                   int num_pages, int window, float scale);
 }  // namespace sprout
 
 using namespace sprout;
 
 // kernel_kind: 0 = the engine's choice, 1 = the float32-arithmetic kernel.
-extern "C" int sp_attention_tile_q(int dtype, int hd, int max_q_len, int kernel_kind) { return 16; }
+static bool use_mfma(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind) {
+  return kernel_kind == 0 && dtype == kBF16 && nkv > 0 && nq % nkv == 0 && attention_mfma_supports(hd, page_size, nq, nkv);
+}
+
+// What the chosen kernel wants of the caller.
+//   plan[0]: queries per tile of the tile list
+//   plan[1]: 1 if the tile list holds every sequence, 0 if only sequences with more than one query
+//            (the others are then given as `decode_seqs`)
+extern "C" int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind, int* plan) {
+  if (use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind)) {
+    plan[0] = attention_mfma_tile_q(hd);
+    plan[1] = attention_mfma_decode_supports(nq, nkv) ? 0 : 1;
+  } else {
+    plan[0] = 16;
+    plan[1] = 1;
+  }
+  return 0;
+}
+
+extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
+                                                 int n_decode, int max_decode_ctx) {
+  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind) || !attention_mfma_decode_supports(nq, nkv)) return 0;
+  return (int64_t)attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx);
+}
 
 extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                             const void* v_pool, const int32_t* block_tables, int max_blocks,
                             const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
-                            const int32_t* tiles, int n_tiles, int tile_q, void* out, int nq, int nkv, int hd,
-                            int page_size, int num_pages, int window, float scale, int kernel_kind) {
+                            const int32_t* tiles, int n_tiles, int tile_q, const int32_t* decode_seqs, int n_decode,
+                            int max_decode_ctx, float* workspace, int64_t workspace_floats, void* out, int nq,
+                            int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind) {
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
   SP_REQUIRE(hd > 0 && hd <= 256, "sp_attention: head size %d is outside 1..256", hd);
   SP_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0, "sp_attention: bad cache geometry");
   SP_REQUIRE(q_stride >= nq * hd, "sp_attention: q row stride %d is smaller than %d", q_stride, nq * hd);
-  SP_REQUIRE(tile_q == sp_attention_tile_q(dtype, hd, 0, kernel_kind), "sp_attention: tiles were built for %d queries", tile_q);
-  if (n_tiles == 0) return 0;
+  int plan[2];
+  sp_attention_plan(dtype, hd, page_size, nq, nkv, kernel_kind, plan);
+  SP_REQUIRE(tile_q == plan[0], "sp_attention: tiles were built for %d queries, the kernel takes %d", tile_q, plan[0]);
+  SP_REQUIRE(plan[1] == 0 || n_decode == 0, "sp_attention: this kernel takes every sequence in the tile list");
+  SP_REQUIRE(n_tiles >= 0 && n_decode >= 0 && (n_tiles == 0 || tiles) && (n_decode == 0 || decode_seqs),
+             "sp_attention: missing tile or sequence list");
   hipStream_t s = (hipStream_t)stream;
-  return attention_generic(s, dtype, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len,
-                           ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale);
+  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind)) {
+    if (n_tiles == 0) return 0;
+    return attention_generic(s, dtype, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len,
+                             ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale);
+  }
+  SP_REQUIRE(max_decode_ctx >= 0 && max_decode_ctx <= max_blocks * page_size,
+             "sp_attention: decode context %d exceeds the block tables", max_decode_ctx);
+  const int64_t need = (int64_t)attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx);
+  SP_REQUIRE(need == 0 || (workspace && workspace_floats >= need),
+             "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
+             (long long)need);
+  return attention_mfma(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
+                        n_tiles, decode_seqs, n_decode, max_decode_ctx, workspace, out, nq, nkv, hd, page_size,
+                        num_pages, window, scale);
 }

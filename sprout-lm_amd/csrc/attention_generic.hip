@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       if (j >= k_lo && j < k_end) {
         const int page = bt[j / page_size];
         if (page >= 0 && page < num_pages)
-          v = to_float(v_pool[((size_t(page) * nkv + g) * page_size + j % page_size) * hd + d]);
+          v = to_float(v_pool[((size_t(page) * nkv + g) * hd + d) * page_size + j % page_size]);
       }
       KVs[jj * kv_stride + d] = v;
     }

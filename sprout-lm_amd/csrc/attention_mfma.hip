@@ -1,0 +1,364 @@
+// bfloat16 attention over the paged cache on the matrix cores (16x16x32 MFMA, float32 softmax).
+//
+// Both kernels walk the keys 32 at a time and keep everything in registers:
+//   S^T[key, row]  = K[key, :] . Q[row, :]         A = 16 keys of K (16-byte loads per lane), B = Q
+//   O^T[dim, row] += V^T[dim, key] . P^T[key, row]  A = V^T (the value pool is stored [dim][key]), B = P
+// The MFMA result layout of S^T (4 consecutive keys per lane for one row) is exactly the B-operand
+// layout of P^T once the 32 keys of a step are numbered (group of 4, tile) instead of in order, and
+// V^T is loaded with the same numbering, so probabilities never leave registers.
+//
+// Prefill: one wave per (tile of 16 * NQT queries of one sequence, head).
+// Decode (one query per sequence): one block per (256 keys, key/value head, sequence); the rows of
+// the MFMA are the query heads of the group, so keys and values are read once per group.  The four
+// waves take 64 keys each and are merged in LDS; blocks are merged by a second small kernel.
+// Keys are always cut at the same places, so a position's result does not depend on the batch.
+#include "mfma.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kDecodeChunk = 256;   // keys per decode block
+constexpr int kDecodeWaveKeys = 64; // keys per wave of a decode block
+
+struct PagedKV {
+  const uint16_t* k;     // key pool, already offset to the key/value head: + page * page_stride + slot * HD + d
+  const uint16_t* v;     // value pool, offset to the head: + page * page_stride + d * page_size + slot
+  const int32_t* table;  // this sequence's block table
+  int page_size, num_pages;
+  size_t page_stride;    // elements between pages: nkv * page_size * HD
+};
+
+__device__ __forceinline__ int page_of(const PagedKV& kv, int key) {
+  const int page = kv.table[key / kv.page_size];
+  return min(max(page, 0), kv.num_pages - 1);   // a bad table entry must not become a wild address
+}
+
+// One step of 32 keys starting at key0 (a multiple of 32) for NQT tiles of 16 rows.
+// qpos[qt]: position of this lane's row (column l % 16 of tile qt), or -1 for a row that does not exist.
+// Loads are clamped to keys in [k_lo, k_hi]; what lies outside is masked by position anyway.
+template <int DT, int NQT>
+__device__ __forceinline__ void attend_step(const bf16x8 (&qop)[NQT][(DT + 1) / 2], floatx4 (&o)[NQT][DT],
+                                            float (&m)[NQT], float (&lsum)[NQT], const PagedKV& kv, int key0,
+                                            int k_lo, int k_hi, const int (&qpos)[NQT], int window, float scale2) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  const int lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+
+  floatx4 s[NQT][2];
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    const int key = min(max(key0 + 16 * kt + lr, k_lo), k_hi);
+    const uint16_t* krow = kv.k + size_t(page_of(kv, key)) * kv.page_stride + size_t(key % kv.page_size) * HD;
+    bf16x8 ka[HC];
+#pragma unroll
+    for (int c = 0; c < HC; ++c) {
+      const int d0 = 32 * c + 8 * lj;
+      ka[c] = d0 < HD ? as_bf16x8(ldg128(krow + d0)) : as_bf16x8(make_uint4(0, 0, 0, 0));
+    }
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      s[qt][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < HC; ++c) s[qt][kt] = mfma16(ka[c], qop[qt][c], s[qt][kt]);
+    }
+  }
+
+  // V^T operands: row = dim 16 * dt + lr; k slots (lj, 0..3) = keys key0 + 4 lj + 0..3, (lj, 4..7) = the same + 16
+  uint2 va[DT][2];
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    int kb = key0 + 16 * kt + 4 * lj;
+    kb = min(max(kb, (k_lo >> 2) << 2), (k_hi >> 2) << 2);
+    const uint16_t* vbase = kv.v + size_t(page_of(kv, kb)) * kv.page_stride + kb % kv.page_size;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      va[dt][kt] = *reinterpret_cast<const uint2*>(vbase + size_t(16 * dt + lr) * kv.page_size);
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float sv[2][4];
+    float mx = m[qt];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = key0 + 16 * kt + 4 * lj + r;
+        const bool visible = key <= qpos[qt] && key >= k_lo && (window <= 0 || qpos[qt] - key < window);
+        sv[kt][r] = visible ? s[qt][kt][r] * scale2 : -INFINITY;
+        mx = fmaxf(mx, sv[kt][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float alpha = 1.f, p[2][4] = {};
+    if (mx != -INFINITY) {
+      alpha = m[qt] == -INFINITY ? 0.f : exp2f(m[qt] - mx);
+      float sum = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          p[kt][r] = sv[kt][r] == -INFINITY ? 0.f : exp2f(sv[kt][r] - mx);
+          sum += p[kt][r];
+        }
+      lsum[qt] = lsum[qt] * alpha + sum;
+      m[qt] = mx;
+    }
+    const uint4 pb = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
+                                pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      floatx4 acc = o[qt][dt];
+      acc *= alpha;
+      const uint4 a = make_uint4(va[dt][0].x, va[dt][0].y, va[dt][1].x, va[dt][1].y);
+      o[qt][dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void load_q_operand(bf16x8 (&qop)[(DT + 1) / 2], const uint16_t* qrow) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  const int lj = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int c = 0; c < HC; ++c) {
+    const int d0 = 32 * c + 8 * lj;
+    qop[c] = (qrow && d0 < HD) ? as_bf16x8(ldg128(qrow + d0)) : as_bf16x8(make_uint4(0, 0, 0, 0));
+  }
+}
+
+// ------------------------------------------------------------------------------------------ prefill
+template <int DT, int NQT>
+__global__ __launch_bounds__(64) void attention_prefill_kernel(
+    const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
+    const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_size, int num_pages,
+    int window, float scale2) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
+  const int h = blockIdx.y, g = h / (nq / nkv);
+  const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
+  const int nvalid = min(16 * NQT, qlen - q_off);
+  if (nvalid <= 0) return;
+  const int pos0 = ctx - qlen + q_off;
+  const int lane = threadIdx.x, lr = lane & 15, lj = lane >> 4;
+
+  PagedKV kv;
+  kv.page_size = page_size;
+  kv.num_pages = num_pages;
+  kv.page_stride = size_t(nkv) * page_size * HD;
+  kv.k = k_pool + size_t(g) * page_size * HD;
+  kv.v = v_pool + size_t(g) * page_size * HD;
+  kv.table = block_tables + size_t(seq) * max_blocks;
+
+  bf16x8 qop[NQT][HC];
+  int qpos[NQT];
+  floatx4 o[NQT][DT];
+  float m[NQT], lsum[NQT];
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int row = 16 * qt + lr;
+    const bool valid = row < nvalid;
+    qpos[qt] = valid ? pos0 + row : -1;
+    load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
+    m[qt] = -INFINITY;
+    lsum[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int k_hi = pos0 + nvalid - 1;
+  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  for (int key0 = (k_lo >> 5) << 5; key0 <= k_hi; key0 += 32)
+    attend_step<DT, NQT>(qop, o, m, lsum, kv, key0, k_lo, k_hi, qpos, window, scale2);
+
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float l = lsum[qt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int row = 16 * qt + lr;
+    if (row >= nvalid) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {   // lane holds dims 16 dt + 4 lj + 0..3 of its row
+      const floatx4 v = o[qt][dt] * inv;
+      *reinterpret_cast<uint2*>(dst + 16 * dt + 4 * lj) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------ decode
+// Partial results of a block, for the merge kernel: part_o [seq][head][split][HD] (not yet divided),
+// part_ml [seq][head][split][2] = (running maximum in log2 units, sum).
+template <int DT>
+__global__ __launch_bounds__(256) void attention_decode_kernel(
+    const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
+    const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ decode_seqs,
+    uint16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int nq,
+    int nkv, int page_size, int num_pages, int window, float scale2) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  __shared__ float s_o[4][16][HD + 1];
+  __shared__ float s_m[4][16], s_l[4][16];
+  const int split = blockIdx.x, g = blockIdx.y, di = blockIdx.z;
+  const int seq = decode_seqs[di];
+  const int ctx = ctx_len[seq], pos = ctx - 1;
+  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int chunk0 = split * kDecodeChunk;
+  if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) return;   // no visible key in this chunk
+  const int G = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+
+  PagedKV kv;
+  kv.page_size = page_size;
+  kv.num_pages = num_pages;
+  kv.page_stride = size_t(nkv) * page_size * HD;
+  kv.k = k_pool + size_t(g) * page_size * HD;
+  kv.v = v_pool + size_t(g) * page_size * HD;
+  kv.table = block_tables + size_t(seq) * max_blocks;
+
+  bf16x8 qop[1][HC];
+  int qpos[1] = {lr < G ? pos : -1};
+  load_q_operand<DT>(qop[0], lr < G ? q + size_t(q_start[seq]) * q_stride + (g * G + lr) * HD : nullptr);
+  floatx4 o[1][DT];
+  float m[1] = {-INFINITY}, lsum[1] = {0.f};
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[0][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int w0 = chunk0 + wave * kDecodeWaveKeys;
+#pragma unroll
+  for (int i = 0; i < kDecodeWaveKeys / 32; ++i) {
+    const int key0 = w0 + 32 * i;
+    if (key0 <= pos && key0 + 32 > k_lo) attend_step<DT, 1>(qop, o, m, lsum, kv, key0, k_lo, pos, qpos, window, scale2);
+  }
+  float l = lsum[0];
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (lj == 0) { s_m[wave][lr] = m[0]; s_l[wave][lr] = l; }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s_o[wave][lr][16 * dt + 4 * lj + r] = o[0][dt][r];
+  __syncthreads();
+
+  for (int i = threadIdx.x; i < G * HD; i += 256) {
+    const int qh = i / HD, d = i % HD;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, s_m[w][qh]);
+    float num = 0.f, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = s_m[w][qh] == -INFINITY ? 0.f : exp2f(s_m[w][qh] - mx);
+      num += f * s_o[w][qh][d];
+      den += f * s_l[w][qh];
+    }
+    const int head = g * G + qh;
+    if (n_splits == 1) {
+      out[size_t(q_start[seq]) * (size_t(nq) * HD) + head * HD + d] = f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+    } else {
+      const size_t slot = (size_t(di) * nq + head) * n_splits + split;
+      part_o[slot * HD + d] = num;
+      if (d == 0) { part_ml[2 * slot] = mx; part_ml[2 * slot + 1] = den; }
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                             const float* __restrict__ part_ml,
+                                                             const int32_t* __restrict__ q_start,
+                                                             const int32_t* __restrict__ ctx_len,
+                                                             const int32_t* __restrict__ decode_seqs,
+                                                             uint16_t* __restrict__ out, int n_splits, int nq,
+                                                             int window) {
+  constexpr int HD = 16 * DT;
+  const int di = blockIdx.x, head = blockIdx.y;
+  const int seq = decode_seqs[di];
+  const int pos = ctx_len[seq] - 1;
+  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int first = k_lo / kDecodeChunk, last = pos / kDecodeChunk;   // the splits that wrote something
+  const size_t base = (size_t(di) * nq + head) * n_splits;
+  float mx = -INFINITY;
+  for (int s = first; s <= last; ++s) mx = fmaxf(mx, part_ml[2 * (base + s)]);
+  for (int d = threadIdx.x; d < HD; d += 64) {
+    float num = 0.f, den = 0.f;
+    for (int s = first; s <= last; ++s) {
+      const float ms = part_ml[2 * (base + s)];
+      const float f = ms == -INFINITY ? 0.f : exp2f(ms - mx);
+      num += f * part_o[(base + s) * HD + d];
+      den += f * part_ml[2 * (base + s) + 1];
+    }
+    out[size_t(q_start[seq]) * (size_t(nq) * HD) + head * HD + d] = f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+  }
+}
+
+// ------------------------------------------------------------------------------------------ host side
+bool attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
+  const int dt = hd / 16;
+  const bool hd_ok = hd % 16 == 0 && (dt <= 6 || dt == 8);
+  return hd_ok && page_size % 4 == 0;
+}
+bool attention_mfma_decode_supports(int nq, int nkv) { return nq / nkv <= 16; }
+int attention_mfma_tile_q(int hd) { return hd <= 64 ? 64 : 32; }
+
+size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx) {
+  const size_t splits = (max_ctx + kDecodeChunk - 1) / kDecodeChunk;
+  return splits <= 1 ? 0 : size_t(n_decode) * nq * splits * (hd + 2);
+}
+
+template <int DT>
+static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                       const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                       const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs,
+                       int n_decode, int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int page_size,
+                       int num_pages, int window, float scale) {
+  constexpr int HD = 16 * DT;
+  constexpr int NQT = HD <= 64 ? 4 : 2;
+  const float scale2 = scale * kLog2e;
+  const uint16_t *qp = (const uint16_t*)q, *kp = (const uint16_t*)k_pool, *vp = (const uint16_t*)v_pool;
+  if (n_tiles > 0) {
+    attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
+        qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
+        page_size, num_pages, window, scale2);
+    if (check_launch("sp_attention (prefill)")) return 1;
+  }
+  if (n_decode > 0) {
+    const int n_splits = max(1, (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk);
+    float* part_o = workspace;
+    float* part_ml = workspace ? workspace + size_t(n_decode) * nq * n_splits * HD : nullptr;
+    attention_decode_kernel<DT><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+        qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
+        n_splits, nq, nkv, page_size, num_pages, window, scale2);
+    if (check_launch("sp_attention (decode)")) return 1;
+    if (n_splits > 1) {
+      attention_merge_kernel<DT><<<dim3(n_decode, nq), 64, 0, s>>>(part_o, part_ml, q_start, ctx_len, decode_seqs,
+                                                                    (uint16_t*)out, n_splits, nq, window);
+      if (check_launch("sp_attention (merge)")) return 1;
+    }
+  }
+  return 0;
+}
+
+int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                   const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                   const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
+                   int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int hd, int page_size,
+                   int num_pages, int window, float scale) {
+#define SP_MFMA(DT)                                                                                              \
+  case DT:                                                                                                       \
+    return launch_mfma<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len,    \
+                           tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, workspace, out, nq, nkv,       \
+                           page_size, num_pages, window, scale)
+  switch (hd / 16) {
+    SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
+  }
+#undef SP_MFMA
+  set_error("sp_attention: no matrix-core kernel for head size %d", hd);
+  return 1;
+}
+
+}  // namespace sprout

@@ -59,7 +59,8 @@ __global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, in
 
 // ---------------------------------------------------------------- rotation + cache write
 // One block per token.  Pair (d, d + rotary_dim/2) of each q and k head turns by
-// positions[t] * inv_freq[d]; k (rotated) and v go to the pools.
+// positions[t] * inv_freq[d]; k (rotated) and v go to the pools.  Keys lie [page][group][slot][dim]; values lie
+// [page][group][dim][slot], so that the keys of one dimension are contiguous for the P.V matrix product.
 template <typename T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
                                   const float* __restrict__ inv_freq, int rotary_dim,
@@ -101,7 +102,7 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict
   }
   for (int i = threadIdx.x; i < nkv * hd; i += blockDim.x) {
     const int g = i / hd, d = i % hd;
-    v_pool[((size_t(page) * nkv + g) * page_size + off) * hd + d] = row[size_t(nq + nkv + g) * hd + d];
+    v_pool[((size_t(page) * nkv + g) * hd + d) * page_size + off] = row[size_t(nq + nkv + g) * hd + d];
   }
 }
 

@@ -1,10 +1,172 @@
-// bfloat16 matrix products on the matrix cores (placeholder until the MFMA kernels are in).
-#include "common.h"
+// bfloat16 matrix products on the matrix cores: out[T, N] = x[T, K] . w[N, K]^T, float32 sums.
+//
+// "Skinny" kernel (T <= 64, decoding): the step is bound by reading w once, so every wave streams
+// its rows of w straight from memory into registers (16-byte loads, a 128-byte line per row and
+// instruction), the few activations wait in LDS, and the product runs on 16x16x32 MFMA with the
+// weights as the A operand: D[n, t].  Small matrices are cut along K over several blocks, whose
+// partial sums are added into the float32 output with hardware atomics (accumulate mode only).
+#include "mfma.h"
+#include "sprout_hip.h"
 
 namespace sprout {
-int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode,
-              int out_dtype, void* out, int T, int N, int K, bool* handled) {
+
+enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2 };
+
+template <int TN> struct SkinnyChunk { static constexpr int KC = TN >= 3 ? 448 : 512; };
+
+// grid: (blocks of 4 * RW row tiles, K splits).  block: 256 threads = 4 waves, each RW tiles of 16 rows.
+template <int TN, int RW, int MODE, typename TB>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const uint16_t* __restrict__ x,
+                                                          const uint16_t* __restrict__ w,
+                                                          const TB* __restrict__ bias, void* __restrict__ out,
+                                                          int T, int N, int K, int k_per_split) {
+  constexpr int KC = SkinnyChunk<TN>::KC;
+  constexpr int LD = KC / 8 + 1;                      // row pitch of the staged activations, in uint4
+  extern __shared__ uint4 xs[];                       // [TN * 16][LD]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int lr = lane & 15, lj = lane >> 4;
+  const int tile0 = (blockIdx.x * 4 + wave) * RW;
+  const int k_begin = blockIdx.y * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+
+  const uint16_t* wrow[RW];
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw) wrow[rw] = w + size_t(min(N - 1, (tile0 + rw) * 16 + lr)) * K;
+
+  floatx4 acc[RW][TN];
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) acc[rw][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int kc = k_begin; kc < k_end; kc += KC) {
+    __syncthreads();
+    for (int i = threadIdx.x; i < TN * 16 * (KC / 8); i += 256) {
+      const int t = i / (KC / 8), c = i % (KC / 8), k = kc + c * 8;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (t < T && k < k_end) v = ldg128(x + size_t(t) * K + k);   // K and the split are multiples of 8
+      xs[t * LD + c] = v;
+    }
+    __syncthreads();
+    const int klen = min(KC, k_end - kc);
+    for (int kk = 0; kk < klen; kk += 64) {
+      const int k = kc + kk + 16 * lj;                // this lane's 16 elements of the 64-wide step
+      const bool in0 = k < k_end, in1 = k + 8 < k_end;
+      uint4 a0[RW], a1[RW];
+#pragma unroll
+      for (int rw = 0; rw < RW; ++rw) {
+        a0[rw] = in0 ? ldg128(wrow[rw] + k) : make_uint4(0, 0, 0, 0);
+        a1[rw] = in1 ? ldg128(wrow[rw] + k + 8) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const uint4 b0 = xs[(tn * 16 + lr) * LD + (kk >> 3) + 2 * lj];
+        const uint4 b1 = xs[(tn * 16 + lr) * LD + (kk >> 3) + 2 * lj + 1];
+#pragma unroll
+        for (int rw = 0; rw < RW; ++rw) {
+          acc[rw][tn] = mfma16(as_bf16x8(a0[rw]), as_bf16x8(b0), acc[rw][tn]);
+          acc[rw][tn] = mfma16(as_bf16x8(a1[rw]), as_bf16x8(b1), acc[rw][tn]);
+        }
+      }
+    }
+  }
+
+  // lane holds out[t = tn * 16 + lr][n = tile * 16 + 4 * lj + r], r = 0..3
+#pragma unroll
+  for (int rw = 0; rw < RW; ++rw) {
+    const int n0 = (tile0 + rw) * 16 + 4 * lj;
+    if (n0 >= N) continue;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int t = tn * 16 + lr;
+      if (t >= T) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = acc[rw][tn][r];
+        if (bias && blockIdx.y == 0 && n0 + r < N) v[r] += to_float(bias[n0 + r]);
+      }
+      const size_t o = size_t(t) * N + n0;
+      if (MODE == kStore) {
+        uint16_t* dst = reinterpret_cast<uint16_t*>(out) + o;
+        if (n0 + 4 <= N && (N & 3) == 0) {
+          *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        } else {
+          for (int r = 0; r < 4 && n0 + r < N; ++r) dst[r] = f32_to_bf16_bits(v[r]);
+        }
+      } else if (MODE == kStoreF32) {
+        float* dst = reinterpret_cast<float*>(out) + o;
+        if (n0 + 4 <= N && (N & 3) == 0) {
+          *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+          for (int r = 0; r < 4 && n0 + r < N; ++r) dst[r] = v[r];
+        }
+      } else {
+        float* dst = reinterpret_cast<float*>(out) + o;
+        if (gridDim.y == 1) {
+          for (int r = 0; r < 4 && n0 + r < N; ++r) dst[r] += v[r];
+        } else {
+          for (int r = 0; r < 4 && n0 + r < N; ++r) unsafeAtomicAdd(dst + r, v[r]);
+        }
+      }
+    }
+  }
+}
+
+template <int TN, int RW, int MODE, typename TB>
+static int launch_skinny(hipStream_t s, const void* x, const void* w, const void* bias, void* out, int T, int N, int K,
+                         int splits, int k_per_split) {
+  constexpr int KC = SkinnyChunk<TN>::KC;
+  const int tiles = (N + 15) / 16;
+  dim3 grid((tiles + 4 * RW - 1) / (4 * RW), splits);
+  const size_t lds = size_t(TN) * 16 * (KC / 8 + 1) * sizeof(uint4);
+  gemm_skinny_kernel<TN, RW, MODE, TB><<<grid, 256, lds, s>>>((const uint16_t*)x, (const uint16_t*)w, (const TB*)bias,
+                                                               out, T, N, K, k_per_split);
+  return check_launch("sp_gemm (skinny)");
+}
+
+template <int TN, int RW, typename TB>
+static int skinny_mode(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
+                       int K, int splits, int k_per_split) {
+  if (mode == kStore) return launch_skinny<TN, RW, kStore, TB>(s, x, w, bias, out, T, N, K, splits, k_per_split);
+  if (mode == kAccumulate) return launch_skinny<TN, RW, kAccumulate, TB>(s, x, w, bias, out, T, N, K, splits, k_per_split);
+  return launch_skinny<TN, RW, kStoreF32, TB>(s, x, w, bias, out, T, N, K, splits, k_per_split);
+}
+
+template <typename TB>
+static int skinny_shape(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
+                        int K) {
+  const int tiles = (N + 15) / 16;
+  const int rw = tiles >= 4096 ? 2 : 1;
+  int splits = 1, k_per_split = K;
+  if (mode == kAccumulate) {
+    const int want = (1536 + tiles - 1) / tiles;          // enough waves to keep every SIMD loading
+    splits = max(1, min(want, K / 256));
+    k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+    splits = (K + k_per_split - 1) / k_per_split;
+  }
+#define SP_SKINNY(TN)                                                                                              \
+  (rw == 2 ? skinny_mode<TN, 2, TB>(s, x, w, bias, mode, out, T, N, K, splits, k_per_split)                        \
+           : skinny_mode<TN, 1, TB>(s, x, w, bias, mode, out, T, N, K, splits, k_per_split))
+  if (T <= 16) return SP_SKINNY(1);
+  if (T <= 32) return SP_SKINNY(2);
+  return SP_SKINNY(4);
+#undef SP_SKINNY
+}
+
+// mode 0 stores bfloat16 here; a float32 store of mode 0 is passed in as mode 2 by the caller.
+int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, int out_dtype,
+              void* out, int T, int N, int K, bool* handled) {
   *handled = false;
+  if (K % 8 != 0) return 0;                               // rows of w must start on 16-byte boundaries
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) & 15) return 0;
+  if (mode == kStore && out_dtype == kF32) mode = kStoreF32;
+  if (T <= 64) {
+    *handled = true;
+    if (bias && bias_dtype == kBF16) return skinny_shape<bf16_t>(s, a, w, bias, mode, out, T, N, K);
+    return skinny_shape<float>(s, a, w, bias, mode, out, T, N, K);
+  }
   return 0;
 }
+
 }  // namespace sprout

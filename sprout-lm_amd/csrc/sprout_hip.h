@@ -25,7 +25,7 @@ int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w
 // Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
 // inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
 // (= page * page_size + offset; negative: not written).  nkv == 0: only q is rotated.
-// Pools are [pages][nkv][page_size][hd] of `dtype`.
+// The key pool is [pages][nkv][page_size][hd], the value pool [pages][nkv][hd][page_size], of `dtype`.
 int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, const float* inv_freq,
                   int rotary_dim, const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int nq,
                   int nkv, int hd, int page_size, int num_pages);
@@ -33,14 +33,21 @@ int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, 
 // Causal attention of a mixed batch over the paged pools.
 // q: [T, q_stride] (head h at column h * hd), out: [T, nq * hd].
 // Sequence s owns tokens q_start[s] .. q_start[s] + q_len[s]; their positions end at ctx_len[s] - 1.
-// tiles: [n_tiles][2] = (sequence, first query of the tile within the sequence's tokens).
+// sp_attention_plan tells how the caller must list the work: tiles [n_tiles][2] = (sequence, first
+// query of the tile within the sequence's tokens) of plan[0] queries each, over every sequence
+// (plan[1] == 1) or over the sequences with more than one query only, the others being listed in
+// decode_seqs (plan[1] == 0).  max_decode_ctx: largest ctx_len among decode_seqs.
 // window <= 0: all keys; else keys with position - key < window.
+// workspace: sp_attention_workspace_floats(...) floats of scratch for partial results.
+int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind, int* plan);
+int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
+                                      int n_decode, int max_decode_ctx);
 int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                  const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
-                 const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
-                 int tile_q, void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
-                 float scale, int kernel_kind);
-int sp_attention_tile_q(int dtype, int hd, int max_q_len, int kernel_kind);
+                 const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, int tile_q,
+                 const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
+                 int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size, int num_pages,
+                 int window, float scale, int kernel_kind);
 
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I);

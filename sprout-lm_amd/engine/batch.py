@@ -11,7 +11,7 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
-TILE_SIZES = (16, 64, 128)   # query-tile sizes an attention kernel may ask for
+from .. import ops
 
 
 @dataclass
@@ -29,7 +29,7 @@ class CacheSlotView:
 
     writes: bool
     k: torch.Tensor | None = None            # [pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None = None
+    v: torch.Tensor | None = None            # [pages, kv_heads, head_dim, page_size]
     block_tables: torch.Tensor | None = None  # int32 [sequences, max_blocks]
     slot_mapping: torch.Tensor | None = None  # int32 [tokens]: page * page_size + offset
     state: torch.Tensor | None = None         # [max_sequences, *shape] for a fixed-size state slot
@@ -64,28 +64,13 @@ class StepContext:
         self.max_q_len = 0
         self.token_ids = self.positions = self.q_start = self.q_len = self.ctx_len = None
         self.logit_rows = self.state_slots = self.seq_of_token = None
-        self._tiles: dict[int, tuple[torch.Tensor, int]] = {}
+        self.attention = None   # ops.AttentionBatch of this step
         self.group_tables: list[torch.Tensor] = []
         self.group_slots: list[torch.Tensor] = []
         self.host = {}   # the same arrays on the host (numpy), for parts that plan on the CPU
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)
-
-    def attention_tiles(self, dtype, head_dim: int):
-        from .. import ops
-        tile_q = ops.attention_tile_q(dtype, head_dim, self.max_q_len, self.attention_kind)
-        tiles, n = self._tiles[tile_q]
-        return tiles, n, tile_q
-
-
-def _tiles_for(q_lens, tile_q: int) -> np.ndarray:
-    out = []
-    for s, n in enumerate(q_lens):
-        for off in range(0, n, tile_q):
-            out.append((s, off))
-    return np.asarray(out, dtype=np.int32).reshape(-1, 2)
-
 
 class DescriptorStager:
     """Pinned host buffers, used in turn, through which a step's integer arrays reach the device."""
@@ -147,8 +132,9 @@ def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, wor
     state_slots = np.asarray([e.seq.state_slot for e in entries], dtype=np.int32)
 
     arrays = [token_ids, positions, starts, q_len, ctx_len, logit_rows, state_slots, seq_of_token]
-    tile_arrays = [_tiles_for(q_lens, t) for t in TILE_SIZES]
-    arrays += tile_arrays
+    lists = ops.attention_lists(q_lens)
+    list_names = sorted(lists)
+    arrays += [lists[name] for name in list_names]
     for gi, group in enumerate(cache.groups):
         width = max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
         tables = np.full((len(entries), width), -1, dtype=np.int32)
@@ -165,9 +151,11 @@ def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, wor
     dev = stager.upload(arrays)
     (ctx.token_ids, ctx.positions, ctx.q_start, ctx.q_len, ctx.ctx_len, ctx.logit_rows, ctx.state_slots,
      ctx.seq_of_token) = dev[:8]
-    for t, arr, d in zip(TILE_SIZES, tile_arrays, dev[8:8 + len(TILE_SIZES)]):
-        ctx._tiles[t] = (d, arr.shape[0])
-    rest = dev[8 + len(TILE_SIZES):]
+    on_device = {name: (d, len(lists[name])) for name, d in zip(list_names, dev[8:8 + len(list_names)])}
+    decode_ctx = [int(c) for c, q in zip(ctx_len, q_lens) if q == 1]
+    ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, len(entries), on_device,
+                                       max(decode_ctx, default=0))
+    rest = dev[8 + len(list_names):]
     ctx.group_tables = rest[0::2]
     ctx.group_slots = rest[1::2]
     ctx.n_tokens, ctx.n_seqs, ctx.n_logits = T, len(entries), len(rows)

@@ -1,8 +1,8 @@
 """Python faces of the HIP kernels.  Each takes torch tensors on the GPU, checks shapes on the host
 and launches on torch's current stream."""
-from .kernels import (attention, attention_tile_q, cast, embed, gemm, rmsnorm, rope_cache, sample,
+from .kernels import (AttentionBatch, attention, attention_lists, attention_plan, cast, embed, gemm, rmsnorm, rope_cache, sample,
                       sample_workspace_floats, silu_mul)
 from .library import KernelError, library
 
-__all__ = ["attention", "attention_tile_q", "cast", "embed", "gemm", "rmsnorm", "rope_cache", "sample",
+__all__ = ["AttentionBatch", "attention", "attention_lists", "attention_plan", "cast", "embed", "gemm", "rmsnorm", "rope_cache", "sample",
            "sample_workspace_floats", "silu_mul", "KernelError", "library"]

@@ -37,6 +37,17 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _check_pools(k_pool, v_pool, nkv: int, hd: int, dtype, what: str) -> tuple[int, int]:
+    """Keys [pages, nkv, page_size, hd] and values [pages, nkv, hd, page_size]; returns (pages, page_size)."""
+    _gpu(k_pool, "key pool"); _gpu(v_pool, "value pool")
+    if k_pool.dim() != 4 or k_pool.shape[1] != nkv or k_pool.shape[3] != hd or k_pool.dtype != dtype:
+        raise KernelError(f"{what}: key pool {tuple(k_pool.shape)} {k_pool.dtype} does not fit nkv={nkv} hd={hd} {dtype}")
+    num_pages, _, page_size, _ = k_pool.shape
+    if tuple(v_pool.shape) != (num_pages, nkv, hd, page_size) or v_pool.dtype != dtype:
+        raise KernelError(f"{what}: value pool {tuple(v_pool.shape)} {v_pool.dtype} must be [{num_pages}, {nkv}, {hd}, {page_size}] {dtype}")
+    return num_pages, page_size
+
+
 def embed(table: torch.Tensor, tokens: torch.Tensor, residual: torch.Tensor) -> None:
     """residual[t] = table[tokens[t]] as float32."""
     _gpu(table, "embedding table"); _gpu(residual, "residual")
@@ -92,7 +103,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: torch.Tensor
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int, nq: int, nkv: int,
                hd: int, slot_mapping: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
                v_pool: torch.Tensor | None = None) -> None:
-    """Rotate q and k heads of qkv in place and write k, v into the pools ([pages, nkv, page, hd])."""
+    """Rotate q and k heads of qkv in place and write k, v into the pools (keys [pages, nkv, page, hd], values
+    [pages, nkv, hd, page])."""
     _gpu(qkv, "qkv")
     T = qkv.shape[0]
     if qkv.shape[1] != (nq + 2 * nkv) * hd:
@@ -104,47 +116,105 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tenso
     page_size = num_pages = 0
     if nkv:
         _ints(slot_mapping, T, "slot_mapping")
-        for pool in (k_pool, v_pool):
-            _gpu(pool, "cache pool")
-            if pool.dtype != qkv.dtype or pool.dim() != 4 or pool.shape[1] != nkv or pool.shape[3] != hd:
-                raise KernelError(f"rope_cache: pool {tuple(pool.shape)} {pool.dtype} does not fit nkv={nkv} hd={hd} {qkv.dtype}")
-        num_pages, _, page_size, _ = k_pool.shape
-        if tuple(v_pool.shape) != tuple(k_pool.shape):
-            raise KernelError("rope_cache: key and value pools differ in shape")
+        num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, qkv.dtype, "rope_cache")
     check(library().sp_rope_cache(_stream(), _code(qkv, "qkv"), qkv.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(),
                                   rotary_dim, _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), T, nq, nkv, hd, page_size,
                                   num_pages))
 
 
-def attention_tile_q(dtype: torch.dtype, hd: int, max_q_len: int, kind: int = 0) -> int:
-    return library().sp_attention_tile_q(_CODES[dtype], hd, max_q_len, kind)
+TILE_SIZES = (16, 32, 64)   # query-tile sizes an attention kernel may ask for
+
+
+def attention_lists(q_lens) -> dict:
+    """Host-side work lists of a batch for the attention kernels (numpy int32 arrays).
+
+    tiles_all_<n>: (sequence, first query) of every tile of n queries, over all sequences;
+    tiles_multi_<n>: the same over the sequences with more than one query; decode_seqs: the others.
+    """
+    import numpy as np
+    out = {}
+    for n in TILE_SIZES:
+        every = [(s, off) for s, q in enumerate(q_lens) for off in range(0, q, n)]
+        out[f"tiles_all_{n}"] = np.asarray(every, dtype=np.int32).reshape(-1, 2)
+        multi = [(s, off) for s, q in enumerate(q_lens) if q > 1 for off in range(0, q, n)]
+        out[f"tiles_multi_{n}"] = np.asarray(multi, dtype=np.int32).reshape(-1, 2)
+    out["decode_seqs"] = np.asarray([s for s, q in enumerate(q_lens) if q == 1], dtype=np.int32)
+    return out
+
+
+class AttentionBatch:
+    """The device-side description of a step's sequences that `attention` reads."""
+
+    def __init__(self, q_start, q_len, ctx_len, n_seqs: int, lists: dict, max_decode_ctx: int):
+        """`lists`: name -> (device int32 tensor, number of entries), names as in `attention_lists`."""
+        self.q_start, self.q_len, self.ctx_len, self.n_seqs = q_start, q_len, ctx_len, n_seqs
+        self.lists, self.max_decode_ctx = lists, max_decode_ctx
+
+    @classmethod
+    def build(cls, q_lens, ctx_lens, device) -> "AttentionBatch":
+        """From host lists, one upload per array (tests and small tools; the engine packs its own)."""
+        import numpy as np
+        to = lambda a: torch.as_tensor(np.ascontiguousarray(a), dtype=torch.int32).to(device)
+        starts = np.concatenate([[0], np.cumsum(q_lens)[:-1]]) if len(q_lens) else np.zeros(0)
+        lists = {k: (to(v), len(v)) for k, v in attention_lists(q_lens).items()}
+        decode_ctx = [c for c, q in zip(ctx_lens, q_lens) if q == 1]
+        return cls(to(starts), to(q_lens), to(ctx_lens), len(q_lens), lists, max(decode_ctx, default=0))
+
+
+def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: int, kind: int = 0) -> tuple[int, bool]:
+    """(queries per tile, whether the tile list must hold every sequence) of the kernel that will run."""
+    import ctypes
+    plan = (ctypes.c_int * 2)()
+    check(library().sp_attention_plan(_CODES[dtype], hd, page_size, nq, nkv, kind, plan))
+    return plan[0], bool(plan[1])
 
 
 def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
-              q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, tiles: torch.Tensor, n_tiles: int,
-              tile_q: int, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
-              n_seqs: int, kind: int = 0) -> None:
-    """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h)."""
-    for t, what in ((q, "q"), (k_pool, "key pool"), (v_pool, "value pool"), (out, "attention output")):
+              batch: AttentionBatch, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
+              workspace=None, kind: int = 0) -> None:
+    """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h).
+
+    `workspace(n)` must return a float32 device tensor of at least n elements (default: a new one).
+    """
+    for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
     T = out.shape[0]
-    if out.shape[1] != nq * hd or q.shape[0] < T or q.dtype != out.dtype or k_pool.dtype != q.dtype:
-        raise KernelError(f"attention: shapes or dtypes do not fit: q {tuple(q.shape)} {q.dtype}, out {tuple(out.shape)} {out.dtype}, pool {k_pool.dtype}")
+    if out.shape[1] != nq * hd or q.shape[0] < T or q.dtype != out.dtype:
+        raise KernelError(f"attention: shapes or dtypes do not fit: q {tuple(q.shape)} {q.dtype}, out {tuple(out.shape)} {out.dtype}")
     if q_stride > q.shape[1] or q_stride < nq * hd:
         raise KernelError("attention: bad q row stride")
-    if k_pool.dim() != 4 or k_pool.shape[1] != nkv or k_pool.shape[3] != hd or tuple(k_pool.shape) != tuple(v_pool.shape):
-        raise KernelError(f"attention: pool {tuple(k_pool.shape)} does not fit nkv={nkv} hd={hd}")
-    num_pages, _, page_size, _ = k_pool.shape
+    if nkv <= 0 or nq % nkv:
+        raise KernelError(f"attention: {nq} query heads do not divide into {nkv} groups")
+    if not 0 < hd <= 256:
+        raise KernelError(f"attention: head size {hd} is outside 1..256")
+    num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, q.dtype, "attention")
     _gpu(block_tables, "block tables")
+    n_seqs = batch.n_seqs
     if block_tables.dtype != torch.int32 or block_tables.dim() != 2 or block_tables.shape[0] < n_seqs:
         raise KernelError("attention: block tables must be int32 [sequences, max_blocks]")
-    for t, what in ((q_start, "q_start"), (q_len, "q_len"), (ctx_len, "ctx_len")):
+    for t, what in ((batch.q_start, "q_start"), (batch.q_len, "q_len"), (batch.ctx_len, "ctx_len")):
         _ints(t, n_seqs, what)
+    tile_q, every = attention_plan(q.dtype, hd, page_size, nq, nkv, kind)
+    tiles, n_tiles = batch.lists[f"tiles_{'all' if every else 'multi'}_{tile_q}"]
+    decode, n_decode = (None, 0) if every else batch.lists["decode_seqs"]
     _ints(tiles, 2 * n_tiles, "tiles")
+    max_decode_ctx = batch.max_decode_ctx if n_decode else 0
+    if n_decode:
+        _ints(decode, n_decode, "decode_seqs")
+        if max_decode_ctx > block_tables.shape[1] * page_size:
+            raise KernelError("attention: a decode context is longer than its block table")
+    need = library().sp_attention_workspace_floats(_code(q, "q"), hd, page_size, nq, nkv, kind, n_decode, max_decode_ctx)
+    ws = None
+    if need:
+        ws = workspace(need) if workspace is not None else torch.empty(need, dtype=torch.float32, device=q.device)
+        if ws.dtype != torch.float32 or ws.numel() < need:
+            raise KernelError("attention: workspace too small")
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
-                                 block_tables.data_ptr(), block_tables.shape[1], q_start.data_ptr(), q_len.data_ptr(),
-                                 ctx_len.data_ptr(), tiles.data_ptr(), n_tiles, tile_q, out.data_ptr(), nq, nkv, hd,
-                                 page_size, num_pages, int(window) if window else 0, float(scale), kind))
+                                 block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
+                                 batch.q_len.data_ptr(), batch.ctx_len.data_ptr(), _ptr(tiles) if n_tiles else None,
+                                 n_tiles, tile_q, _ptr(decode) if n_decode else None, n_decode, max_decode_ctx, _ptr(ws),
+                                 need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
+                                 float(scale), kind))
 
 
 def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:

@@ -23,13 +23,16 @@ def _declare(lib):
         "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
                           c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
-                         c_int, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
-        "sp_attention_tile_q": [c_int, c_int, c_int, c_int],
+                         c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int, c_int,
+                         c_int, c_float, c_int],
+        "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
         "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int],
         "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
     }
+    lib.sp_attention_workspace_floats.argtypes = [c_int] * 8
+    lib.sp_attention_workspace_floats.restype = c_i64
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

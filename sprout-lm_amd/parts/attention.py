@@ -74,8 +74,8 @@ class Attention(Mixer):
                        self.head_dim, cache.slot_mapping if nkv else None, cache.k if nkv else None,
                        cache.v if nkv else None)
         attn = ctx.buffer("attn", (T, self.heads * self.head_dim), ctx.act_dtype)
-        tiles, n_tiles, tile_q = ctx.attention_tiles(ctx.act_dtype, self.head_dim)
-        ops.attention(qkv, width, cache.k, cache.v, cache.block_tables, ctx.q_start, ctx.q_len, ctx.ctx_len, tiles,
-                      n_tiles, tile_q, attn, self.heads, self.kv_heads, self.head_dim, self.window, self.scale,
-                      ctx.n_seqs, kind=ctx.attention_kind)
+        ops.attention(qkv, width, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads, self.kv_heads,
+                      self.head_dim, self.window, self.scale,
+                      workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
+                      kind=ctx.attention_kind)
         ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)

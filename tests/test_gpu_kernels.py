@@ -133,7 +133,7 @@ def test_rope_and_cache_write(nq, nkv, hd, rotary, page, dtype):
     inv = torch.tensor(theta ** (-2.0 * np.arange(rotary // 2) / rotary), dtype=torch.float32, device=DEV)
     Q = t(qkv, dtype)
     kp = torch.zeros(pages, nkv, page, hd, dtype=dtype, device=DEV)
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros(pages, nkv, hd, page, dtype=dtype, device=DEV)
     ops.rope_cache(Q, torch.tensor(pos, dtype=torch.int32, device=DEV), inv, rotary, nq, nkv, hd,
                    torch.tensor(slots, device=DEV), kp, vp)
     want_qk = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, rotary, theta)
@@ -141,7 +141,7 @@ def test_rope_and_cache_write(nq, nkv, hd, rotary, page, dtype):
     got = Q.float().cpu().numpy()
     assert np.abs(got[:, :(nq + nkv) * hd] - want_qk).max() <= tol * 4
     assert np.array_equal(got[:, (nq + nkv) * hd:], qkv[:, (nq + nkv) * hd:])
-    kp, vp = kp.float().cpu().numpy(), vp.float().cpu().numpy()
+    kp, vp = kp.float().cpu().numpy(), vp.float().cpu().numpy().transpose(0, 1, 3, 2)   # values lie [.., dim, slot]
     written = np.zeros((pages, page), bool)
     for i in range(T):
         if slots[i] < 0:
@@ -206,13 +206,11 @@ def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=Non
         t0 += qlen
     if dtype == torch.bfloat16:
         q, kp = bf16(q), bf16(kp)
-    tile_q = ops.attention_tile_q(dtype, hd, max(ql for _, ql in seqs), kind)
-    tiles = np.asarray([(s, off) for s, (_, ql) in enumerate(seqs) for off in range(0, ql, tile_q)], np.int32)
     out = torch.full((T, nq * hd), float("nan"), dtype=dtype, device=DEV)
     scale = 1 / math.sqrt(hd)
-    ops.attention(t(q, dtype), nq * hd, t(kp, dtype), t(vp, dtype), t(tables, torch.int32), t(starts, torch.int32),
-                  t([ql for _, ql in seqs], torch.int32), t([c for c, _ in seqs], torch.int32), t(tiles, torch.int32),
-                  len(tiles), tile_q, out, nq, nkv, hd, window, scale, len(seqs), kind=kind)
+    batch = ops.AttentionBatch.build([ql for _, ql in seqs], [c for c, _ in seqs], DEV)
+    ops.attention(t(q, dtype), nq * hd, t(kp, dtype), t(vp.transpose(0, 1, 3, 2), dtype), t(tables, torch.int32), batch,
+                  out, nq, nkv, hd, window, scale, kind=kind)
     got = out.float().cpu().numpy()
     want = np.concatenate([plain_attention(q[starts[s]:starts[s] + ql].astype(np.float64), keys[s].astype(np.float64),
                                            values[s].astype(np.float64), nq, nkv, hd, c - ql, window, scale)
@@ -255,14 +253,14 @@ def test_attention_refuses_what_it_cannot_take():
     from sprout_lm_amd import ops
     q = torch.zeros(1, 4 * 16, device=DEV)
     pool = torch.zeros(2, 3, 16, 16, device=DEV)
-    ints = torch.zeros(4, dtype=torch.int32, device=DEV)
+    batch = ops.AttentionBatch.build([1], [1], DEV)
     table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
     with pytest.raises(ops.KernelError, match="groups"):
-        ops.attention(q, 64, pool, pool, table, ints, ints, ints, ints, 1, 16, torch.empty_like(q), 4, 3, 16, None, 0.25, 1, kind=1)
+        ops.attention(q, 64, pool, pool, table, batch, torch.empty_like(q), 4, 3, 16, None, 0.25, kind=1)
     big = torch.zeros(1, 512, device=DEV)
     pool = torch.zeros(2, 1, 16, 512, device=DEV)
     with pytest.raises(ops.KernelError, match="head size"):
-        ops.attention(big, 512, pool, pool, table, ints, ints, ints, ints, 1, 16, torch.empty_like(big), 1, 1, 512, None, 0.1, 1, kind=1)
+        ops.attention(big, 512, pool, pool.transpose(2, 3).contiguous(), table, batch, torch.empty_like(big), 1, 1, 512, None, 0.1, kind=1)
 
 
 def test_sampling_greedy_ties_nonfinite_and_temperature():
