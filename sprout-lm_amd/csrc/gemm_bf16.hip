@@ -154,6 +154,9 @@ static int skinny_shape(hipStream_t s, const void* x, const void* w, const void*
 #undef SP_SKINNY
 }
 
+int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                    int T, int N, int K);
+
 // mode 0 stores bfloat16 here; a float32 store of mode 0 is passed in as mode 2 by the caller.
 int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, int out_dtype,
               void* out, int T, int N, int K, bool* handled) {
@@ -166,7 +169,145 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
     if (bias && bias_dtype == kBF16) return skinny_shape<bf16_t>(s, a, w, bias, mode, out, T, N, K);
     return skinny_shape<float>(s, a, w, bias, mode, out, T, N, K);
   }
-  return 0;
+  *handled = true;
+  return gemm_bf16_tiled(s, a, w, bias_dtype, bias, mode, out, T, N, K);
+}
+
+}  // namespace sprout
+
+// ------------------------------------------------------------------------------------------------
+// Tiled kernel (T > 64, prefill): both operands go through LDS in steps of 64 along K; 4 waves in a
+// 2 x 2 arrangement, each computing WM x WN tiles of 32 x 32 on 32x32x16 MFMA with the activations as
+// the A operand, so that lanes run along n in the result and stores are contiguous.  The next step's
+// global loads are in flight while the current one is multiplied.
+namespace sprout {
+
+constexpr int TBK = 64;            // depth of one staging step
+constexpr int TPITCH = TBK + 8;    // LDS row pitch in elements: 144 bytes, 16-byte aligned rows
+
+template <int WM, int WN, int MODE, typename TB>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ x,
+                                                         const uint16_t* __restrict__ w,
+                                                         const TB* __restrict__ bias, void* __restrict__ out, int T,
+                                                         int N, int K) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int XL = BM * TBK / 8 / 256, WL = BN * TBK / 8 / 256;   // 16-byte loads per thread and operand
+  __shared__ __attribute__((aligned(16))) uint16_t xs[BM * TPITCH];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[BN * TPITCH];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int li = lane & 31, lk = lane >> 5;
+  const int t0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+  floatx16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  uint4 xr[XL], wr[WL];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int idx = threadIdx.x + i * 256, row = idx >> 3, c = idx & 7, k = k0 + c * 8;
+      xr[i] = (t0 + row < T && k < K) ? ldg128(x + size_t(t0 + row) * K + k) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+      const int idx = threadIdx.x + i * 256, row = idx >> 3, c = idx & 7, k = k0 + c * 8;
+      wr[i] = (n0 + row < N && k < K) ? ldg128(w + size_t(n0 + row) * K + k) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+      const int idx = threadIdx.x + i * 256, row = idx >> 3, c = idx & 7;
+      *reinterpret_cast<uint4*>(xs + row * TPITCH + c * 8) = xr[i];
+    }
+#pragma unroll
+    for (int i = 0; i < WL; ++i) {
+      const int idx = threadIdx.x + i * 256, row = idx >> 3, c = idx & 7;
+      *reinterpret_cast<uint4*>(ws + row * TPITCH + c * 8) = wr[i];
+    }
+  };
+
+  load_global(0);
+  store_lds();
+  __syncthreads();
+  for (int k0 = 0; k0 < K; k0 += TBK) {
+    const bool more = k0 + TBK < K;
+    if (more) load_global(k0 + TBK);
+#pragma unroll
+    for (int ks = 0; ks < TBK / 16; ++ks) {
+      bf16x8 a[WM], b[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        a[i] = as_bf16x8(*reinterpret_cast<const uint4*>(xs + ((wm * WM + i) * 32 + li) * TPITCH + ks * 16 + lk * 8));
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        b[j] = as_bf16x8(*reinterpret_cast<const uint4*>(ws + ((wn * WN + j) * 32 + li) * TPITCH + ks * 16 + lk * 8));
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+    if (more) {
+      store_lds();
+      __syncthreads();
+    }
+  }
+
+  // lane holds out[t = tile row 8 * (r / 4) + 4 * lk + r % 4][n = tile column li]
+#pragma unroll
+  for (int j = 0; j < WN; ++j) {
+    const int n = n0 + (wn * WN + j) * 32 + li;
+    if (n >= N) continue;
+    const float bv = bias ? to_float(bias[n]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int t = t0 + (wm * WM + i) * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
+        if (t >= T) continue;
+        const float v = acc[i][j][r] + bv;
+        const size_t o = size_t(t) * N + n;
+        if (MODE == kStore) reinterpret_cast<uint16_t*>(out)[o] = f32_to_bf16_bits(v);
+        else if (MODE == kStoreF32) reinterpret_cast<float*>(out)[o] = v;
+        else reinterpret_cast<float*>(out)[o] += v;
+      }
+    }
+  }
+}
+
+template <int WM, int WN, typename TB>
+static int launch_tiled(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
+                        int K) {
+  dim3 grid((N + 64 * WN - 1) / (64 * WN), (T + 64 * WM - 1) / (64 * WM));
+  const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
+  const TB* bp = (const TB*)bias;
+  if (mode == kStore) gemm_tiled_kernel<WM, WN, kStore, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K);
+  else if (mode == kAccumulate) gemm_tiled_kernel<WM, WN, kAccumulate, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K);
+  else gemm_tiled_kernel<WM, WN, kStoreF32, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K);
+  return check_launch("sp_gemm (tiled)");
+}
+
+template <typename TB>
+static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
+                       int K) {
+  auto blocks = [&](int bm, int bn) { return ((T + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  if (blocks(256, 128) >= 512) return launch_tiled<4, 2, TB>(s, x, w, bias, mode, out, T, N, K);
+  if (blocks(128, 128) >= 384) return launch_tiled<2, 2, TB>(s, x, w, bias, mode, out, T, N, K);
+  if (blocks(128, 64) >= 256) return launch_tiled<2, 1, TB>(s, x, w, bias, mode, out, T, N, K);
+  return launch_tiled<1, 1, TB>(s, x, w, bias, mode, out, T, N, K);
+}
+
+int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                    int T, int N, int K) {
+  if (bias && bias_dtype == kBF16) return tiled_shape<bf16_t>(s, a, w, bias, mode, out, T, N, K);
+  return tiled_shape<float>(s, a, w, bias, mode, out, T, N, K);
 }
 
 }  // namespace sprout

@@ -18,7 +18,8 @@ def bf16(x):
 
 
 @pytest.mark.parametrize("T,N,K", [(1, 1, 1), (1, 37, 33), (3, 130, 31), (5, 64, 1025), (17, 151, 96), (64, 100, 70),
-                                   (77, 300, 129), (200, 96, 224), (130, 257, 511)])
+                                   (77, 300, 129), (200, 96, 224), (130, 257, 511), (129, 257, 200), (300, 331, 240),
+                                   (513, 1152, 896), (2, 896, 4864), (40, 640, 1000), (64, 151, 72), (1000, 130, 136)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
