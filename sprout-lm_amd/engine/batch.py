@@ -41,6 +41,7 @@ class Workspace:
 
     def __init__(self, device):
         self.device = device
+        self.frozen = False      # while a graph is recorded nothing may be allocated
         self._flat: dict[tuple[str, torch.dtype], torch.Tensor] = {}
 
     def get(self, name: str, shape, dtype) -> torch.Tensor:
@@ -50,6 +51,8 @@ class Workspace:
         key = (name, dtype)
         flat = self._flat.get(key)
         if flat is None or flat.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"Workspace buffer {name!r} would grow while a graph is recorded.")
             flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
         return flat[:n].view(shape)

@@ -49,10 +49,7 @@ class Engine:
                 or self.options.max_sequences > cache.max_sequences:
             raise ValueError("Engine options and the model's cache differ in block_size, num_blocks or max_sequences.")
         self.model, self.cache = model, cache
-        if sampler is None:
-            from ..sampling.sampler import Sampler
-            sampler = Sampler(model.device, model.vocab_size)
-        self.sampler = sampler
+        self.sampler = sampler     # None: the model samples on the device (`step_and_sample`)
         self.scheduler = Scheduler(cache, self.options, model.vocab_size, model.max_positions, model.stop_token_ids)
         self._auto_ids = itertools.count()
 
@@ -108,10 +105,13 @@ class Engine:
         if work:
             entries = [StepEntry(w.request.seq, w.tokens, [len(w.tokens) - 1] if w.samples else []) for w in work]
             try:
-                logits = self.model.step(entries)
                 sampling = [w for w in work if w.samples]
-                tokens = self.sampler.sample(logits, [w.request.params for w in sampling],
-                                             [len(w.request.output) for w in sampling])
+                params = [w.request.params for w in sampling]
+                counters = [len(w.request.output) for w in sampling]
+                if self.sampler is None:
+                    tokens = self.model.step_and_sample(entries, params, counters)
+                else:
+                    tokens = self.sampler.sample(self.model.step(entries), params, counters)
             except Exception as error:
                 self.scheduler.fail_all(str(error))
                 raise

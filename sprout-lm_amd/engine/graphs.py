@@ -1,0 +1,172 @@
+"""Decode steps as HIP graphs.
+
+A step in which every request brings exactly one token launches a long chain of small kernels; the
+host cannot issue them as fast as the GPU runs them.  Such steps are recorded once per batch shape
+into a HIP graph (through torch's capture of the current stream, which our kernels launch on) and
+replayed with new values in the same device buffers.  Sampling is part of the graph, so one
+descriptor upload, one graph launch and one small download make a step.
+
+Shapes are bucketed: the number of sequences to a power of two (missing ones are filled with
+one-token dummies that write no cache), the block-table width and the key splits of attention to a
+power-of-two context.  Nothing in a graph depends on the values of a step.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .. import ops
+from .batch import CacheSlotView, StepContext, Workspace
+
+
+def _bucket(n: int, floor: int = 1) -> int:
+    return max(floor, 1 << max(0, (n - 1)).bit_length())
+
+
+class _DecodeGraph:
+    """Static buffers and the recorded graph of one (sequences, context) bucket."""
+
+    def __init__(self, runner, n_seqs: int, ctx_bucket: int):
+        self.runner, self.S = runner, n_seqs
+        cache = runner.cache
+        bs = cache.block_size
+        self.max_blocks = -(-ctx_bucket // bs)
+        self.ctx_bucket = ctx_bucket
+        S, G = n_seqs, len(cache.groups)
+        # layout of the int32 staging buffer
+        names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots",
+                 "seq_of_token", "decode_seqs", "counter", "temperature"]
+        self.offsets, total = {}, 0
+        for name in names:
+            self.offsets[name] = (total, S)
+            total += (S + 3) // 4 * 4
+        self.offsets["seed"] = (total, 2 * S)
+        total += (2 * S + 3) // 4 * 4
+        for g in range(G):
+            self.offsets[f"slots{g}"] = (total, S)
+            total += (S + 3) // 4 * 4
+            self.offsets[f"tables{g}"] = (total, S * self.max_blocks)
+            total += (S * self.max_blocks + 3) // 4 * 4
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        view = lambda name: self.dev[self.offsets[name][0]:self.offsets[name][0] + self.offsets[name][1]]
+        self.h = {name: self.host_np[o:o + n] for name, (o, n) in self.offsets.items()}
+        # constant parts
+        arange = np.arange(S, dtype=np.int32)
+        for name in ("q_start", "logit_rows", "seq_of_token", "decode_seqs"):
+            self.h[name][:] = arange
+        self.h["q_len"][:] = 1
+
+        # buffers of its own: a graph holds their addresses, so they must never be reallocated
+        ctx = StepContext(Workspace(runner.device), runner.dtype, runner.attention_kind)
+        ctx.token_ids, ctx.positions, ctx.q_start = view("token_ids"), view("positions"), view("q_start")
+        ctx.q_len, ctx.ctx_len, ctx.logit_rows = view("q_len"), view("ctx_len"), view("logit_rows")
+        ctx.state_slots, ctx.seq_of_token = view("state_slots"), view("seq_of_token")
+        empty = (self.dev[:0].view(0, 2), 0)
+        every = torch.from_numpy(np.stack([arange, np.zeros_like(arange)], axis=1)).to(runner.device)
+        lists = {f"tiles_multi_{t}": empty for t in ops.kernels.TILE_SIZES}
+        lists.update({f"tiles_all_{t}": (every, S) for t in ops.kernels.TILE_SIZES})
+        lists["decode_seqs"] = (view("decode_seqs"), S)
+        ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, S, lists, ctx_bucket)
+        ctx.group_tables = [view(f"tables{g}").view(S, self.max_blocks) for g in range(G)]
+        ctx.group_slots = [view(f"slots{g}") for g in range(G)]
+        ctx.n_tokens = ctx.n_seqs = ctx.n_logits = S
+        ctx.max_q_len = 1
+        self.ctx = ctx
+        self.temperature = view("temperature").view(torch.float32)
+        self.seed = view("seed").view(torch.int64)
+        self.counter = view("counter")
+        self.sampled = torch.zeros(S, dtype=torch.int32, device=runner.device)
+        self.sample_ws = torch.empty(max(1, ops.sample_workspace_floats(S, runner.vocab_size)), dtype=torch.float32,
+                                     device=runner.device)
+        self.graph = None
+        self.logits = None
+
+    def fill(self, entries, params, counters) -> None:
+        """Write this step's values into the pinned staging buffer."""
+        cache, h, n, S = self.runner.cache, self.h, len(entries), self.S
+        bs = cache.block_size
+        lengths = np.fromiter((e.seq.length for e in entries), dtype=np.int32, count=n)
+        h["token_ids"][:n] = [e.tokens[0] for e in entries]
+        h["token_ids"][n:] = 0
+        h["positions"][:n] = lengths
+        h["positions"][n:] = 0
+        h["ctx_len"][:n] = lengths + 1
+        h["ctx_len"][n:] = 1
+        h["state_slots"][:n] = [e.seq.state_slot for e in entries]
+        h["state_slots"][n:] = 0
+        h["counter"][:n] = counters
+        h["temperature"].view(np.float32)[:n] = [p.temperature for p in params]
+        h["temperature"][n:] = 0
+        h["seed"].view(np.int64)[:n] = [p.seed for p in params]
+        for g in range(len(cache.groups)):
+            tables = h[f"tables{g}"].reshape(S, self.max_blocks)
+            slots = h[f"slots{g}"]
+            slots[n:] = -1
+            tables[n:] = 0
+            for i, e in enumerate(entries):
+                blocks = e.seq.blocks[g]
+                nb = min(len(blocks), self.max_blocks)
+                tables[i, :nb] = blocks[:nb]
+                pos = int(lengths[i])
+                slots[i] = blocks[pos // bs] * bs + pos % bs
+
+    def launch(self) -> None:
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.graph is None:
+            self._record()
+        else:
+            self.graph.replay()
+
+    def _body(self):
+        self.logits = self.runner.forward(self.ctx)
+        ops.sample(self.logits, self.sampled, self.sample_ws, self.temperature, self.seed, self.counter)
+
+    def _record(self) -> None:
+        # once eagerly, so that every workspace buffer exists before anything is recorded
+        self._body()
+        torch.cuda.current_stream().synchronize()
+        self.ctx.workspace.frozen = True
+        graph = torch.cuda.CUDAGraph()
+        try:
+            with torch.cuda.graph(graph):
+                self._body()
+        finally:
+            self.ctx.workspace.frozen = False
+        self.graph = graph
+        # the eager run above already produced this step's results; replaying would only repeat it
+
+
+class DecodeGraphs:
+    def __init__(self, runner, max_graphs: int = 32):
+        self.runner = runner
+        self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self.max_graphs = max_graphs
+        self.replays = 0
+
+    def usable(self, entries) -> bool:
+        runner = self.runner
+        return (runner.parts.graph_safe and not runner.cache.state_groups and len(entries) > 0
+                and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries))
+
+    def run(self, entries, params, counters) -> list[int]:
+        """One decode step of `entries` with sampling; returns the sampled token ids."""
+        runner = self.runner
+        n = len(entries)
+        S = _bucket(n)
+        longest = max(e.seq.length for e in entries) + 1
+        ctx_bucket = min(_bucket(longest, 256), -(-runner.max_positions // 256) * 256)
+        key = (S, ctx_bucket)
+        state = self.graphs.get(key)
+        if state is None:
+            if len(self.graphs) >= self.max_graphs:
+                self.graphs.pop(next(iter(self.graphs)))
+            state = self.graphs[key] = _DecodeGraph(runner, S, ctx_bucket)
+        state.fill(entries, params, counters)
+        state.launch()
+        self.replays += 1
+        tokens = state.sampled[:n].tolist()      # waits for the step
+        for e in entries:
+            runner.cache.commit(e.seq, e.seq.length + 1)
+        return tokens

@@ -43,7 +43,7 @@ class ModelRunner:
     """
 
     def __init__(self, plan: ModelPlan, tensors: dict, dtype: torch.dtype, device, block_size: int, num_blocks: int,
-                 max_sequences: int, prefix_caching: bool = False, stop_token_ids=None):
+                 max_sequences: int, prefix_caching: bool = False, stop_token_ids=None, use_graphs: bool = True):
         self.plan, self.dtype, self.device = plan, dtype, device
         self.parts = plan.instantiate()
         self.parts.bind(tensors, device, dtype)
@@ -54,6 +54,9 @@ class ModelRunner:
         self.stop_token_ids = tuple(stop_token_ids if stop_token_ids is not None else plan.eos_token_ids)
         self.attention_kind = 1 if dtype == torch.float32 else 0
         self.vocab_size, self.hidden_size, self.max_positions = plan.vocab_size, plan.hidden_size, plan.max_positions
+        self.use_graphs = use_graphs
+        self._graphs = None
+        self._sampler = None
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -119,6 +122,26 @@ class ModelRunner:
         for e in entries:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
         return logits
+
+    def step_and_sample(self, entries: list[StepEntry], params, counters) -> list[int]:
+        """One step plus sampling at every wanted place; returns the sampled token ids on the host.
+
+        Steps in which every request brings one token are replayed from a recorded HIP graph.
+        """
+        from ..sampling.sampler import NonFiniteLogits, Sampler
+        if self.use_graphs:
+            if self._graphs is None:
+                from .graphs import DecodeGraphs
+                self._graphs = DecodeGraphs(self)
+            if self._graphs.usable(entries):
+                self.validate(entries)
+                tokens = self._graphs.run(entries, params, counters)
+                if any(t < 0 or t >= self.vocab_size for t in tokens):
+                    raise NonFiniteLogits("Non-finite logits: the model produced NaN or infinity.")
+                return tokens
+        if self._sampler is None:
+            self._sampler = Sampler(self.device, self.vocab_size)
+        return self._sampler.sample(self.step(entries), params, counters)
 
     def forward(self, ctx) -> torch.Tensor:
         T, H = ctx.n_tokens, self.hidden_size

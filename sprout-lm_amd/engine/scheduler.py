@@ -37,6 +37,18 @@ class Request:
     def history(self) -> list:
         return self.prompt + self.output
 
+    def history_length(self) -> int:
+        return len(self.prompt) + len(self.output)
+
+    def history_slice(self, start: int, stop: int) -> list:
+        """history()[start:stop] without building the whole history."""
+        n = len(self.prompt)
+        if stop <= n:
+            return self.prompt[start:stop]
+        if start >= n:
+            return self.output[start - n:stop - n]
+        return self.prompt[start:] + self.output[:stop - n]
+
 
 @dataclass
 class Work:
@@ -136,10 +148,10 @@ class Scheduler:
                 break
             if request.status != "running":
                 continue   # an older request preempted it while this step was planned
-            history = request.history()
+            total = request.history_length()
             phase = self._phase(request)
             start = request.seq.length
-            remaining = len(history) - start - (phase == "recompute")
+            remaining = total - start - (phase == "recompute")
             count = min(budget, 1 if phase == "decode" else self.options.prefill_chunk_size, remaining)
             if count <= 0:
                 continue
@@ -147,8 +159,8 @@ class Scheduler:
             budget += refund
             if not ok:
                 continue
-            tokens = history[start:start + count]
-            planned[request.id] = Work(request, phase, start, tokens, samples=start + count == len(history))
+            tokens = request.history_slice(start, start + count)
+            planned[request.id] = Work(request, phase, start, tokens, samples=start + count == total)
             budget -= count
         return [planned[r.id] for r in batch if r.id in planned]
 

@@ -103,6 +103,9 @@ class ModelParts:
         if sorted(slots) != list(range(len(slots))):
             raise ValueError("Cache slots of the run order must be numbered 0..n-1 without gaps.")
         self.cache_slot_specs = [slots[i] for i in range(len(slots))]
+        every = [part for _, part in self._named] + list(self.blocks)
+        every += [getattr(b.mixer, "position", None) for b in self.blocks if hasattr(b, "mixer")]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in every if part is not None)
 
     def expected_tensors(self) -> dict[str, TensorSpec]:
         out = {}

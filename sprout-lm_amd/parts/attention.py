@@ -24,6 +24,8 @@ class Attention(Mixer):
     (rows of q, then k, then v), concatenated when the tensors are bound.
     """
 
+    graph_safe = True
+
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
                  out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None):
         if heads % kv_heads:

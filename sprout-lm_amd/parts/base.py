@@ -45,6 +45,10 @@ class Part:
     """Base of every part."""
 
     kind = ""
+    # True if `forward` only launches work on the current stream from device-resident inputs (no
+    # host-side decisions from the step's values, no allocation): such a part may be recorded into
+    # a HIP graph and replayed with new values in the same buffers.
+    graph_safe = False
 
     def tensors(self) -> dict[str, TensorSpec]:
         """Local tensor name -> what is expected of it."""

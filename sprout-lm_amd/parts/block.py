@@ -8,6 +8,8 @@ from .base import Block, register_part
 class PreNormBlock(Block):
     """x += mixer(norm(x)); x += feed_forward(norm(x)).  The residual stream x is float32."""
 
+    graph_safe = True
+
     def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 

@@ -8,6 +8,8 @@ from .base import Part, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab: int, hidden: int):
         self.vocab, self.hidden = vocab, hidden
 
@@ -21,6 +23,8 @@ class TokenEmbedding(Part):
 @register_part("head", "linear_head")
 class LinearHead(Part):
     """logits = W . x in float32.  With `tied`, W is the embedding table and the head has no tensor."""
+
+    graph_safe = True
 
     def __init__(self, vocab: int, hidden: int, tied: bool):
         self.vocab, self.hidden, self.tied = vocab, hidden, tied

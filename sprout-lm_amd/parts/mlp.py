@@ -12,6 +12,8 @@ from .base import FeedForward, register_part
 class GatedMLP(FeedForward):
     """down(act(gate(x)) * up(x)), no biases.  gate and up are kept as one matrix [2 * inner, hidden]."""
 
+    graph_safe = True
+
     def __init__(self, hidden: int, inner: int, activation: str = "silu"):
         if activation != "silu":
             raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; only 'silu'.")

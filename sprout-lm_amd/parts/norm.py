@@ -10,6 +10,8 @@ from .base import Norm, register_part
 class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight; sums in float32, the weight is used as it is."""
 
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size, self.eps = size, eps
 

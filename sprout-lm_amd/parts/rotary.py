@@ -14,6 +14,8 @@ class NeoxRotary(PositionEncoding):
     and cosines are float32 in the kernel.
     """
 
+    graph_safe = True
+
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
         self.head_dim, self.theta = head_dim, theta
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
@@ -31,6 +33,8 @@ class NoPosition(PositionEncoding):
     """No position encoding: queries and keys are used as projected."""
 
     rotary_dim = 0
+
+    graph_safe = True
 
     def __init__(self, head_dim: int = 0):
         self.head_dim = head_dim
