@@ -156,6 +156,8 @@ static int skinny_shape(hipStream_t s, const void* x, const void* w, const void*
 
 int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
                     int T, int N, int K);
+int gemm_decode_plain(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                      int T, int N, int K);
 
 // mode 0 stores bfloat16 here; a float32 store of mode 0 is passed in as mode 2 by the caller.
 int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, int out_dtype,
@@ -166,6 +168,8 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
   if (mode == kStore && out_dtype == kF32) mode = kStoreF32;
   if (T <= 64) {
     *handled = true;
+    // few rows: split K between the waves of a block (and between blocks when accumulating)
+    if ((N + 15) / 16 < 2048) return gemm_decode_plain(s, a, w, bias_dtype, bias, mode, out, T, N, K);
     if (bias && bias_dtype == kBF16) return skinny_shape<bf16_t>(s, a, w, bias, mode, out, T, N, K);
     return skinny_shape<float>(s, a, w, bias, mode, out, T, N, K);
   }

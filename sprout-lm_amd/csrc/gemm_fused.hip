@@ -1,0 +1,351 @@
+// Skinny bfloat16 products for decoding (T <= 64) with the work of the neighbouring small kernels
+// folded in.  One block of four waves owns TILES tiles of 16 weight rows; the waves split K between
+// them (64 elements at a time, interleaved), so that even a matrix with few rows keeps many loads in
+// flight, and their partial sums meet in LDS.  What can be folded in:
+//   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from
+//                    the float32 residual and kept in LDS (no separate norm kernel, no round trip)
+//   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
+//             kEpiRope   the two tiles are rotation partners (dims d and d + head/2 of one head): adds
+//                        the bias, rotates q and k heads, writes q and scatters k, v into the paged cache
+//             kEpiSilu   the two tiles are gate rows and the matching up rows: writes silu(gate) * up
+// Accumulating products may also be split along K over several blocks (hardware float atomics).
+#include "mfma.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+enum { kEpiStore = 0, kEpiAccumulate = 1, kEpiStoreF32 = 2, kEpiRope = 3, kEpiSilu = 4 };
+
+struct FusedArgs {
+  const uint16_t* x;         // activations [T, K] bfloat16 (without NORM)
+  const float* residual;     // float32 [T, K] (with NORM)
+  const void* norm_w;        // [K]
+  int norm_w_bf16;
+  float eps;
+  const uint16_t* w;         // [N, K]
+  const void* bias;          // [N] or null
+  int bias_bf16;
+  void* out;                 // [T, N] (store / accumulate); [T, N / 2] for kEpiSilu; q rows [T, nq * hd] for kEpiRope
+  int T, N, K, k_per_split;
+  int partner;               // rows between a tile and its partner tile (kEpiRope: hd / 2, kEpiSilu: N / 2)
+  // kEpiRope
+  const int32_t* positions;
+  const float* inv_freq;
+  const int32_t* slot_mapping;
+  uint16_t* k_pool;
+  uint16_t* v_pool;
+  int nq, nkv, hd, page_size, rotary_dim;
+};
+
+__device__ __forceinline__ float load_param(const void* p, int is_bf16, int i) {
+  return is_bf16 ? __uint_as_float(uint32_t(reinterpret_cast<const uint16_t*>(p)[i]) << 16)
+                 : reinterpret_cast<const float*>(p)[i];
+}
+
+// First row of tile `which` (0 or 1) of block `b`.
+template <int EPI>
+__device__ __forceinline__ int tile_row0(const FusedArgs& a, int b, int which) {
+  if (EPI == kEpiRope) {
+    const int per_head = a.hd / 32;                       // pairs of tiles per head
+    const int head = b / per_head, j = b % per_head;
+    return head * a.hd + 16 * j + which * a.partner;
+  }
+  if (EPI == kEpiSilu) return 16 * b + which * a.partner;
+  return 16 * (2 * b + which);
+}
+
+template <int TN, int EPI, bool NORM>
+__global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
+  extern __shared__ uint4 lds[];
+  // reduction buffer [4 waves][2 tiles][TN][64 lanes] float4, then (NORM) activations [TN * 16][K / 8 + 1] uint4
+  float4* red = reinterpret_cast<float4*>(lds);
+  uint4* xs = lds + 4 * 2 * TN * 64;
+  const int LD = a.K / 8 + 1;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int k_begin = blockIdx.y * a.k_per_split;
+  const int k_end = min(a.K, k_begin + a.k_per_split);
+
+  int row0[2];
+  row0[0] = tile_row0<EPI>(a, blockIdx.x, 0);
+  row0[1] = tile_row0<EPI>(a, blockIdx.x, 1);
+  const uint16_t* wrow[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
+
+  if (NORM) {
+    // 16 threads per token: sum of squares, then the normalised row as bfloat16 into LDS
+    for (int t0 = 0; t0 < TN * 16; t0 += 16) {
+      const int t = t0 + (threadIdx.x >> 4), part = threadIdx.x & 15;
+      float sum = 0.f;
+      if (t < a.T)
+        for (int k = part * 4; k < a.K; k += 64) {
+          const float4 v = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k);
+          sum = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sum))));
+        }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+      const float scale = 1.0f / sqrtf(sum / float(a.K) + a.eps);
+      for (int k = part * 8; k < a.K; k += 128) {
+        uint4 packed = make_uint4(0, 0, 0, 0);
+        if (t < a.T) {
+          const float4 v0 = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k);
+          const float4 v1 = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k + 4);
+          const float n[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
+                              v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
+          float y[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) y[i] = n[i] * load_param(a.norm_w, a.norm_w_bf16, k + i);
+          packed = make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]),
+                              pack_bf16x2(y[6], y[7]));
+        }
+        xs[t * LD + (k >> 3)] = packed;
+      }
+    }
+    __syncthreads();
+  }
+
+  floatx4 acc[2][TN];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // this wave's steps of 64 along K: wave, wave + 4, ...; four steps are loaded before they are multiplied
+  const int steps = (k_end - k_begin + 63) / 64;
+  for (int s0 = wave; s0 < steps; s0 += 16) {
+    uint4 wa[4][2][2], xb[4][TN][2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
+      const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        wa[u][i][0] = in0 ? ldg128(wrow[i] + k) : make_uint4(0, 0, 0, 0);
+        wa[u][i][1] = in1 ? ldg128(wrow[i] + k + 8) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) {
+        const int t = tn * 16 + lr;
+        if (NORM) {
+          xb[u][tn][0] = in0 ? xs[t * LD + (k >> 3)] : make_uint4(0, 0, 0, 0);
+          xb[u][tn][1] = in1 ? xs[t * LD + (k >> 3) + 1] : make_uint4(0, 0, 0, 0);
+        } else {
+          const bool row = t < a.T;
+          xb[u][tn][0] = (row && in0) ? ldg128(a.x + size_t(t) * a.K + k) : make_uint4(0, 0, 0, 0);
+          xb[u][tn][1] = (row && in1) ? ldg128(a.x + size_t(t) * a.K + k + 8) : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          acc[i][tn] = mfma16(as_bf16x8(wa[u][i][0]), as_bf16x8(xb[u][tn][0]), acc[i][tn]);
+          acc[i][tn] = mfma16(as_bf16x8(wa[u][i][1]), as_bf16x8(xb[u][tn][1]), acc[i][tn]);
+        }
+  }
+
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+      red[((wave * 2 + i) * TN + tn) * 64 + lane] = make_float4(acc[i][tn][0], acc[i][tn][1], acc[i][tn][2], acc[i][tn][3]);
+  __syncthreads();
+
+  // thread -> (token t of the tile, row i of the tile); the MFMA lane that holds it is (i / 4) * 16 + t, element i % 4
+  const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
+  const int src_lane = (ei >> 2) * 16 + et, src_r = ei & 3;
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn) {
+    const int t = tn * 16 + et;
+    float v[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * 2 + i) * TN + tn) * 64 + src_lane])[src_r];
+      const int n = row0[i] + ei;
+      if (a.bias && blockIdx.y == 0 && n < a.N) sum += load_param(a.bias, a.bias_bf16, n);
+      v[i] = sum;
+    }
+    if (t >= a.T) continue;
+    if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int n = row0[i] + ei;
+        if (n >= a.N) continue;
+        const size_t o = size_t(t) * a.N + n;
+        if (EPI == kEpiStore) reinterpret_cast<uint16_t*>(a.out)[o] = f32_to_bf16_bits(v[i]);
+        else if (EPI == kEpiStoreF32) reinterpret_cast<float*>(a.out)[o] = v[i];
+        else if (gridDim.y == 1) reinterpret_cast<float*>(a.out)[o] += v[i];
+        else unsafeAtomicAdd(reinterpret_cast<float*>(a.out) + o, v[i]);
+      }
+    } else if (EPI == kEpiSilu) {
+      const int n = row0[0] + ei;
+      if (n < a.partner) {
+        // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
+        const float g = to_float(bf16_t{f32_to_bf16_bits(v[0])}), u = to_float(bf16_t{f32_to_bf16_bits(v[1])});
+        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
+      }
+    } else {  // kEpiRope
+      const int head = row0[0] / a.hd, d = row0[0] % a.hd + ei;      // d < hd / 2; partner dim d + hd / 2
+      // projections are kept as bfloat16 before the rotation, as in the unfused path
+      float lo = to_float(bf16_t{f32_to_bf16_bits(v[0])}), hi = to_float(bf16_t{f32_to_bf16_bits(v[1])});
+      const int half = a.hd / 2;
+      if (head < a.nq + a.nkv && d < a.rotary_dim / 2 && half == a.rotary_dim / 2) {
+        float sn, cs;
+        sincosf(float(a.positions[t]) * a.inv_freq[d], &sn, &cs);
+        const float rl = lo * cs - hi * sn, rh = hi * cs + lo * sn;
+        lo = rl;
+        hi = rh;
+      }
+      const uint16_t blo = f32_to_bf16_bits(lo), bhi = f32_to_bf16_bits(hi);
+      if (head < a.nq) {
+        uint16_t* q = reinterpret_cast<uint16_t*>(a.out) + size_t(t) * (size_t(a.nq) * a.hd) + head * a.hd;
+        q[d] = blo;
+        q[d + half] = bhi;
+      } else {
+        const int slot = a.slot_mapping[t];
+        if (slot >= 0) {
+          const int page = slot / a.page_size, off = slot % a.page_size;
+          if (head < a.nq + a.nkv) {
+            uint16_t* k = a.k_pool + ((size_t(page) * a.nkv + (head - a.nq)) * a.page_size + off) * a.hd;
+            k[d] = blo;
+            k[d + half] = bhi;
+          } else {
+            uint16_t* vp = a.v_pool + (size_t(page) * a.nkv + (head - a.nq - a.nkv)) * a.hd * a.page_size + off;
+            vp[size_t(d) * a.page_size] = blo;
+            vp[size_t(d + half) * a.page_size] = bhi;
+          }
+        }
+      }
+    }
+  }
+}
+
+static size_t fused_lds_bytes(int TN, bool norm, int K) {
+  return sizeof(float4) * 4 * 2 * TN * 64 + (norm ? sizeof(uint4) * size_t(TN) * 16 * (K / 8 + 1) : 0);
+}
+
+template <int TN, int EPI, bool NORM>
+static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+  const size_t lds = fused_lds_bytes(TN, NORM, a.K);
+  static bool raised = false;
+  if (lds > 48 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fused_kernel<TN, EPI, NORM>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      set_error("sp_gemm_fused: cannot raise the LDS limit: %s", hipGetErrorString(e));
+      return 1;
+    }
+    raised = true;
+  }
+  gemm_fused_kernel<TN, EPI, NORM><<<dim3(blocks, splits), 256, lds, s>>>(a);
+  return check_launch("sp_gemm_fused");
+}
+
+template <int EPI, bool NORM>
+static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+  if (a.T <= 16) return launch_fused<1, EPI, NORM>(s, a, blocks, splits);
+  if (a.T <= 32) return launch_fused<2, EPI, NORM>(s, a, blocks, splits);
+  return launch_fused<4, EPI, NORM>(s, a, blocks, splits);
+}
+
+template <int EPI>
+static int fused_norm(hipStream_t s, const FusedArgs& a, bool norm, int blocks, int splits) {
+  return norm ? fused_tokens<EPI, true>(s, a, blocks, splits) : fused_tokens<EPI, false>(s, a, blocks, splits);
+}
+
+// Whether the fused kernels take this shape.  K in 16-byte rows, T <= 64, and for the norm prologue
+// the normalised activations must fit into LDS beside the reduction buffer.
+static bool fused_shape_ok(int T, int K, bool norm) {
+  if (T < 1 || T > 64 || K % 8) return false;
+  const int TN = T <= 16 ? 1 : T <= 32 ? 2 : 4;
+  return fused_lds_bytes(TN, norm, K) <= 150 * 1024;
+}
+
+}  // namespace sprout
+
+using namespace sprout;
+
+extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w,
+                              float eps, const void* w, int bias_dtype, const void* bias, int mode, void* out, int T,
+                              int N, int K);
+
+extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
+  if (!fused_shape_ok(T, K, norm != 0)) return 0;
+  if (kind == kEpiRope) return hd % 32 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
+  if (kind == kEpiSilu) return N % 32 == 0;
+  return kind == kEpiStore || kind == kEpiAccumulate || kind == kEpiStoreF32;
+}
+
+namespace sprout {
+int gemm_decode_plain(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                      int T, int N, int K) {
+  return sp_gemm_decode((void*)s, x, nullptr, 0, nullptr, 0.f, w, bias_dtype, bias, mode, out, T, N, K);
+}
+}  // namespace sprout
+
+// Plain product through the K-splitting kernel: out = x . w^T (+ bias), modes as sp_gemm.
+// With residual != null the activations are rmsnorm(residual) * norm_w instead of x.
+extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w,
+                              float eps, const void* w, int bias_dtype, const void* bias, int mode, void* out, int T,
+                              int N, int K) {
+  SP_REQUIRE(mode >= 0 && mode <= 2, "sp_gemm_decode: unknown mode %d", mode);
+  SP_REQUIRE(fused_shape_ok(T, K, residual != nullptr), "sp_gemm_decode: shape T=%d K=%d is not taken", T, K);
+  SP_REQUIRE((x || residual) && w && out && N > 0, "sp_gemm_decode: null operand");
+  FusedArgs a = {};
+  a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
+  a.w = (const uint16_t*)w; a.bias = bias; a.bias_bf16 = bias_dtype == kBF16; a.out = out;
+  a.T = T; a.N = N; a.K = K;
+  const int blocks = (N + 31) / 32;
+  int splits = 1;
+  a.k_per_split = (K + 63) / 64 * 64;
+  if (mode == kEpiAccumulate && !residual) {
+    splits = max(1, min((768 + blocks - 1) / blocks, K / 256));
+    a.k_per_split = ((K + splits - 1) / splits + 63) / 64 * 64;
+    splits = (K + a.k_per_split - 1) / a.k_per_split;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  if (mode == kEpiStore) return fused_norm<kEpiStore>(s, a, residual != nullptr, blocks, splits);
+  if (mode == kEpiAccumulate) return fused_norm<kEpiAccumulate>(s, a, residual != nullptr, blocks, splits);
+  return fused_norm<kEpiStoreF32>(s, a, residual != nullptr, blocks, splits);
+}
+
+// q/k/v projection with bias, rotation and cache write.  w is [(nq + 2 nkv) * hd, K] (q, k, v rows).
+// q_out: [T, nq * hd] bfloat16.  Activations: x, or rmsnorm(residual) * norm_w if residual != null.
+extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int norm_w_dtype,
+                                 const void* norm_w, float eps, const void* w, int bias_dtype, const void* bias,
+                                 void* q_out, const int32_t* positions, const float* inv_freq, int rotary_dim,
+                                 const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int K, int nq,
+                                 int nkv, int hd, int page_size) {
+  const int N = (nq + 2 * nkv) * hd;
+  SP_REQUIRE(sp_fused_supported(kEpiRope, T, N, K, hd, rotary_dim, residual != nullptr),
+             "sp_qkv_rope_cache: shape T=%d K=%d hd=%d rotary=%d is not taken", T, K, hd, rotary_dim);
+  SP_REQUIRE((x || residual) && w && q_out && positions && inv_freq && slot_mapping && k_pool && v_pool,
+             "sp_qkv_rope_cache: null operand");
+  FusedArgs a = {};
+  a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
+  a.w = (const uint16_t*)w; a.bias = bias; a.bias_bf16 = bias_dtype == kBF16; a.out = q_out;
+  a.T = T; a.N = N; a.K = K; a.k_per_split = (K + 63) / 64 * 64; a.partner = hd / 2;
+  a.positions = positions; a.inv_freq = inv_freq; a.slot_mapping = slot_mapping;
+  a.k_pool = (uint16_t*)k_pool; a.v_pool = (uint16_t*)v_pool;
+  a.nq = nq; a.nkv = nkv; a.hd = hd; a.page_size = page_size; a.rotary_dim = rotary_dim;
+  const int blocks = (nq + 2 * nkv) * (hd / 32);
+  return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
+}
+
+// out[T, I] = silu(x . w_gate^T) * (x . w_up^T) with w = [gate rows; up rows] of [2 I, K].
+extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype,
+                               const void* norm_w, float eps, const void* w, void* out, int T, int I, int K) {
+  SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr),
+             "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
+  SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
+  FusedArgs a = {};
+  a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
+  a.w = (const uint16_t*)w; a.out = out;
+  a.T = T; a.N = 2 * I; a.K = K; a.k_per_split = (K + 63) / 64 * 64; a.partner = I;
+  return fused_norm<kEpiSilu>((hipStream_t)stream, a, residual != nullptr, (I + 15) / 16, 1);
+}

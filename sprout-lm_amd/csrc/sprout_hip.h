@@ -22,6 +22,21 @@ int sp_rmsnorm(void* stream, const float* x, const int32_t* rows, int w_dtype, c
 int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w, int bias_dtype,
             const void* bias, int mode, int out_dtype, void* out, int T, int N, int K);
 
+// Decode-sized products (T <= 64, bfloat16) with neighbouring work folded in.  Activations are x
+// [T, K] bfloat16, or, with residual != null, rmsnorm(residual [T, K] float32) * norm_w computed inside.
+// sp_fused_supported(kind, ...): kind 0..2 = plain modes of sp_gemm, 3 = sp_qkv_rope_cache, 4 = sp_gate_up_silu.
+int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm);
+int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
+                   const void* w, int bias_dtype, const void* bias, int mode, void* out, int T, int N, int K);
+// q, k, v projection (+ bias), rotation of q and k, q to q_out [T, nq * hd], k and v into the paged pools.
+int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w,
+                      float eps, const void* w, int bias_dtype, const void* bias, void* q_out,
+                      const int32_t* positions, const float* inv_freq, int rotary_dim, const int32_t* slot_mapping,
+                      void* k_pool, void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size);
+// out [T, I] = silu(x . w[:I]^T) * (x . w[I:]^T)
+int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
+                    const void* w, void* out, int T, int I, int K);
+
 // Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
 // inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
 // (= page * page_size + offset; negative: not written).  nkv == 0: only q is rotated.

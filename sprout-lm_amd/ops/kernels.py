@@ -217,6 +217,60 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  float(scale), kind))
 
 
+FUSED_ROPE, FUSED_SILU = 3, 4
+
+
+def fused_supported(kind: int, T: int, N: int, K: int, hd: int = 0, rotary_dim: int = 0, norm: bool = False) -> bool:
+    """Whether the decode-sized fused kernels take this shape (see sprout_hip.h)."""
+    return bool(library().sp_fused_supported(kind, T, N, K, hd, rotary_dim, int(norm)))
+
+
+def _activations(x, residual, norm_weight, K: int, what: str):
+    """Checks the two ways activations reach a fused kernel; returns (x ptr, residual ptr, norm dtype, norm ptr, T)."""
+    if residual is not None:
+        _gpu(residual, "residual"); _gpu(norm_weight, "norm weight")
+        if residual.dtype != torch.float32 or residual.shape[1] != K or norm_weight.numel() != K:
+            raise KernelError(f"{what}: residual must be float32 [T, {K}] with a norm weight of {K}")
+        return None, residual.data_ptr(), _code(norm_weight, "norm weight"), norm_weight.data_ptr(), residual.shape[0]
+    _gpu(x, "activations")
+    if x.dtype != torch.bfloat16 or x.shape[1] != K:
+        raise KernelError(f"{what}: activations must be bfloat16 [T, {K}], got {x.dtype} {tuple(x.shape)}")
+    return x.data_ptr(), None, 0, None, x.shape[0]
+
+
+def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_freq, rotary_dim: int, slot_mapping,
+                   k_pool, v_pool, nq: int, nkv: int, hd: int, x=None, residual=None, norm_weight=None,
+                   eps: float = 0.0) -> None:
+    """q, k, v = activations . w^T + bias; rotate q and k; q to q_out, k and v into the paged pools.
+
+    Activations are x (bfloat16) or rmsnorm(residual) * norm_weight computed inside the kernel."""
+    _gpu(w, "qkv weight"); _gpu(q_out, "q output")
+    N, K = w.shape
+    xp, rp, nd, npt, T = _activations(x, residual, norm_weight, K, "qkv_rope_cache")
+    if w.dtype != torch.bfloat16 or N != (nq + 2 * nkv) * hd or tuple(q_out.shape) != (T, nq * hd) or q_out.dtype != torch.bfloat16:
+        raise KernelError("qkv_rope_cache: weight or q output does not fit the head counts")
+    if bias is not None:
+        _gpu(bias, "qkv bias")
+        if bias.numel() != N:
+            raise KernelError("qkv_rope_cache: bias size")
+    _ints(positions, T, "positions"); _ints(slot_mapping, T, "slot_mapping"); _gpu(inv_freq, "inv_freq")
+    _, page_size = _check_pools(k_pool, v_pool, nkv, hd, torch.bfloat16, "qkv_rope_cache")
+    check(library().sp_qkv_rope_cache(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(),
+                                      _code(bias, "bias") if bias is not None else 0, _ptr(bias), q_out.data_ptr(),
+                                      positions.data_ptr(), inv_freq.data_ptr(), rotary_dim, slot_mapping.data_ptr(),
+                                      k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd, page_size))
+
+
+def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0) -> None:
+    """out = silu(a . w[:I]^T) * (a . w[I:]^T) for activations a as in `qkv_rope_cache`."""
+    _gpu(w, "gate/up weight"); _gpu(out, "gated output")
+    N, K = w.shape
+    xp, rp, nd, npt, T = _activations(x, residual, norm_weight, K, "gate_up_silu")
+    if w.dtype != torch.bfloat16 or N % 2 or tuple(out.shape) != (T, N // 2) or out.dtype != torch.bfloat16:
+        raise KernelError("gate_up_silu: weight [2 I, K] and output [T, I] bfloat16 expected")
+    check(library().sp_gate_up_silu(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), out.data_ptr(), T, N // 2, K))
+
+
 def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
     """out[t, i] = silu(gu[t, i]) * gu[t, I + i]."""
     _gpu(gu, "gate/up"); _gpu(out, "gated output")

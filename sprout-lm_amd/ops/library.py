@@ -26,6 +26,12 @@ def _declare(lib):
                          c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_float, c_int],
         "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
+        "sp_fused_supported": [c_int] * 7,
+        "sp_gemm_decode": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_void, c_int,
+                           c_int, c_int],
+        "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,
+                              c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int],
+        "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int],
         "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int],
         "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],

@@ -8,6 +8,7 @@ import torch
 from .. import ops
 from ..cache.spec import PagedKVSpec
 from ..weights.loader import TensorSpec
+from .norm import RMSNorm
 from .base import Mixer, register_part
 
 
@@ -62,8 +63,41 @@ class Attention(Mixer):
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
+    def _fused(self, T: int, cache, norm: bool) -> bool:
+        """Whether the decode-sized fused projection kernel takes this call."""
+        return (self.own_kv and cache.writes and self.w_qkv.dtype == torch.bfloat16
+                and ops.fused_supported(ops.FUSED_ROPE, T, self.w_qkv.shape[0], self.hidden, self.head_dim,
+                                        self.position.rotary_dim, norm))
+
+    def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
+        T = residual.shape[0]
+        if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, cache, True):
+            return False
+        q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
+        ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
+                           cache.slot_mapping, cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
+                           residual=residual, norm_weight=norm.w["weight"], eps=norm.eps)
+        self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
+        return True
+
+    def _attend(self, ctx, q, q_stride, residual, cache):
+        T = q.shape[0]
+        attn = ctx.buffer("attn", (T, self.heads * self.head_dim), ctx.act_dtype)
+        ops.attention(q, q_stride, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads, self.kv_heads,
+                      self.head_dim, self.window, self.scale,
+                      workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
+                      kind=ctx.attention_kind)
+        ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)
+
     def forward(self, ctx, h, residual, cache):
         T = h.shape[0]
+        if ctx.act_dtype == torch.bfloat16 and T <= 64 and self._fused(T, cache, False):
+            q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
+            ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq,
+                               self.position.rotary_dim, cache.slot_mapping, cache.k, cache.v, self.heads,
+                               self.kv_heads, self.head_dim, x=h)
+            self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
+            return
         nkv = self.kv_heads if (self.own_kv and cache.writes) else 0
         width = (self.heads + 2 * nkv) * self.head_dim
         qkv = ctx.buffer("qkv", (T, width), ctx.act_dtype)
@@ -75,9 +109,4 @@ class Attention(Mixer):
         ops.rope_cache(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim, self.heads, nkv,
                        self.head_dim, cache.slot_mapping if nkv else None, cache.k if nkv else None,
                        cache.v if nkv else None)
-        attn = ctx.buffer("attn", (T, self.heads * self.head_dim), ctx.act_dtype)
-        ops.attention(qkv, width, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads, self.kv_heads,
-                      self.head_dim, self.window, self.scale,
-                      workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
-                      kind=ctx.attention_kind)
-        ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)
+        self._attend(ctx, qkv, width, residual, cache)

@@ -80,14 +80,23 @@ class Mixer(Part):
         return None
 
     def forward(self, ctx, h, residual, cache):
-        """residual += mixer(h).  `cache` is this call's cache slot (`ctx.cache_slot(...)` view) or None."""
+        """residual += mixer(h).  `cache` is this call's cache slot view (engine.batch.CacheSlotView) or None."""
         raise NotImplementedError
+
+    def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
+        """Optional shortcut: residual += mixer(norm(residual)) with the norm folded into the mixer's
+        first kernel.  Returns False (and does nothing) where the mixer has no such kernel."""
+        return False
 
 
 class FeedForward(Part):
     def forward(self, ctx, h, residual):
         """residual += feed_forward(h), token by token."""
         raise NotImplementedError
+
+    def forward_from_residual(self, ctx, norm, residual) -> bool:
+        """Optional shortcut, as Mixer.forward_from_residual."""
+        return False
 
 
 class Block(Part):

@@ -19,7 +19,9 @@ class PreNormBlock(Block):
     def forward(self, ctx, residual, cache):
         T, H = residual.shape
         h = ctx.buffer("normed", (T, H), ctx.act_dtype)
-        self.mixer_norm.forward(ctx, residual, h)
-        self.mixer.forward(ctx, h, residual, cache)
-        self.ffn_norm.forward(ctx, residual, h)
-        self.ffn.forward(ctx, h, residual)
+        if not self.mixer.forward_from_residual(ctx, self.mixer_norm, residual, cache):
+            self.mixer_norm.forward(ctx, residual, h)
+            self.mixer.forward(ctx, h, residual, cache)
+        if not self.ffn.forward_from_residual(ctx, self.ffn_norm, residual):
+            self.ffn_norm.forward(ctx, residual, h)
+            self.ffn.forward(ctx, h, residual)

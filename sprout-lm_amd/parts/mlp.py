@@ -5,6 +5,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import TensorSpec
+from .norm import RMSNorm
 from .base import FeedForward, register_part
 
 
@@ -29,10 +30,26 @@ class GatedMLP(FeedForward):
         self.w_down = tensors["down_proj.weight"]
         self.w = {}
 
+    def _fused(self, T: int, norm: bool) -> bool:
+        return self.w_gate_up.dtype == torch.bfloat16 and ops.fused_supported(ops.FUSED_SILU, T, 2 * self.inner,
+                                                                               self.hidden, norm=norm)
+
+    def forward_from_residual(self, ctx, norm, residual) -> bool:
+        T = residual.shape[0]
+        if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
+            return False
+        act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
+        ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=norm.w["weight"], eps=norm.eps)
+        ops.gemm(act, self.w_down, residual, accumulate=True)
+        return True
+
     def forward(self, ctx, h, residual):
         T = h.shape[0]
-        gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
-        ops.gemm(h, self.w_gate_up, gu)
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        ops.silu_mul(gu, act)
+        if ctx.act_dtype == torch.bfloat16 and T <= 64 and self._fused(T, False):
+            ops.gate_up_silu(self.w_gate_up, act, x=h)
+        else:
+            gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
+            ops.gemm(h, self.w_gate_up, gu)
+            ops.silu_mul(gu, act)
         ops.gemm(act, self.w_down, residual, accumulate=True)

@@ -300,3 +300,74 @@ def test_sampling_greedy_ties_nonfinite_and_temperature():
     cold = torch.full((4000,), 0.05, device=DEV)
     ops.sample(S, out, ws, cold, seed, counter)
     assert (out == 0).float().mean().item() > 0.99
+
+
+# ---- decode-sized fused kernels --------------------------------------------------------------------
+
+def _normed(res, w, eps):
+    x = res.astype(np.float64)
+    return bf16(x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * w)
+
+
+@pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64])
+@pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
+    from sprout_lm_amd import ops
+    if not ops.fused_supported(ops.FUSED_ROPE, T, (nq + 2 * nkv) * hd, K, hd, hd, norm):
+        pytest.skip("shape not taken by the fused kernel")
+    rng = np.random.default_rng(T * 7 + hd)
+    N, pages, theta, eps = (nq + 2 * nkv) * hd, 40, 10000.0, 1e-5
+    w = bf16(rng.standard_normal((N, K)) / math.sqrt(K))
+    b = bf16(rng.standard_normal(N) * 0.3)
+    res = (rng.standard_normal((T, K)) * 2).astype(np.float32)
+    nw = bf16(rng.uniform(0.5, 1.5, K))
+    x = _normed(res, nw, eps) if norm else bf16(res)
+    pos = rng.integers(0, 300, T)
+    slots = rng.permutation(pages * page)[:T].astype(np.int32)
+    if T > 2:
+        slots[2] = -1
+    inv = torch.tensor(theta ** (-2.0 * np.arange(hd // 2) / hd), dtype=torch.float32, device=DEV)
+    kp = torch.zeros(pages, nkv, page, hd, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(pages, nkv, hd, page, dtype=torch.bfloat16, device=DEV)
+    q_out = torch.full((T, nq * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    args = dict(residual=t(res), norm_weight=t(nw, torch.bfloat16), eps=eps) if norm else dict(x=t(x, torch.bfloat16))
+    ops.qkv_rope_cache(t(w, torch.bfloat16), t(b, torch.bfloat16), q_out, t(pos, torch.int32), inv, hd, t(slots, torch.int32),
+                       kp, vp, nq, nkv, hd, **args)
+    qkv = bf16(x.astype(np.float64) @ w.astype(np.float64).T + b)
+    want = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, hd, theta)
+    got_q = q_out.float().cpu().numpy()
+    scale = 1 + np.abs(want).max()
+    assert np.abs(got_q - want[:, :nq * hd]).max() <= 2 ** -7 * scale
+    kp, vp = kp.float().cpu().numpy(), vp.float().cpu().numpy().transpose(0, 1, 3, 2)
+    for i in range(T):
+        if slots[i] < 0:
+            continue
+        pg, off = divmod(int(slots[i]), page)
+        assert np.abs(kp[pg, :, off].reshape(-1) - want[i, nq * hd:]).max() <= 2 ** -7 * scale
+        assert np.abs(vp[pg, :, off].reshape(-1) - qkv[i, (nq + nkv) * hd:]).max() <= 2 ** -7 * scale
+    written = np.zeros((pages, page), bool)
+    written[[s // page for s in slots if s >= 0], [s % page for s in slots if s >= 0]] = True
+    assert np.all((kp == 0) | written[:, None, :, None]) and np.all((vp == 0) | written[:, None, :, None])
+
+
+@pytest.mark.parametrize("T", [1, 8, 16, 33, 64])
+@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
+    from sprout_lm_amd import ops
+    if not ops.fused_supported(ops.FUSED_SILU, T, 2 * I, K, norm=norm):
+        pytest.skip("shape not taken by the fused kernel")
+    rng = np.random.default_rng(T + I)
+    eps = 1e-6
+    w = bf16(rng.standard_normal((2 * I, K)) / math.sqrt(K) * 2)
+    res = (rng.standard_normal((T, K)) * 3).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)       # a norm weight kept in 32-bit
+    x = _normed(res, nw, eps) if norm else bf16(res)
+    args = dict(residual=t(res), norm_weight=t(nw), eps=eps) if norm else dict(x=t(x, torch.bfloat16))
+    out = torch.empty(T, I, dtype=torch.bfloat16, device=DEV)
+    ops.gate_up_silu(t(w, torch.bfloat16), out, **args)
+    gu = bf16(x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float64)
+    g, u = gu[:, :I], gu[:, I:]
+    want = g / (1 + np.exp(-g)) * u
+    assert np.abs(out.float().cpu().numpy() - want).max() <= 2 ** -6 * (1 + np.abs(want).max())
