@@ -72,33 +72,80 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
 
+  // The first weights are requested before anything else: they do not depend on the prologue, and
+  // their way from memory is the longest wait of the kernel.
+  const int steps = (k_end - k_begin + 63) / 64;
+  uint4 wa[4][2][2];
+  auto load_weights = [&](int s0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
+      const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        wa[u][i][0] = in0 ? ldg128(wrow[i] + k) : make_uint4(0, 0, 0, 0);
+        wa[u][i][1] = in1 ? ldg128(wrow[i] + k + 8) : make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  load_weights(wave);
+  __builtin_amdgcn_sched_barrier(0);   // keep these loads ahead of the prologue
+
   if (NORM) {
-    // 16 threads per token: sum of squares, then the normalised row as bfloat16 into LDS
-    for (int t0 = 0; t0 < TN * 16; t0 += 16) {
-      const int t = t0 + (threadIdx.x >> 4), part = threadIdx.x & 15;
-      float sum = 0.f;
-      if (t < a.T)
-        for (int k = part * 4; k < a.K; k += 64) {
-          const float4 v = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k);
-          sum = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sum))));
-        }
+    // RMSNorm of up to 16 tokens: 16 threads per token, each owning every 16th group of four columns,
+    // so that a token's loads are all in flight together and its sum closes with four lane exchanges.
+    const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
+    const float* row = a.residual + size_t(min(t, a.T - 1)) * a.K;     // rows past T repeat the last one
+    float4 v[16], wn[16];
+    auto load_values = [&](int k0) {
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-      const float scale = 1.0f / sqrtf(sum / float(a.K) + a.eps);
-      for (int k = part * 8; k < a.K; k += 128) {
-        uint4 packed = make_uint4(0, 0, 0, 0);
-        if (t < a.T) {
-          const float4 v0 = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k);
-          const float4 v1 = *reinterpret_cast<const float4*>(a.residual + size_t(t) * a.K + k + 4);
-          const float n[8] = {v0.x * scale, v0.y * scale, v0.z * scale, v0.w * scale,
-                              v1.x * scale, v1.y * scale, v1.z * scale, v1.w * scale};
-          float y[8];
+      for (int j = 0; j < 16; ++j) {
+        const int k = k0 + 4 * part + 64 * j;
+        v[j] = k < a.K ? *reinterpret_cast<const float4*>(row + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    };
+    auto load_norm_weights = [&](int k0) {   // one vector load per group of four columns
+      if (a.norm_w_bf16) {
+        const uint16_t* nw = reinterpret_cast<const uint16_t*>(a.norm_w);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) y[i] = n[i] * load_param(a.norm_w, a.norm_w_bf16, k + i);
-          packed = make_uint4(pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3]), pack_bf16x2(y[4], y[5]),
-                              pack_bf16x2(y[6], y[7]));
+        for (int j = 0; j < 16; ++j) {
+          const int k = k0 + 4 * part + 64 * j;
+          const uint2 b = k < a.K ? *reinterpret_cast<const uint2*>(nw + k) : make_uint2(0, 0);
+          wn[j] = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
+                              __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
         }
-        xs[t * LD + (k >> 3)] = packed;
+      } else {
+        const float* nw = reinterpret_cast<const float*>(a.norm_w);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int k = k0 + 4 * part + 64 * j;
+          wn[j] = k < a.K ? *reinterpret_cast<const float4*>(nw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    };
+    float sum = 0.f;
+    for (int k0 = 0; k0 < a.K; k0 += 1024) {
+      load_values(k0);
+      if (a.K <= 1024) load_norm_weights(0);               // requested together with the values
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sum = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, sum))));
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    const float scale = rsqrtf(sum / float(a.K) + a.eps);
+    for (int k0 = 0; k0 < a.K; k0 += 1024) {
+      if (a.K > 1024) {                                    // wide rows: the values are read again
+        load_values(k0);
+        load_norm_weights(k0);
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int k = k0 + 4 * part + 64 * j;
+        if (k < a.K) {
+          uint2* dst = reinterpret_cast<uint2*>(xs + t * LD) + (k >> 2);
+          *dst = make_uint2(pack_bf16x2(v[j].x * scale * wn[j].x, v[j].y * scale * wn[j].y),
+                            pack_bf16x2(v[j].z * scale * wn[j].z, v[j].w * scale * wn[j].w));
+        }
       }
     }
     __syncthreads();
@@ -111,18 +158,13 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // this wave's steps of 64 along K: wave, wave + 4, ...; four steps are loaded before they are multiplied
-  const int steps = (k_end - k_begin + 63) / 64;
   for (int s0 = wave; s0 < steps; s0 += 16) {
-    uint4 wa[4][2][2], xb[4][TN][2];
+    if (s0 != wave) load_weights(s0);
+    uint4 xb[4][TN][2];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
       const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        wa[u][i][0] = in0 ? ldg128(wrow[i] + k) : make_uint4(0, 0, 0, 0);
-        wa[u][i][1] = in1 ? ldg128(wrow[i] + k + 8) : make_uint4(0, 0, 0, 0);
-      }
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn) {
         const int t = tn * 16 + lr;
@@ -258,10 +300,11 @@ static int fused_norm(hipStream_t s, const FusedArgs& a, bool norm, int blocks, 
   return norm ? fused_tokens<EPI, true>(s, a, blocks, splits) : fused_tokens<EPI, false>(s, a, blocks, splits);
 }
 
-// Whether the fused kernels take this shape.  K in 16-byte rows, T <= 64, and for the norm prologue
-// the normalised activations must fit into LDS beside the reduction buffer.
+// Whether the fused kernels take this shape.  K in 16-byte rows, T <= 64; the norm prologue takes up to
+// 16 tokens, whose normalised activations must fit into LDS beside the reduction buffer.
 static bool fused_shape_ok(int T, int K, bool norm) {
   if (T < 1 || T > 64 || K % 8) return false;
+  if (norm && T > 16) return false;   // the prologue normalises one tile of 16 tokens
   const int TN = T <= 16 ? 1 : T <= 32 ? 2 : 4;
   return fused_lds_bytes(TN, norm, K) <= 150 * 1024;
 }

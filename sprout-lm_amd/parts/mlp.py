@@ -34,8 +34,12 @@ class GatedMLP(FeedForward):
         return self.w_gate_up.dtype == torch.bfloat16 and ops.fused_supported(ops.FUSED_SILU, T, 2 * self.inner,
                                                                                self.hidden, norm=norm)
 
+    fuse_input_norm = False   # see Attention.fuse_input_norm: no gain measured on MI355X
+
     def forward_from_residual(self, ctx, norm, residual) -> bool:
         T = residual.shape[0]
+        if not self.fuse_input_norm:
+            return False
         if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
             return False
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
