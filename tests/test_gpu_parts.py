@@ -1,0 +1,347 @@
+"""Each part alone against its plain function, and a toy architecture defined here that the engine
+has never seen: a mixer with state of its own, a windowed attention layer in a cache group of its
+own, a layer that runs twice, and a layer that reads another layer's cache."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def dev(x, dtype=torch.float32):
+    return torch.as_tensor(np.asarray(x)).to(DEV).to(dtype).contiguous()
+
+
+class PartHarness:
+    """Runs one part on a batch of sequences through the engine's own cache manager and batch builder."""
+
+    def __init__(self, cache_specs, dtype, page_size=8, pages=64):
+        from sprout_lm_amd.cache import CacheManager
+        from sprout_lm_amd.engine.batch import DescriptorStager, Workspace
+        self.dtype = dtype
+        self.cache = CacheManager(cache_specs, page_size, pages, 8, prefix_caching=False)
+        self.cache.attach_storage(dtype, DEV)
+        self.workspace, self.stager = Workspace(DEV), DescriptorStager(DEV)
+
+    def context(self, seqs_and_counts):
+        from sprout_lm_amd.engine.batch import StepEntry, build_context
+        entries = []
+        for seq, n in seqs_and_counts:
+            assert self.cache.reserve(seq, seq.length + n)
+            entries.append(StepEntry(seq, [0] * n, []))
+        return build_context(entries, self.cache, self.stager, self.workspace, self.dtype,
+                             1 if self.dtype == torch.float32 else 0), entries
+
+    def slot_view(self, ctx, slot, writes=True):
+        from sprout_lm_amd.engine.batch import CacheSlotView
+        kind, g, index = self.cache.slot_location[slot]
+        group = self.cache.groups[g]
+        return CacheSlotView(writes, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
+                             slot_mapping=ctx.group_slots[g], page_size=self.cache.block_size)
+
+    def commit(self, entries):
+        for e in entries:
+            self.cache.commit(e.seq, e.seq.length + len(e.tokens))
+
+
+def rounded(x, dtype):
+    return P.bf16_round(x) if dtype == torch.bfloat16 else np.asarray(x, np.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_embedding_head_parts(dtype):
+    from sprout_lm_amd.parts import make_part
+    rng = np.random.default_rng(0)
+    Hd, V = 72, 131
+    norm = make_part("norm", "rmsnorm", size=Hd, eps=1e-4)
+    w = rounded(rng.uniform(0.5, 1.5, Hd), dtype)
+    norm.bind({"weight": dev(w, dtype)})
+    x = rng.standard_normal((5, Hd)).astype(np.float32)
+    out = torch.empty(5, Hd, dtype=dtype, device=DEV)
+    norm.forward(None, dev(x), out)
+    tol = 2e-6 if dtype == torch.float32 else 2 ** -8
+    assert np.abs(out.float().cpu().numpy() - P.rms_norm(x, w, 1e-4)).max() <= tol * 4
+    table = rounded(rng.standard_normal((V, Hd)), dtype)
+    emb = make_part("embedding", "token_embedding", vocab=V, hidden=Hd)
+    emb.bind({"weight": dev(table, dtype)})
+    res = torch.empty(3, Hd, device=DEV)
+    emb.forward(None, torch.tensor([130, 0, 7], dtype=torch.int32, device=DEV), res)
+    assert np.array_equal(res.cpu().numpy(), table[[130, 0, 7]])
+    head = make_part("head", "linear_head", vocab=V, hidden=Hd, tied=True)
+    head.bind({})
+    head.tie(emb.w["weight"])
+    hrows = rounded(rng.standard_normal((3, Hd)), dtype)
+    logits = torch.empty(3, V, device=DEV)
+    head.forward(None, dev(hrows, dtype), logits)
+    assert np.abs(logits.cpu().numpy() - P.linear(hrows, table)).max() <= 1e-4
+    assert make_part("head", "linear_head", vocab=V, hidden=Hd, tied=False).tensors()["weight"].shape == (V, Hd)
+
+
+def attention_weights(rng, hidden, heads, kv_heads, hd, dtype, own_kv=True):
+    names = [("q_proj", heads * hd)] + ([("k_proj", kv_heads * hd), ("v_proj", kv_heads * hd)] if own_kv else [])
+    w = {}
+    for name, rows in names:
+        w[f"{name}.weight"] = rounded(rng.standard_normal((rows, hidden)) * 0.2, dtype)
+        w[f"{name}.bias"] = rounded(rng.uniform(-0.3, 0.3, rows), dtype)
+    w["o_proj.weight"] = rounded(rng.standard_normal((hidden, heads * hd)) * 0.2, dtype)
+    return w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,hd,window", [(4, 2, 16, None), (3, 1, 32, None), (6, 2, 48, 7), (2, 2, 64, 20)])
+def test_attention_part_alone_in_portions(dtype, heads, kv_heads, hd, window):
+    """One attention part, two sequences fed in uneven portions beside each other, against the plain function."""
+    from sprout_lm_amd.models.plan import PartPlan
+    rng = np.random.default_rng(heads * 10 + hd)
+    hidden, theta = 40, 5000.0
+    part = PartPlan("mixer", "attention", {"hidden": hidden, "heads": heads, "kv_heads": kv_heads, "head_dim": hd,
+                                           "position": PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": theta}),
+                                           "window": window}).make()
+    w = attention_weights(rng, hidden, heads, kv_heads, hd, dtype)
+    part.bind({k: dev(v, dtype) for k, v in w.items()})
+    part.prepare(DEV, dtype)
+    harness = PartHarness([part.cache_spec()], dtype)
+    lengths = [37, 22]
+    hs = [rounded(rng.standard_normal((n, hidden)), dtype) for n in lengths]
+    store = P.bf16_round if dtype == torch.bfloat16 else P.f32
+    want = []
+    for h in hs:   # the plain mixer: projections, rotation, attention, output projection
+        pos = np.arange(len(h))
+        q = store(P.rope_neox(store(P.linear(h, w["q_proj.weight"], w["q_proj.bias"])), pos, hd, theta))
+        k = store(P.rope_neox(store(P.linear(h, w["k_proj.weight"], w["k_proj.bias"])), pos, hd, theta))
+        v = store(P.linear(h, w["v_proj.weight"], w["v_proj.bias"]))
+        a = store(P.causal_gqa_attention(q, k, v, heads, kv_heads, hd, window=window))
+        want.append(P.linear(a, w["o_proj.weight"]))
+    seqs = [harness.cache.create() for _ in lengths]
+    fed = [0, 0]
+    got = [np.zeros((n, hidden), np.float32) for n in lengths]
+    portions = [(16, 1), (5, 9), (1, 1), (2, 3), (13, 8)]
+    for step in portions:
+        batch = [(s, min(n, lengths[i] - fed[i])) for i, (s, n) in enumerate(zip(seqs, step)) if fed[i] < lengths[i]]
+        index = [i for i in range(2) if fed[i] < lengths[i]]
+        ctx, entries = harness.context(batch)
+        h = torch.cat([dev(hs[i][fed[i]:fed[i] + n], dtype) for i, (_, n) in zip(index, batch)])
+        residual = torch.zeros(h.shape[0], hidden, device=DEV)
+        part.forward(ctx, h, residual, harness.slot_view(ctx, 0))
+        out = residual.cpu().numpy()
+        harness.commit(entries)
+        row = 0
+        for i, (_, n) in zip(index, batch):
+            got[i][fed[i]:fed[i] + n] = out[row:row + n]
+            fed[i] += n
+            row += n
+    assert fed == lengths
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for g, wnt in zip(got, want):
+        assert np.abs(g - wnt).max() <= tol * (1 + np.abs(wnt).max())
+    if window:   # pages that the window has passed came back
+        assert any(p == -1 for p in seqs[0].blocks[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 7, 40, 150])
+def test_feed_forward_and_block_parts(dtype, T):
+    from sprout_lm_amd.models.plan import PartPlan
+    rng = np.random.default_rng(T)
+    hidden, inner = 56, 104
+    cfg = dict(hidden_size=hidden, num_attention_heads=1, num_key_value_heads=1, rms_norm_eps=1e-5, rope_theta=1e4)
+    w = {"model.layers.0.mlp.gate_proj.weight": rounded(rng.standard_normal((inner, hidden)) * 0.2, dtype),
+         "model.layers.0.mlp.up_proj.weight": rounded(rng.standard_normal((inner, hidden)) * 0.2, dtype),
+         "model.layers.0.mlp.down_proj.weight": rounded(rng.standard_normal((hidden, inner)) * 0.2, dtype),
+         "model.layers.0.post_attention_layernorm.weight": rounded(rng.uniform(0.7, 1.3, hidden), dtype)}
+    ffn = PartPlan("feed_forward", "gated_mlp", {"hidden": hidden, "inner": inner}).make()
+    ffn.bind({k.split("mlp.")[1]: dev(v, dtype) for k, v in w.items() if "mlp." in k})
+    harness = PartHarness([], dtype)
+    ctx, _ = harness.context([])
+    h = rounded(rng.standard_normal((T, hidden)), dtype)
+    base = rng.standard_normal((T, hidden)).astype(np.float32)
+    residual = dev(base)
+    ffn.forward(ctx, dev(h, dtype), residual)
+    store = P.bf16_round if dtype == torch.bfloat16 else P.f32
+    gate = store(P.linear(h, w["model.layers.0.mlp.gate_proj.weight"]))
+    up = store(P.linear(h, w["model.layers.0.mlp.up_proj.weight"]))
+    want = base + P.linear(store(P.swiglu(gate, up)), w["model.layers.0.mlp.down_proj.weight"])
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    assert np.abs(residual.cpu().numpy() - want).max() <= tol * (1 + np.abs(want).max())
+    with pytest.raises(ValueError, match="silu"):
+        PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "gelu"}).make()
+
+
+# ----------------------------------------------------------------------------------------------------
+# A toy architecture, registered here and nowhere in the engine.
+
+def register_toy():
+    from dataclasses import dataclass
+    from typing import ClassVar
+
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cache import StateSpec
+    from sprout_lm_amd.config.base import ModelConfig
+    from sprout_lm_amd.models.plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+    from sprout_lm_amd.parts import Mixer, register_part, registered_parts
+    from sprout_lm_amd.weights import TensorSpec
+
+    if "toy_running_mean" in registered_parts("mixer"):
+        return
+
+    @register_part("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """y_t = W . mean(h_0 .. h_t): the state per request is the running sum and the count."""
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def cache_spec(self):
+            return StateSpec((self.hidden + 1,), "float32")
+
+        def tensors(self):
+            return {"proj.weight": TensorSpec((self.hidden, self.hidden))}
+
+        def forward(self, ctx, h, residual, cache):
+            for start, n, slot in zip(ctx.host["q_start"], ctx.host["q_len"], ctx.host["state_slots"]):
+                state = cache.state[slot]
+                sums = torch.cumsum(h[start:start + n].float(), 0) + state[:-1]
+                counts = state[-1] + torch.arange(1, n + 1, device=h.device)
+                mean = (sums / counts[:, None]).to(h.dtype).float()
+                residual[start:start + n] += mean @ self.w["proj.weight"].float().T
+                state[:-1] = sums[-1]
+                state[-1] = counts[-1]
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyMeanForCausalLM"
+        model_types: ClassVar[tuple] = ("toy_mean",)
+        hidden: int = 0
+        inner: int = 0
+        vocab: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        window: int = 0
+        eps: float = 0.0
+        theta: float = 0.0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "window", "eps", "theta")})
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "model_type": "toy_mean", "hidden": self.hidden,
+                    "inner": self.inner, "vocab": self.vocab, "heads": self.heads, "kv_heads": self.kv_heads,
+                    "window": self.window, "eps": self.eps, "theta": self.theta}
+
+    def build_toy(cfg):
+        hd = cfg.hidden // cfg.heads
+        norm = lambda prefix: PartPlan("norm", "rmsnorm", {"size": cfg.hidden, "eps": cfg.eps}, prefix)
+        rotary = lambda: PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": cfg.theta})
+        attention = lambda prefix, **extra: PartPlan("mixer", "attention", {
+            "hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.kv_heads, "head_dim": hd, "position": rotary(),
+            **extra}, prefix)
+        mlp = lambda prefix: PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner}, prefix)
+        mixers = [attention("l0.attn."), PartPlan("mixer", "toy_running_mean", {"hidden": cfg.hidden}, "l1.mean."),
+                  attention("l2.attn.", window=cfg.window), attention("l3.attn.", own_kv=False)]
+        layers = [LayerPlan("pre_norm", {"mixer_norm": norm(f"l{i}.n1."), "mixer": m, "ffn_norm": norm(f"l{i}.n2."),
+                                         "ffn": mlp(f"l{i}.mlp.")}) for i, m in enumerate(mixers)]
+        # layer 0 runs twice (slots 0 and 3); layer 3 reads what layer 0's first run cached
+        schedule = [LayerCall(0, 0), LayerCall(1, 1), LayerCall(2, 2), LayerCall(3, 0, writes=False), LayerCall(0, 3)]
+        return ModelPlan("ToyMeanForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
+                         PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.hidden}, "embed."),
+                         layers, schedule, norm("final."),
+                         PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.hidden, "tied": True}, "head."))
+
+    S.register_architecture("ToyMeanForCausalLM", ToyConfig, build_toy, model_types=("toy_mean",))
+
+
+TOY = dict(model_type="toy_mean", hidden=48, inner=80, vocab=97, heads=3, kv_heads=1, window=6, eps=1e-5, theta=1e4)
+
+
+def plain_toy_logits(w, tokens, store):
+    c = TOY
+    hd = c["hidden"] // c["heads"]
+    pos = np.arange(len(tokens))
+    x = P.f32(w["embed.weight"][np.asarray(tokens)])
+
+    def mlp(x, i):
+        n = store(P.rms_norm(x, w[f"l{i}.n2.weight"], c["eps"]))
+        gate, up = store(P.linear(n, w[f"l{i}.mlp.gate_proj.weight"])), store(P.linear(n, w[f"l{i}.mlp.up_proj.weight"]))
+        return P.f32(x + P.linear(store(P.swiglu(gate, up)), w[f"l{i}.mlp.down_proj.weight"]))
+
+    def attn(x, i, window=None, kv=None):
+        n = store(P.rms_norm(x, w[f"l{i}.n1.weight"], c["eps"]))
+        p = f"l{i}.attn."
+        q = store(P.rope_neox(store(P.linear(n, w[p + "q_proj.weight"], w[p + "q_proj.bias"])), pos, hd, c["theta"]))
+        if kv is None:
+            k = store(P.rope_neox(store(P.linear(n, w[p + "k_proj.weight"], w[p + "k_proj.bias"])), pos, hd, c["theta"]))
+            v = store(P.linear(n, w[p + "v_proj.weight"], w[p + "v_proj.bias"]))
+        else:
+            k, v = kv
+        a = store(P.causal_gqa_attention(q, k, v, c["heads"], c["kv_heads"], hd, window=window))
+        return P.f32(x + P.linear(a, w[p + "o_proj.weight"])), (k, v)
+
+    x, kv0 = attn(x, 0)
+    x = mlp(x, 0)
+    n = store(P.rms_norm(x, w["l1.n1.weight"], c["eps"])).astype(np.float64)
+    mean = store(np.cumsum(n, 0) / np.arange(1, len(tokens) + 1)[:, None])
+    x = mlp(P.f32(x + P.linear(mean, w["l1.mean.proj.weight"])), 1)
+    x, _ = attn(x, 2, window=c["window"])
+    x = mlp(x, 2)
+    x, _ = attn(x, 3, kv=kv0)
+    x = mlp(x, 3)
+    x, _ = attn(x, 0)
+    x = mlp(x, 0)
+    return P.linear(store(P.rms_norm(x, w["final.weight"], c["eps"])), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
+    register_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    folder = str(tmp_path / "toy")
+    write_model_folder(folder, S.config_from_dict(TOY), seed=3, dtype=torch.bfloat16, std=0.15)
+    assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["ToyMeanForCausalLM"]
+    runner = ModelRunner.from_folder(folder, dtype, block_size=4, num_blocks=40, max_sequences=3)
+    assert not runner.parts.graph_safe                       # the toy mixer plans on the host: no graph replay
+    kinds = [(g.spec.window, g.slots) for g in runner.cache.groups]
+    assert kinds == [(None, [0, 3]), (6, [2])] and runner.cache.state_groups[0].slots == [1]
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    store = P.bf16_round if dtype == "bfloat16" else P.f32
+    requests = {"a": H.random_tokens(97, 41, 1), "b": H.random_tokens(97, 23, 2), "c": H.random_tokens(97, 30, 3)}
+    want = {k: plain_toy_logits(w, t, store) for k, t in requests.items()}
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    # a and b run beside each other in uneven portions; c starts when b has ended, in b's state slot and pages
+    seqs = {"a": runner.cache.create(), "b": runner.cache.create()}
+    fed = {k: 0 for k in requests}
+    plan = [{"a": 9, "b": 2}, {"a": 1, "b": 13}, {"a": 5, "b": 8}, {"a": 1}, {"a": 3, "c": 11}, {"a": 1, "c": 1},
+            {"a": 21, "c": 2}, {"c": 16}]
+    worst = 0.0
+    for step in plan:
+        if "c" in step and "c" not in seqs:
+            seqs.pop("b").release()
+            seqs["c"] = runner.cache.create()
+        entries, rows = [], []
+        for rid, n in step.items():
+            n = min(n, len(requests[rid]) - fed[rid])
+            assert runner.cache.reserve(seqs[rid], fed[rid] + n)
+            entries.append(StepEntry(seqs[rid], requests[rid][fed[rid]:fed[rid] + n], list(range(n))))
+            rows += [(rid, fed[rid] + i) for i in range(n)]
+            fed[rid] += n
+        got = runner.step(entries).cpu().numpy()
+        for row, (rid, pos) in zip(got, rows):
+            err = np.abs(row - want[rid][pos]).max()
+            worst = max(worst, err)
+            assert err <= tol * (1 + np.abs(want[rid][pos]).max()), f"{rid} position {pos}: {err:.3e}"
+    assert fed == {k: len(v) for k, v in requests.items()}
+    for s in seqs.values():
+        s.release()
+    assert runner.cache.free_pages() == [40, 40]
+    print(f"toy {dtype}: worst error {worst:.3e}")
