@@ -213,6 +213,142 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------ prefill, shared
+// One block per (tile of 16 * NQT queries, key/value head): wave w works on query head g * G + w, and all
+// G waves read the same keys and values, which the block fetches once per step into LDS (next step's
+// loads in flight while the current one is multiplied).  Needs pages of a multiple of 8 tokens.
+template <int DT, int NQT>
+__global__ __launch_bounds__(512) void attention_prefill_shared_kernel(
+    const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
+    const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
+    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_size, int num_pages,
+    int window, float scale2) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  constexpr int KP = HD + 8;          // key row pitch in LDS (elements): 16 bytes of padding
+  constexpr int VP = 32 + 4;          // value row pitch: 32 keys + 8 bytes of padding
+  constexpr int CHUNKS = 8 * HD;      // 16-byte pieces of one step: 4 HD of keys, 4 HD of values
+  constexpr int MAXC = 8;             // pieces per thread with one wave in the block
+  __shared__ __attribute__((aligned(16))) uint16_t ks[2][32 * KP];
+  __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD * VP];
+
+  const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
+  const int g = blockIdx.y, G = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int h = g * G + wave;
+  const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
+  const int nvalid = min(16 * NQT, qlen - q_off);
+  if (nvalid <= 0) return;
+  const int pos0 = ctx - qlen + q_off;
+
+  PagedKV kv;
+  kv.page_size = page_size;
+  kv.num_pages = num_pages;
+  kv.page_stride = size_t(nkv) * page_size * HD;
+  kv.k = k_pool + size_t(g) * page_size * HD;
+  kv.v = v_pool + size_t(g) * page_size * HD;
+  kv.table = block_tables + size_t(seq) * max_blocks;
+
+  bf16x8 qop[NQT][HC];
+  int qpos[NQT];
+  floatx4 o[NQT][DT];
+  float m[NQT], lsum[NQT];
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    const int row = 16 * qt + lr;
+    const bool valid = row < nvalid;
+    qpos[qt] = valid ? pos0 + row : -1;
+    load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
+    m[qt] = -INFINITY;
+    lsum[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int k_hi = pos0 + nvalid - 1;
+  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int per_thread = (CHUNKS + blockDim.x - 1) / blockDim.x;   // <= MAXC for HD <= 64 ... checked on the host
+
+  uint4 stage[MAXC];
+  auto fetch = [&](int key0) {
+#pragma unroll
+    for (int u = 0; u < MAXC; ++u) {
+      const int i = threadIdx.x + u * blockDim.x;
+      if (u < per_thread && i < CHUNKS) {
+        if (i < 4 * HD) {                      // keys: row r of the step, dims 8 c .. 8 c + 7
+          const int r = i / (HD / 8), c = i % (HD / 8);
+          const int key = min(max(key0 + r, k_lo), k_hi);
+          stage[u] = ldg128(kv.k + size_t(page_of(kv, key)) * kv.page_stride + size_t(key % page_size) * HD + 8 * c);
+        } else {                               // values: dim d, keys 8 c .. 8 c + 7 of the step
+          const int j = i - 4 * HD, d = j >> 2, c = j & 3;
+          const int kb = min(max(key0 + 8 * c, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+          stage[u] = ldg128(kv.v + size_t(page_of(kv, kb)) * kv.page_stride + size_t(d) * page_size + kb % page_size);
+        }
+      }
+    }
+  };
+  auto deposit = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < MAXC; ++u) {
+      const int i = threadIdx.x + u * blockDim.x;
+      if (u < per_thread && i < CHUNKS) {
+        if (i < 4 * HD) {
+          const int r = i / (HD / 8), c = i % (HD / 8);
+          *reinterpret_cast<uint4*>(&ks[buf][r * KP + 8 * c]) = stage[u];
+        } else {
+          const int j = i - 4 * HD, d = j >> 2, c = j & 3;
+          uint2* dst = reinterpret_cast<uint2*>(&vs[buf][d * VP + 8 * c]);   // rows are 8-byte aligned
+          dst[0] = make_uint2(stage[u].x, stage[u].y);
+          dst[1] = make_uint2(stage[u].z, stage[u].w);
+        }
+      }
+    }
+  };
+
+  int key0 = (k_lo >> 5) << 5;
+  fetch(key0);
+  deposit(0);
+  __syncthreads();
+  int buf = 0;
+  for (; key0 <= k_hi; key0 += 32, buf ^= 1) {
+    const bool more = key0 + 32 <= k_hi;
+    if (more) fetch(key0 + 32);
+    KVStep<DT> r;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int c = 0; c < HC; ++c) {
+        const int d0 = 32 * c + 8 * lj;
+        r.ka[kt][c] = d0 < HD ? as_bf16x8(*reinterpret_cast<const uint4*>(&ks[buf][(16 * kt + lr) * KP + d0]))
+                              : as_bf16x8(make_uint4(0, 0, 0, 0));
+      }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+        r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[buf][(16 * dt + lr) * VP + 16 * kt + 4 * lj]);
+    attend_step<DT, NQT>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    if (more) deposit(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    float l = lsum[qt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int row = 16 * qt + lr;
+    if (row >= nvalid) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const floatx4 v = o[qt][dt] * inv;
+      *reinterpret_cast<uint2*>(dst + 16 * dt + 4 * lj) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------ decode
 // Partial results of a block, for the merge kernel: part_o [seq][head][split][HD] (not yet divided),
 // part_ml [seq][head][split][2] = (running maximum in log2 units, sum).
@@ -358,7 +494,7 @@ bool attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
   return hd_ok && page_size % 4 == 0;
 }
 bool attention_mfma_decode_supports(int nq, int nkv) { return nq / nkv <= 16; }
-int attention_mfma_tile_q(int hd) { return hd <= 64 ? 64 : 32; }
+int attention_mfma_tile_q(int hd) { return 32; }
 
 size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx) {
   const size_t splits = (max_ctx + kDecodeChunk - 1) / kDecodeChunk;
@@ -372,13 +508,21 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
                        int n_decode, int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int page_size,
                        int num_pages, int window, float scale) {
   constexpr int HD = 16 * DT;
-  constexpr int NQT = HD <= 64 ? 4 : 2;
+  constexpr int NQT = 2;
   const float scale2 = scale * kLog2e;
   const uint16_t *qp = (const uint16_t*)q, *kp = (const uint16_t*)k_pool, *vp = (const uint16_t*)v_pool;
   if (n_tiles > 0) {
-    attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
-        qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
-        page_size, num_pages, window, scale2);
+    const int G = nq / nkv;
+    // the shared kernel stages 8 HD pieces of 16 bytes per step with 64 G threads, at most 8 per thread
+    if (page_size % 8 == 0 && G <= 8 && 8 * HD <= 8 * 64 * G) {
+      attention_prefill_shared_kernel<DT, NQT><<<dim3(n_tiles, nkv), 64 * G, 0, s>>>(
+          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
+          page_size, num_pages, window, scale2);
+    } else {
+      attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
+          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
+          page_size, num_pages, window, scale2);
+    }
     if (check_launch("sp_attention (prefill)")) return 1;
   }
   if (n_decode > 0) {
