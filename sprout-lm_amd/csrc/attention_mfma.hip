@@ -71,12 +71,18 @@ __device__ __forceinline__ void load_step(KVStep<DT>& r, const PagedKV& kv, int 
   }
 }
 
+constexpr float kNoKeyYet = -1.0e30f;   // running maximum before any key: finite, so that no inf - inf arises
+
 // Scores, running softmax and P.V of one loaded step for NQT tiles of 16 rows.
 // qpos[qt]: position of this lane's row (column l % 16 of tile qt), or -1 for a row that does not exist.
-template <int DT, int NQT>
-__device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
-                                            floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT], int key0,
-                                            int k_lo, const int (&qpos)[NQT], int window, float scale2) {
+// MASKED false: every key of the step is visible to every existing row (the caller has checked), and
+// rows that do not exist compute values nobody reads.  The running maximum m is in log2 units and
+// starts at kNoKeyYet.
+template <int DT, int NQT, bool MASKED>
+__device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
+                                                 floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT],
+                                                 int key0, int k_lo, const int (&qpos)[NQT], int window,
+                                                 float scale2) {
   constexpr int HC = (DT + 1) / 2;
   const int lane = threadIdx.x & 63, lj = lane >> 4;
 
@@ -92,33 +98,32 @@ __device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&
 
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
-    float sv[2][4];
-    float mx = m[qt];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int key = key0 + 16 * kt + 4 * lj + r4;
-        const bool visible = key <= qpos[qt] && key >= k_lo && (window <= 0 || qpos[qt] - key < window);
-        sv[kt][r4] = visible ? s[qt][kt][r4] * scale2 : -INFINITY;
-        mx = fmaxf(mx, sv[kt][r4]);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    float alpha = 1.f, p[2][4] = {};
-    if (mx != -INFINITY) {
-      alpha = m[qt] == -INFINITY ? 0.f : exp2f(m[qt] - mx);
-      float sum = 0.f;
+    if (MASKED) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
-          p[kt][r4] = sv[kt][r4] == -INFINITY ? 0.f : exp2f(sv[kt][r4] - mx);
-          sum += p[kt][r4];
+          const int key = key0 + 16 * kt + 4 * lj + r4;
+          const bool visible = key <= qpos[qt] && key >= k_lo && (window <= 0 || qpos[qt] - key < window);
+          if (!visible) s[qt][kt][r4] = -INFINITY;
         }
-      lsum[qt] = lsum[qt] * alpha + sum;
-      m[qt] = mx;
     }
+    float raw = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
+                      fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
+    raw = fmaxf(raw, __shfl_xor(raw, 16, 64));
+    raw = fmaxf(raw, __shfl_xor(raw, 32, 64));
+    const float mx = fmaxf(m[qt], raw * scale2);            // finite: m starts finite
+    const float alpha = __builtin_amdgcn_exp2f(m[qt] - mx);
+    m[qt] = mx;
+    float p[2][4], sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        p[kt][r4] = __builtin_amdgcn_exp2f(fmaf(s[qt][kt][r4], scale2, -mx));   // exp2(-inf) = 0 for masked keys
+        sum += p[kt][r4];
+      }
+    lsum[qt] = fmaf(lsum[qt], alpha, sum);
     const uint4 pb = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                                 pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
 #pragma unroll
@@ -129,6 +134,19 @@ __device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&
       o[qt][dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
     }
   }
+}
+
+// `first_pos`: smallest position among the rows that exist; a step whose 32 keys all lie at or before
+// it (and inside [k_lo, ...) with no window) needs no masking.
+template <int DT, int NQT>
+__device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
+                                            floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT], int key0,
+                                            int k_lo, const int (&qpos)[NQT], int window, float scale2,
+                                            int first_pos) {
+  if (window <= 0 && key0 >= k_lo && key0 + 31 <= first_pos)
+    attend_step_impl<DT, NQT, false>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+  else
+    attend_step_impl<DT, NQT, true>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
 }
 
 template <int DT>
@@ -177,7 +195,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
     const bool valid = row < nvalid;
     qpos[qt] = valid ? pos0 + row : -1;
     load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
-    m[qt] = -INFINITY;
+    m[qt] = kNoKeyYet;
     lsum[qt] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -192,7 +210,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   for (; key0 <= k_hi; key0 += 32) {
     const bool more = key0 + 32 <= k_hi;
     if (more) load_step<DT>(nxt, kv, key0 + 32, k_lo, k_hi);
-    attend_step<DT, NQT>(cur, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step<DT, NQT>(cur, qop, o, m, lsum, key0, k_lo, qpos, window, scale2, pos0);
     if (more) cur = nxt;
   }
 
@@ -213,41 +231,59 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   }
 }
 
-// ------------------------------------------------------------------------------------------ prefill, shared
-// One block per (tile of 16 * NQT queries, key/value head): wave w works on query head g * G + w, and all
-// G waves read the same keys and values, which the block fetches once per step into LDS (next step's
-// loads in flight while the current one is multiplied).  Needs pages of a multiple of 8 tokens.
+// ------------------------------------------------------------------------------------------ prefill, staged
+// One block of four waves per (tile of 16 * NQT queries, head).  The keys are walked in stages of 128
+// that the block copies into LDS; wave w takes keys 32 w .. 32 w + 31 of every stage with a running
+// softmax of its own, and the four waves are merged in LDS at the end.  Against one wave walking all
+// keys this cuts the chain of dependent steps by four, and several blocks per CU hide the copy.
+// The sequence's page numbers are copied to LDS first, so that a fetch is one trip to memory.
+// Needs pages of 8, 16, 32, ... tokens (a power of two).
+constexpr int kStageKeys = 128;
+constexpr int kMaxTableLds = 2048;    // page numbers held in LDS; longer tables are read from memory
+
 template <int DT, int NQT>
-__global__ __launch_bounds__(512) void attention_prefill_shared_kernel(
+__global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_size, int num_pages,
+    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_shift, int num_pages,
     int window, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
-  constexpr int KP = HD + 8;          // key row pitch in LDS (elements): 16 bytes of padding
-  constexpr int VP = 32 + 4;          // value row pitch: 32 keys + 8 bytes of padding
-  constexpr int CHUNKS = 8 * HD;      // 16-byte pieces of one step: 4 HD of keys, 4 HD of values
-  constexpr int MAXC = 8;             // pieces per thread with one wave in the block
-  __shared__ __attribute__((aligned(16))) uint16_t ks[2][32 * KP];
-  __shared__ __attribute__((aligned(16))) uint16_t vs[2][HD * VP];
+  constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
+  constexpr int VP = kStageKeys + 4;          // value row pitch: the stage's keys + 8 bytes of padding
+  constexpr int KCHUNKS = kStageKeys * (HD / 8);      // 16-byte pieces of the stage's keys ...
+  const int page_size = 1 << page_shift, page_mask = page_size - 1;   // pages are a power of two of tokens
+  constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
+  constexpr int PER_THREAD = CHUNKS / 256;
+  constexpr int STAGE_BYTES = (kStageKeys * KP + HD * VP) * 2;
+  constexpr int MERGE_BYTES = 4 * 16 * NQT * (HD + 2) * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
+  __shared__ int32_t s_table[kMaxTableLds];
+  uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* vs = ks + kStageKeys * KP;
 
   const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
-  const int g = blockIdx.y, G = nq / nkv;
+  const int h = blockIdx.y, g = h / (nq / nkv);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
-  const int h = g * G + wave;
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
   const int nvalid = min(16 * NQT, qlen - q_off);
   if (nvalid <= 0) return;
   const int pos0 = ctx - qlen + q_off;
+  const int k_hi = pos0 + nvalid - 1;
+  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
 
-  PagedKV kv;
-  kv.page_size = page_size;
-  kv.num_pages = num_pages;
-  kv.page_stride = size_t(nkv) * page_size * HD;
-  kv.k = k_pool + size_t(g) * page_size * HD;
-  kv.v = v_pool + size_t(g) * page_size * HD;
-  kv.table = block_tables + size_t(seq) * max_blocks;
+  const int32_t* table = block_tables + size_t(seq) * max_blocks;
+  const int first_page = k_lo >> page_shift, n_pages = (k_hi >> page_shift) - first_page + 1;
+  const bool table_in_lds = n_pages <= kMaxTableLds;
+  if (table_in_lds)
+    for (int i = threadIdx.x; i < n_pages; i += 256) s_table[i] = table[first_page + i];
+  auto page_at = [&](int key) {
+    const int page = table_in_lds ? s_table[(key >> page_shift) - first_page] : table[key >> page_shift];
+    return min(max(page, 0), num_pages - 1);
+  };
+  const size_t heads = size_t(nkv);
+  const uint16_t* kbase = k_pool + (size_t(g) << page_shift) * HD;
+  const uint16_t* vbase = v_pool + (size_t(g) << page_shift) * HD;
 
   bf16x8 qop[NQT][HC];
   int qpos[NQT];
@@ -259,93 +295,99 @@ __global__ __launch_bounds__(512) void attention_prefill_shared_kernel(
     const bool valid = row < nvalid;
     qpos[qt] = valid ? pos0 + row : -1;
     load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
-    m[qt] = -INFINITY;
+    m[qt] = kNoKeyYet;
     lsum[qt] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  const int k_hi = pos0 + nvalid - 1;
-  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
-  const int per_thread = (CHUNKS + blockDim.x - 1) / blockDim.x;   // <= MAXC for HD <= 64 ... checked on the host
-
-  uint4 stage[MAXC];
-  auto fetch = [&](int key0) {
+  for (int key0 = (k_lo / kStageKeys) * kStageKeys; key0 <= k_hi; key0 += kStageKeys) {
+    __syncthreads();   // the page numbers are in LDS; the last stage has been used
+    const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
+    uint4 stage[PER_THREAD];
 #pragma unroll
-    for (int u = 0; u < MAXC; ++u) {
-      const int i = threadIdx.x + u * blockDim.x;
-      if (u < per_thread && i < CHUNKS) {
-        if (i < 4 * HD) {                      // keys: row r of the step, dims 8 c .. 8 c + 7
-          const int r = i / (HD / 8), c = i % (HD / 8);
-          const int key = min(max(key0 + r, k_lo), k_hi);
-          stage[u] = ldg128(kv.k + size_t(page_of(kv, key)) * kv.page_stride + size_t(key % page_size) * HD + 8 * c);
-        } else {                               // values: dim d, keys 8 c .. 8 c + 7 of the step
-          const int j = i - 4 * HD, d = j >> 2, c = j & 3;
-          const int kb = min(max(key0 + 8 * c, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
-          stage[u] = ldg128(kv.v + size_t(page_of(kv, kb)) * kv.page_stride + size_t(d) * page_size + kb % page_size);
-        }
+    for (int u = 0; u < PER_THREAD; ++u) {
+      const int i = threadIdx.x + 256 * u;
+      if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
+        const int r = i / (HD / 8), c = i % (HD / 8);
+        int key = key0 + r;
+        if (!interior) key = min(max(key, k_lo), k_hi);
+        stage[u] = ldg128(kbase + (((size_t(page_at(key)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
+      } else {                                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
+        const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
+        int kb = key0 + 8 * c;
+        if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+        stage[u] = ldg128(vbase + ((size_t(page_at(kb)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
       }
     }
-  };
-  auto deposit = [&](int buf) {
 #pragma unroll
-    for (int u = 0; u < MAXC; ++u) {
-      const int i = threadIdx.x + u * blockDim.x;
-      if (u < per_thread && i < CHUNKS) {
-        if (i < 4 * HD) {
-          const int r = i / (HD / 8), c = i % (HD / 8);
-          *reinterpret_cast<uint4*>(&ks[buf][r * KP + 8 * c]) = stage[u];
-        } else {
-          const int j = i - 4 * HD, d = j >> 2, c = j & 3;
-          uint2* dst = reinterpret_cast<uint2*>(&vs[buf][d * VP + 8 * c]);   // rows are 8-byte aligned
-          dst[0] = make_uint2(stage[u].x, stage[u].y);
-          dst[1] = make_uint2(stage[u].z, stage[u].w);
-        }
+    for (int u = 0; u < PER_THREAD; ++u) {
+      const int i = threadIdx.x + 256 * u;
+      if (i < KCHUNKS) {
+        const int r = i / (HD / 8), c = i % (HD / 8);
+        *reinterpret_cast<uint4*>(&ks[r * KP + 8 * c]) = stage[u];
+      } else {
+        const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
+        uint2* dst = reinterpret_cast<uint2*>(&vs[d * VP + 8 * c]);   // rows are 8-byte aligned
+        dst[0] = make_uint2(stage[u].x, stage[u].y);
+        dst[1] = make_uint2(stage[u].z, stage[u].w);
       }
     }
-  };
-
-  int key0 = (k_lo >> 5) << 5;
-  fetch(key0);
-  deposit(0);
-  __syncthreads();
-  int buf = 0;
-  for (; key0 <= k_hi; key0 += 32, buf ^= 1) {
-    const bool more = key0 + 32 <= k_hi;
-    if (more) fetch(key0 + 32);
-    KVStep<DT> r;
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int c = 0; c < HC; ++c) {
-        const int d0 = 32 * c + 8 * lj;
-        r.ka[kt][c] = d0 < HD ? as_bf16x8(*reinterpret_cast<const uint4*>(&ks[buf][(16 * kt + lr) * KP + d0]))
-                              : as_bf16x8(make_uint4(0, 0, 0, 0));
-      }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+    __syncthreads();
+    const int wkey = key0 + 32 * wave;         // this wave's 32 keys of the stage
+    if (wkey <= k_hi && wkey + 32 > k_lo) {
+      KVStep<DT> r;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
-        r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[buf][(16 * dt + lr) * VP + 16 * kt + 4 * lj]);
-    attend_step<DT, NQT>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
-    if (more) deposit(buf ^ 1);
-    __syncthreads();
+#pragma unroll
+        for (int c = 0; c < HC; ++c) {
+          const int d0 = 32 * c + 8 * lj;
+          r.ka[kt][c] = d0 < HD ? as_bf16x8(*reinterpret_cast<const uint4*>(&ks[(32 * wave + 16 * kt + lr) * KP + d0]))
+                                : as_bf16x8(make_uint4(0, 0, 0, 0));
+        }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+          r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[(16 * dt + lr) * VP + 32 * wave + 16 * kt + 4 * lj]);
+      attend_step<DT, NQT>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+    }
   }
 
+  // merge the four waves: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
+  __syncthreads();
+  float* mg = reinterpret_cast<float*>(smem);
+  constexpr int MP = HD + 2;
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     float l = lsum[qt];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    const int row = 16 * qt + lr;
-    if (row >= nvalid) continue;
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD;
+    float* row = mg + (size_t(wave) * 16 * NQT + 16 * qt + lr) * MP;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const floatx4 v = o[qt][dt] * inv;
-      *reinterpret_cast<uint2*>(dst + 16 * dt + 4 * lj) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) row[16 * dt + 4 * lj + r4] = o[qt][dt][r4];
+    if (lj == 0) { row[HD] = m[qt]; row[HD + 1] = l; }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nvalid * (HD / 4); i += 256) {
+    const int row = i / (HD / 4), d = 4 * (i % (HD / 4));
+    float mx = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, mg[(size_t(w) * 16 * NQT + row) * MP + HD]);
+    float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float* src = mg + (size_t(w) * 16 * NQT + row) * MP;
+      const float f = exp2f(src[HD] - mx);
+      den += f * src[HD + 1];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) num[r4] += f * src[d + r4];
     }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD + d;
+    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
   }
 }
 
@@ -383,7 +425,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   int qpos[1] = {lr < G ? pos : -1};
   load_q_operand<DT>(qop[0], lr < G ? q + size_t(q_start[seq]) * q_stride + (g * G + lr) * HD : nullptr);
   floatx4 o[1][DT];
-  float m[1] = {-INFINITY}, lsum[1] = {0.f};
+  float m[1] = {kNoKeyYet}, lsum[1] = {0.f};
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[0][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -399,7 +441,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 #pragma unroll
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i)
-    if (live[i]) attend_step<DT, 1>(steps[i], qop, o, m, lsum, w0 + 32 * i, k_lo, qpos, window, scale2);
+    if (live[i]) attend_step<DT, 1>(steps[i], qop, o, m, lsum, w0 + 32 * i, k_lo, qpos, window, scale2, pos);
   float l = lsum[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -418,7 +460,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     float num = 0.f, den = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float f = s_m[w][qh] == -INFINITY ? 0.f : exp2f(s_m[w][qh] - mx);
+      const float f = exp2f(s_m[w][qh] - mx);
       num += f * s_o[w][qh][d];
       den += f * s_l[w][qh];
     }
@@ -461,7 +503,7 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
     float f = 0.f, l = 0.f;
     if (lane < count) {
       const float ms = part_ml[2 * (base + s0 + lane)];
-      f = ms == -INFINITY ? 0.f : exp2f(ms - mx);
+      f = exp2f(ms - mx);
       l = part_ml[2 * (base + s0 + lane) + 1];
     }
     den += wave_sum(f * l);
@@ -512,12 +554,12 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
   const float scale2 = scale * kLog2e;
   const uint16_t *qp = (const uint16_t*)q, *kp = (const uint16_t*)k_pool, *vp = (const uint16_t*)v_pool;
   if (n_tiles > 0) {
-    const int G = nq / nkv;
-    // the shared kernel stages 8 HD pieces of 16 bytes per step with 64 G threads, at most 8 per thread
-    if (page_size % 8 == 0 && G <= 8 && 8 * HD <= 8 * 64 * G) {
-      attention_prefill_shared_kernel<DT, NQT><<<dim3(n_tiles, nkv), 64 * G, 0, s>>>(
+    if (page_size >= 8 && (page_size & (page_size - 1)) == 0) {
+      int page_shift = 0;
+      while ((1 << page_shift) < page_size) ++page_shift;
+      attention_prefill_staged_kernel<DT, NQT><<<dim3(n_tiles, nq), 256, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
-          page_size, num_pages, window, scale2);
+          page_shift, num_pages, window, scale2);
     } else {
       attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,

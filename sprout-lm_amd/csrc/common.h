@@ -14,12 +14,9 @@ struct bf16_t { uint16_t bits; };
 __device__ __forceinline__ float to_float(float v) { return v; }
 __device__ __forceinline__ float to_float(bf16_t v) { return __uint_as_float(uint32_t(v.bits) << 16); }
 
-// Round to nearest even; NaN stays NaN.
+// Round to nearest even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return uint16_t(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 template <typename T> __device__ __forceinline__ T from_float(float f);
 template <> __device__ __forceinline__ float from_float<float>(float f) { return f; }
