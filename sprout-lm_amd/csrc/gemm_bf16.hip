@@ -180,23 +180,23 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
 }  // namespace sprout
 
 // ------------------------------------------------------------------------------------------------
-// Tiled kernel (T > 64, prefill): both operands go through LDS in steps of 64 along K; 4 waves in a
+// Tiled kernel (T > 64, prefill): both operands go through LDS in steps of 64 or 128 along K; 4 waves in a
 // 2 x 2 arrangement, each computing WM x WN tiles of 32 x 32 on 32x32x16 MFMA with the weights as the
 // A operand (D[n, t]), so that a lane ends with four consecutive n of one token and stores 8 or 16 bytes.
 // The next step is on its way from memory while one is multiplied.  Small accumulating products may be
 // split along K over blockIdx.z (hardware float atomics).
 namespace sprout {
 
-constexpr int TBK = 64;            // depth of one staging step
-constexpr int TPITCH = TBK + 8;    // LDS row pitch in elements: 144 bytes, 16-byte aligned rows
 
-template <int WM, int WN, int MODE, typename TB>
+template <int WM, int WN, int TBK, int MODE, typename TB>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restrict__ x,
                                                          const uint16_t* __restrict__ w,
                                                          const TB* __restrict__ bias, void* __restrict__ out, int T,
                                                          int N, int K, int k_per_split) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int XL = BM * TBK / 8 / 256, WL = BN * TBK / 8 / 256;   // 16-byte loads per thread and operand
+  constexpr int TPITCH = TBK + 8;    // LDS row pitch in elements: rows stay 16-byte aligned, banks shift by 4
+  constexpr int CPR = TBK / 8;       // 16-byte pieces per row of a step
+  constexpr int XL = BM * CPR / 256, WL = BN * CPR / 256;   // 16-byte loads per thread and operand
   __shared__ __attribute__((aligned(16))) uint16_t xs[BM * TPITCH];
   __shared__ __attribute__((aligned(16))) uint16_t ws[BN * TPITCH];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -213,14 +213,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // what this thread copies: rows tid / 8 + 32 i of each operand tile, columns 8 (tid % 8) .. + 7 of a step
-  const int crow = threadIdx.x >> 3, ccol = (threadIdx.x & 7) * 8;
+  // what this thread copies: rows tid / CPR + (256 / CPR) i of each operand tile, columns 8 (tid % CPR) .. + 7
+  constexpr int RSTEP = 256 / CPR;
+  const int crow = threadIdx.x / CPR, ccol = (threadIdx.x % CPR) * 8;
   const uint16_t* xsrc[XL];
   const uint16_t* wsrc[WL];
 #pragma unroll
-  for (int i = 0; i < XL; ++i) xsrc[i] = t0 + crow + 32 * i < T ? x + size_t(t0 + crow + 32 * i) * K + ccol : nullptr;
+  for (int i = 0; i < XL; ++i) xsrc[i] = t0 + crow + RSTEP * i < T ? x + size_t(t0 + crow + RSTEP * i) * K + ccol : nullptr;
 #pragma unroll
-  for (int i = 0; i < WL; ++i) wsrc[i] = n0 + crow + 32 * i < N ? w + size_t(n0 + crow + 32 * i) * K + ccol : nullptr;
+  for (int i = 0; i < WL; ++i) wsrc[i] = n0 + crow + RSTEP * i < N ? w + size_t(n0 + crow + RSTEP * i) * K + ccol : nullptr;
 
   struct Regs { uint4 x[XL]; uint4 w[WL]; };
   auto load_global = [&](Regs& r, int k0) {
@@ -232,9 +233,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   };
   auto store_lds = [&](const Regs& r) {
 #pragma unroll
-    for (int i = 0; i < XL; ++i) *reinterpret_cast<uint4*>(xs + (crow + 32 * i) * TPITCH + ccol) = r.x[i];
+    for (int i = 0; i < XL; ++i) *reinterpret_cast<uint4*>(xs + (crow + RSTEP * i) * TPITCH + ccol) = r.x[i];
 #pragma unroll
-    for (int i = 0; i < WL; ++i) *reinterpret_cast<uint4*>(ws + (crow + 32 * i) * TPITCH + ccol) = r.w[i];
+    for (int i = 0; i < WL; ++i) *reinterpret_cast<uint4*>(ws + (crow + RSTEP * i) * TPITCH + ccol) = r.w[i];
   };
   auto multiply = [&]() {
 #pragma unroll
@@ -312,18 +313,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   }
 }
 
-template <int WM, int WN, typename TB>
-static int launch_tiled(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
-                        int K, int splits) {
+template <int WM, int WN, int TBK, typename TB>
+static int launch_tiled_bk(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T,
+                           int N, int K, int splits) {
   const int k_per_split = ((K + splits - 1) / splits + TBK - 1) / TBK * TBK;
   splits = (K + k_per_split - 1) / k_per_split;
   dim3 grid((N + 64 * WN - 1) / (64 * WN), (T + 64 * WM - 1) / (64 * WM), splits);
   const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
   const TB* bp = (const TB*)bias;
-  if (mode == kStore) gemm_tiled_kernel<WM, WN, kStore, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
-  else if (mode == kAccumulate) gemm_tiled_kernel<WM, WN, kAccumulate, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
-  else gemm_tiled_kernel<WM, WN, kStoreF32, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
+  if (mode == kStore) gemm_tiled_kernel<WM, WN, TBK, kStore, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
+  else if (mode == kAccumulate) gemm_tiled_kernel<WM, WN, TBK, kAccumulate, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
+  else gemm_tiled_kernel<WM, WN, TBK, kStoreF32, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
   return check_launch("sp_gemm (tiled)");
+}
+
+// Long K: steps of 128 halve the number of barriers; only the small tiles have the LDS for it.
+template <int WM, int WN, typename TB>
+static int launch_tiled(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,
+                        int K, int splits) {
+  if (WM * WN <= 2 && K / splits >= 2048) return launch_tiled_bk<WM, WN, 128, TB>(s, x, w, bias, mode, out, T, N, K, splits);
+  return launch_tiled_bk<WM, WN, 64, TB>(s, x, w, bias, mode, out, T, N, K, splits);
 }
 
 // Tile and split choice: large tiles reuse operands better, but the grid must fill 256 CUs several
