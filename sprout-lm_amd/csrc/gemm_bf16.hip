@@ -10,7 +10,7 @@
 
 namespace sprout {
 
-enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2 };
+enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2, kSilu = 3 };   // kSilu: tiled kernel only, see below
 
 template <int TN> struct SkinnyChunk { static constexpr int KC = TN >= 3 ? 448 : 512; };
 
@@ -221,7 +221,19 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 #pragma unroll
   for (int i = 0; i < XL; ++i) xsrc[i] = t0 + crow + RSTEP * i < T ? x + size_t(t0 + crow + RSTEP * i) * K + ccol : nullptr;
 #pragma unroll
-  for (int i = 0; i < WL; ++i) wsrc[i] = n0 + crow + RSTEP * i < N ? w + size_t(n0 + crow + RSTEP * i) * K + ccol : nullptr;
+  for (int i = 0; i < WL; ++i) {
+    const int r = crow + RSTEP * i;          // row of the weight tile in LDS
+    int row = n0 + r;                        // its row in w
+    bool in = row < N;
+    if (MODE == kSilu) {
+      // N counts gate rows; w holds N gate rows, then N up rows.  Tile rows alternate in runs of 32
+      // between gate rows and the matching up rows, so that a lane ends with both of one index.
+      const int gate = blockIdx.x * (BN / 2) + (r / 64) * 32 + (r & 31);
+      in = gate < N;
+      row = ((r >> 5) & 1) ? N + gate : gate;
+    }
+    wsrc[i] = in ? w + size_t(row) * K + ccol : nullptr;
+  }
 
   struct Regs { uint4 x[XL]; uint4 w[WL]; };
   auto load_global = [&](Regs& r, int k0) {
@@ -270,6 +282,33 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
       store_lds(r);
       __syncthreads();
     }
+  }
+
+  if (MODE == kSilu) {
+    // tile column 0 of a wave holds gate rows, column 1 the matching up rows: out[t, n] = silu(gate) * up,
+    // both rounded to bfloat16 first, as where they are stored before the gated product
+    static_assert(MODE != kSilu || WN == 2, "the gated epilogue pairs two tile columns");
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int t = t0 + (wm * WM + i) * 32 + li;
+      if (t >= T) continue;
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int n = blockIdx.x * (BN / 2) + wn * 32 + 8 * rg + 4 * lk;
+        if (n >= N) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float g = to_float(bf16_t{f32_to_bf16_bits(acc[i][0][4 * rg + r])});
+          const float u = to_float(bf16_t{f32_to_bf16_bits(acc[i][WN - 1][4 * rg + r])});
+          v[r] = g / (1.0f + __expf(-g)) * u;
+        }
+        uint16_t* dst = reinterpret_cast<uint16_t*>(out) + size_t(t) * N + n;
+        if (n + 4 <= N && (N & 3) == 0) *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = f32_to_bf16_bits(v[r]);
+      }
+    }
+    return;
   }
 
   // lane holds out[t = tile row li][n = tile column 8 * (r / 4) + 4 * lk + r % 4]: four consecutive n per group
@@ -353,6 +392,14 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
   if (blocks(128, 64) * splits_for(blocks(128, 64)) >= 256)
     return launch_tiled<2, 1, TB>(s, x, w, bias, mode, out, T, N, K, splits_for(blocks(128, 64)));
   return launch_tiled<1, 1, TB>(s, x, w, bias, mode, out, T, N, K, splits_for(blocks(64, 64)));
+}
+
+// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for T > 64: 128-token tiles, 64 gate + 64 up rows per block.
+int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
+  dim3 grid((I + 63) / 64, (T + 127) / 128, 1);
+  gemm_tiled_kernel<2, 2, 64, kSilu, float><<<grid, 256, 0, s>>>((const uint16_t*)x, (const uint16_t*)w, nullptr, out, T, I,
+                                                                 K, (K + 63) / 64 * 64);
+  return check_launch("sp_gate_up_silu (tiled)");
 }
 
 int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,

@@ -317,7 +317,12 @@ extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual
                               float eps, const void* w, int bias_dtype, const void* bias, int mode, void* out, int T,
                               int N, int K);
 
+namespace sprout {
+int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K);
+}
+
 extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
+  if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0;   // the tiled kernel's gated epilogue
   if (!fused_shape_ok(T, K, norm != 0)) return 0;
   if (kind == kEpiRope) return hd % 32 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
   if (kind == kEpiSilu) return N % 32 == 0;
@@ -386,6 +391,7 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
   SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr),
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
+  if (T > 64) return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.out = out;

@@ -50,7 +50,7 @@ class GatedMLP(FeedForward):
     def forward(self, ctx, h, residual):
         T = h.shape[0]
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        if ctx.act_dtype == torch.bfloat16 and T <= 64 and self._fused(T, False):
+        if ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
             ops.gate_up_silu(self.w_gate_up, act, x=h)
         else:
             gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)

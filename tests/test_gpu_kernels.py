@@ -351,8 +351,8 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     assert np.all((kp == 0) | written[:, None, :, None]) and np.all((vp == 0) | written[:, None, :, None])
 
 
-@pytest.mark.parametrize("T", [1, 8, 16, 33, 64])
-@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264)])
+@pytest.mark.parametrize("T", [1, 8, 16, 33, 64, 65, 200, 513])
+@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
