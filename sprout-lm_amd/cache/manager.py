@@ -36,8 +36,12 @@ class StateGroup:
 class SequenceCache:
     """What one request holds: a block table per group, its computed length, a state slot."""
 
+    _next_uid = 0
+
     def __init__(self, manager: "CacheManager", state_slot: int):
         self._manager = manager
+        SequenceCache._next_uid += 1
+        self.uid = SequenceCache._next_uid      # never reused, unlike id(): caches keyed by it stay valid
         self.blocks: list[list[int]] = [[] for _ in manager.groups]
         self.length = 0
         self.state_slot = state_slot

@@ -74,11 +74,12 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 
   // The first weights are requested before anything else: they do not depend on the prologue, and
   // their way from memory is the longest wait of the kernel.
+  constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
   const int steps = (k_end - k_begin + 63) / 64;
-  uint4 wa[4][2][2];
+  uint4 wa[UN][2][2];
   auto load_weights = [&](int s0) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UN; ++u) {
       const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
       const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
 #pragma unroll
@@ -157,12 +158,12 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // this wave's steps of 64 along K: wave, wave + 4, ...; four steps are loaded before they are multiplied
-  for (int s0 = wave; s0 < steps; s0 += 16) {
+  // this wave's steps of 64 along K: wave, wave + 4, ...; UN steps are loaded before they are multiplied
+  for (int s0 = wave; s0 < steps; s0 += 4 * UN) {
     if (s0 != wave) load_weights(s0);
-    uint4 xb[4][TN][2];
+    uint4 xb[UN][TN][2];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < UN; ++u) {
       const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
       const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
 #pragma unroll
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       }
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < UN; ++u)
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll

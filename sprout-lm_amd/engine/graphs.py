@@ -82,35 +82,49 @@ class _DecodeGraph:
                                      device=runner.device)
         self.graph = None
         self.logits = None
+        self._filled = -1          # number of real sequences at the last fill
+        self._rows = [None] * S    # per row: which sequence and how many pages its table row holds
 
     def fill(self, entries, params, counters) -> None:
-        """Write this step's values into the pinned staging buffer."""
+        """Write this step's values into the pinned staging buffer.
+
+        Block-table rows are rewritten only when a row's sequence or its number of pages has changed
+        since the last step (a steady decode batch gains a page every `block_size` steps)."""
         cache, h, n, S = self.runner.cache, self.h, len(entries), self.S
         bs = cache.block_size
         lengths = np.fromiter((e.seq.length for e in entries), dtype=np.int32, count=n)
         h["token_ids"][:n] = [e.tokens[0] for e in entries]
-        h["token_ids"][n:] = 0
         h["positions"][:n] = lengths
-        h["positions"][n:] = 0
         h["ctx_len"][:n] = lengths + 1
-        h["ctx_len"][n:] = 1
         h["state_slots"][:n] = [e.seq.state_slot for e in entries]
-        h["state_slots"][n:] = 0
         h["counter"][:n] = counters
         h["temperature"].view(np.float32)[:n] = [p.temperature for p in params]
-        h["temperature"][n:] = 0
         h["seed"].view(np.int64)[:n] = [p.seed for p in params]
+        if n != self._filled:
+            for name in ("token_ids", "positions", "state_slots", "temperature"):
+                h[name][n:] = 0
+            h["ctx_len"][n:] = 1
+            self._rows = [None] * S
+        last_block = lengths // bs
         for g in range(len(cache.groups)):
             tables = h[f"tables{g}"].reshape(S, self.max_blocks)
             slots = h[f"slots{g}"]
-            slots[n:] = -1
-            tables[n:] = 0
+            if n != self._filled:
+                slots[n:] = -1
+                tables[n:] = 0
+            pages = np.empty(n, dtype=np.int32)
             for i, e in enumerate(entries):
                 blocks = e.seq.blocks[g]
-                nb = min(len(blocks), self.max_blocks)
-                tables[i, :nb] = blocks[:nb]
-                pos = int(lengths[i])
-                slots[i] = blocks[pos // bs] * bs + pos % bs
+                key = (e.seq.uid, g, len(blocks))
+                if self._rows[i] is None or self._rows[i].get(g) != key:
+                    nb = min(len(blocks), self.max_blocks)
+                    tables[i, :nb] = blocks[:nb]
+                    if self._rows[i] is None:
+                        self._rows[i] = {}
+                    self._rows[i][g] = key
+                pages[i] = blocks[last_block[i]]
+            slots[:n] = pages * bs + lengths % bs
+        self._filled = n
 
     def launch(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)

@@ -110,6 +110,28 @@ class ModelRunner:
                 if needed:
                     raise ValueError("Pages for the entry's tokens were not reserved before the step.")
 
+    def validate_decode(self, entries: list[StepEntry]) -> None:
+        """The checks of `validate` for a step of single tokens, in one pass."""
+        seen = set()
+        bs, limit, vocab = self.cache.block_size, self.max_positions, self.vocab_size
+        for e in entries:
+            seq, token = e.seq, e.tokens[0]
+            if id(seq) in seen:
+                raise ValueError("A request appears twice in one step.")
+            seen.add(id(seq))
+            if seq.released:
+                raise ValueError("A request's cache was released before the step.")
+            if not isinstance(token, int) or token < 0 or token >= vocab:
+                raise ValueError(f"Token ids must be integers in [0, {vocab}).")
+            if seq.length >= limit:
+                raise ValueError(f"Position {seq.length} is beyond the model's {limit} positions.")
+            if e.want[0] != 0:
+                raise ValueError("Wanted logit places must index the entry's own tokens.")
+            need = seq.length // bs + 1
+            for blocks in seq.blocks:
+                if len(blocks) < need:
+                    raise ValueError("Pages for the entry's tokens were not reserved before the step.")
+
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Run one batch; returns float32 logits [number of wanted places, vocab] on the device.
 
@@ -134,7 +156,7 @@ class ModelRunner:
                 from .graphs import DecodeGraphs
                 self._graphs = DecodeGraphs(self)
             if self._graphs.usable(entries):
-                self.validate(entries)
+                self.validate_decode(entries)
                 tokens = self._graphs.run(entries, params, counters)
                 if any(t < 0 or t >= self.vocab_size for t in tokens):
                     raise NonFiniteLogits("Non-finite logits: the model produced NaN or infinity.")

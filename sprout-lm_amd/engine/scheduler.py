@@ -142,14 +142,15 @@ class Scheduler:
         self._admit()
         budget = self.options.max_batch_tokens
         planned: dict[str, Work] = {}
-        batch = sorted(self.active.values(), key=lambda r: (self._phase(r) != "decode", r.order))
+        phases = {r.id: self._phase(r) for r in self.active.values()}
+        batch = sorted(self.active.values(), key=lambda r: (phases[r.id] != "decode", r.order))
         for request in batch:
             if budget <= 0:
                 break
             if request.status != "running":
                 continue   # an older request preempted it while this step was planned
             total = request.history_length()
-            phase = self._phase(request)
+            phase = phases[request.id]
             start = request.seq.length
             remaining = total - start - (phase == "recompute")
             count = min(budget, 1 if phase == "decode" else self.options.prefill_chunk_size, remaining)
