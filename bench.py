@@ -43,10 +43,11 @@ def prefill_flops(cfg, T: int) -> float:
     return linear + attention + 2.0 * V * H  # logits of the last position only
 
 
-def make_engine(cfg, dtype, batch, context, layers_note):
+def make_engine(cfg, dtype, batch, context, prefill_tokens):
     from sprout_lm_amd.engine import Engine
     pages_per_request = -(-context // 16)
-    return Engine.from_config(cfg, seed=0, dtype=dtype, block_size=16, num_blocks=batch * (pages_per_request + 1),
+    pages = max(batch * (pages_per_request + 1), -(-prefill_tokens // 16) + 1)
+    return Engine.from_config(cfg, seed=0, dtype=dtype, block_size=16, num_blocks=pages,
                               max_sequences=batch, max_batch_tokens=max(2048, batch), prefill_chunk_size=2048,
                               prefix_caching=False, record_trace=False)
 
@@ -128,7 +129,7 @@ def main() -> int:
     element = 2 if args.dtype == "bf16" else 4
 
     biggest = max(args.batch, 1 if args.no_points else 64)
-    engine = make_engine(cfg, dtype, biggest, args.context, None)
+    engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
     warmup = max(args.warmup, 1)
 
     step_s = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
@@ -144,7 +145,8 @@ def main() -> int:
     flops = prefill_flops(cfg, args.prefill_tokens)
     value = args.batch / step_s
     line = {
-        "metric": "decode tok/s at batch 8 (Qwen2.5-0.5B sizes, context 4096); prefill tok/s at 2,048 tokens; % roofline",
+        "metric": f"decode tok/s at batch {args.batch} ({args.preset} sizes, context {args.context}); "
+                  f"prefill tok/s at {args.prefill_tokens:,} tokens; % roofline",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": warmup,
         "ms_per_step": round(step_s * 1000, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",

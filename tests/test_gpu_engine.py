@@ -144,3 +144,69 @@ def test_first_tokens_and_long_decoding(folders):
             assert np.abs(got - want[p]).max() <= H.tolerance(dtype, want[p]), f"{dtype} position {p}"
         print(f"long decode {dtype}: worst {worst:.3e}")
         seq.release()
+
+
+def test_graph_replays_equal_eager_steps(folders):
+    """Decode steps replayed from a recorded graph give the tokens of eagerly launched steps, replay after
+    replay, with eager prompt steps and synchronisations in between (requests arrive while others decode)."""
+    from sprout_lm_amd.engine import Engine
+    name = "A"
+    vocab = H.CONFIGS[name]["vocab_size"]
+    prompts = [H.random_tokens(vocab, n, 60 + i) for i, n in enumerate((7, 21, 3, 40, 12))]
+
+    def run(use_graphs):
+        engine = Engine.from_folder(folders[name], "bfloat16", block_size=16, num_blocks=48, max_sequences=4,
+                                    max_batch_tokens=32, prefill_chunk_size=16)
+        engine.model.use_graphs = use_graphs
+        engine.add("r0", prompts[0], 30, ignore_eos=True)
+        engine.add("r1", prompts[1], 25, ignore_eos=True)
+        steps = 0
+        while engine.pending:
+            steps += 1
+            if steps == 6:
+                engine.add("r2", prompts[2], 20, temperature=0.8, seed=5, ignore_eos=True)
+            if steps == 15:
+                engine.add("r3", prompts[3], 10, ignore_eos=True)
+                engine.add("r4", prompts[4], 28, temperature=1.2, seed=9, ignore_eos=True)
+            engine.step()
+        replays = engine.model._graphs.replays if engine.model._graphs else 0
+        return [engine.result(f"r{i}")["output"] for i in range(5)], replays
+
+    eager, none = run(False)
+    graphed, replays = run(True)
+    assert none == 0 and replays > 40
+    assert graphed == eager
+
+
+def test_real_layer_sizes_both_dtypes(tmp_path):
+    """Two layers with the sizes of Qwen2.5-0.5B (hidden 896, 14 heads in 2 groups of head size 64, inner 4864,
+    vocabulary 151936, tied): whole prompt, portions and single tokens against the plain implementation."""
+    import torch
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    raw = dict(PRESETS["qwen2.5-0.5b"], num_hidden_layers=2)
+    folder = str(tmp_path / "half_b")
+    write_model_folder(folder, S.config_from_dict(raw), seed=8, dtype=torch.bfloat16, std=0.02)
+    tokens = H.random_tokens(raw["vocab_size"], 83, 17)
+    for dtype in ("float32", "bfloat16"):
+        want = H.plain_logits(folder, dtype, tokens)
+        runner = ModelRunner.from_folder(folder, dtype, block_size=16, num_blocks=16, max_sequences=2)
+        seq = runner.cache.create()
+        rows = {}
+        fed = 0
+        for n in (40, 17, 2, 1, 1, 16, 1, 1, 1, 1, 1, 1):
+            assert runner.cache.reserve(seq, fed + n)
+            got = runner.step([StepEntry(seq, tokens[fed:fed + n], [0, n - 1] if n > 1 else [0])]).cpu().numpy()
+            rows[fed] = got[0]
+            rows[fed + n - 1] = got[-1]
+            fed += n
+        assert fed == len(tokens)
+        for pos, row in rows.items():
+            err = np.abs(row - want[pos])
+            if dtype == "float32":   # the reference's bound for real checkpoints (test/model.integration.ts:69)
+                assert np.all(err <= 1e-3 + 1e-4 * np.abs(want[pos])), f"position {pos}: {err.max():.3e}"
+            else:
+                assert err.max() <= H.tolerance(dtype, want[pos]), f"position {pos}: {err.max():.3e}"
+        seq.release()
