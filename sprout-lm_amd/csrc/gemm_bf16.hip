@@ -197,8 +197,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   constexpr int TPITCH = TBK + 8;    // LDS row pitch in elements: rows stay 16-byte aligned, banks shift by 4
   constexpr int CPR = TBK / 8;       // 16-byte pieces per row of a step
   constexpr int XL = BM * CPR / 256, WL = BN * CPR / 256;   // 16-byte loads per thread and operand
-  __shared__ __attribute__((aligned(16))) uint16_t xs[BM * TPITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t ws[BN * TPITCH];
+  // two buffers of (activation tile, weight tile): one is multiplied while the other is filled
+  extern __shared__ __attribute__((aligned(16))) uint16_t tiles_lds[];
+  constexpr int BUF = (BM + BN) * TPITCH;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave >> 1, wn = wave & 1;
   const int li = lane & 31, lk = lane >> 5;
@@ -243,13 +244,17 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
 #pragma unroll
     for (int i = 0; i < WL; ++i) r.w[i] = (wsrc[i] && kin) ? ldg128(wsrc[i] + k0) : make_uint4(0, 0, 0, 0);
   };
-  auto store_lds = [&](const Regs& r) {
+  auto store_lds = [&](const Regs& r, int buf) {
+    uint16_t* xs = tiles_lds + buf * BUF;
+    uint16_t* ws = xs + BM * TPITCH;
 #pragma unroll
     for (int i = 0; i < XL; ++i) *reinterpret_cast<uint4*>(xs + (crow + RSTEP * i) * TPITCH + ccol) = r.x[i];
 #pragma unroll
     for (int i = 0; i < WL; ++i) *reinterpret_cast<uint4*>(ws + (crow + RSTEP * i) * TPITCH + ccol) = r.w[i];
   };
-  auto multiply = [&]() {
+  auto multiply = [&](int buf) {
+    const uint16_t* xs = tiles_lds + buf * BUF;
+    const uint16_t* ws = xs + BM * TPITCH;
 #pragma unroll
     for (int ks = 0; ks < TBK / 16; ++ks) {
       bf16x8 a[WM], b[WN];
@@ -266,22 +271,20 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     }
   };
 
-  // the next step's loads are in flight while the current one is multiplied; several blocks per CU
-  // cover what remains of the latency (a second set of staging registers cost more in occupancy
-  // than it hid: measured 93 us against 74 us on a 2048 x 9728 x 896 product)
+  // The next step's loads are in flight while the current one is multiplied, and go into the other
+  // LDS buffer afterwards: one barrier per step.  (A second set of staging registers, to have two
+  // steps in flight, cost more in occupancy than it hid: 93 us against 74 us on 2048 x 9728 x 896.)
   Regs r;
   load_global(r, k_begin);
-  store_lds(r);
+  store_lds(r, 0);
   __syncthreads();
-  for (int k0 = k_begin; k0 < k_end; k0 += TBK) {
+  int buf = 0;
+  for (int k0 = k_begin; k0 < k_end; k0 += TBK, buf ^= 1) {
     const bool more = k0 + TBK < k_end;
     if (more) load_global(r, k0 + TBK);
-    multiply();
+    multiply(buf);
+    if (more) store_lds(r, buf ^ 1);
     __syncthreads();
-    if (more) {
-      store_lds(r);
-      __syncthreads();
-    }
   }
 
   if (MODE == kSilu) {
@@ -352,6 +355,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
   }
 }
 
+template <int WM, int WN, int TBK, int MODE, typename TB>
+static int launch_tiled_mode(hipStream_t s, dim3 grid, const uint16_t* x, const uint16_t* w, const TB* bias, void* out,
+                             int T, int N, int K, int k_per_split) {
+  constexpr size_t lds = size_t(2) * 64 * (WM + WN) * (TBK + 8) * sizeof(uint16_t);
+  static bool raised = false;
+  if (lds > 48 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_tiled_kernel<WM, WN, TBK, MODE, TB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (e != hipSuccess) {
+      set_error("sp_gemm (tiled): cannot raise the LDS limit: %s", hipGetErrorString(e));
+      return 1;
+    }
+    raised = true;
+  }
+  gemm_tiled_kernel<WM, WN, TBK, MODE, TB><<<grid, 256, lds, s>>>(x, w, bias, out, T, N, K, k_per_split);
+  return check_launch("sp_gemm (tiled)");
+}
+
 template <int WM, int WN, int TBK, typename TB>
 static int launch_tiled_bk(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T,
                            int N, int K, int splits) {
@@ -360,10 +381,9 @@ static int launch_tiled_bk(hipStream_t s, const void* x, const void* w, const vo
   dim3 grid((N + 64 * WN - 1) / (64 * WN), (T + 64 * WM - 1) / (64 * WM), splits);
   const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
   const TB* bp = (const TB*)bias;
-  if (mode == kStore) gemm_tiled_kernel<WM, WN, TBK, kStore, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
-  else if (mode == kAccumulate) gemm_tiled_kernel<WM, WN, TBK, kAccumulate, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
-  else gemm_tiled_kernel<WM, WN, TBK, kStoreF32, TB><<<grid, 256, 0, s>>>(xp, wp, bp, out, T, N, K, k_per_split);
-  return check_launch("sp_gemm (tiled)");
+  if (mode == kStore) return launch_tiled_mode<WM, WN, TBK, kStore, TB>(s, grid, xp, wp, bp, out, T, N, K, k_per_split);
+  if (mode == kAccumulate) return launch_tiled_mode<WM, WN, TBK, kAccumulate, TB>(s, grid, xp, wp, bp, out, T, N, K, k_per_split);
+  return launch_tiled_mode<WM, WN, TBK, kStoreF32, TB>(s, grid, xp, wp, bp, out, T, N, K, k_per_split);
 }
 
 // Long K: steps of 128 halve the number of barriers; only the small tiles have the LDS for it.
@@ -397,9 +417,8 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
 // out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for T > 64: 128-token tiles, 64 gate + 64 up rows per block.
 int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
   dim3 grid((I + 63) / 64, (T + 127) / 128, 1);
-  gemm_tiled_kernel<2, 2, 64, kSilu, float><<<grid, 256, 0, s>>>((const uint16_t*)x, (const uint16_t*)w, nullptr, out, T, I,
-                                                                 K, (K + 63) / 64 * 64);
-  return check_launch("sp_gate_up_silu (tiled)");
+  return launch_tiled_mode<2, 2, 64, kSilu, float>(s, grid, (const uint16_t*)x, (const uint16_t*)w, nullptr, out, T, I, K,
+                                                    (K + 63) / 64 * 64);
 }
 
 int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
