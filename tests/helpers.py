@@ -39,7 +39,7 @@ def make_model_folder(root: str, name: str, storage=torch.bfloat16) -> str:
     """A model folder of tiny configuration `name`, written by the engine's random-weights mode."""
     import sprout_lm_amd as S
     from sprout_lm_amd.weights import write_model_folder
-    folder = os.path.join(root, f"tiny_{name}")
+    folder = os.path.join(root, f"tiny_{name}_{str(storage).split('.')[-1]}")
     if not os.path.exists(os.path.join(folder, "model.safetensors")):
         cfg = S.config_from_dict(CONFIGS[name])
         write_model_folder(folder, cfg, SEEDS[name], dtype=storage, std=WEIGHT_STD)

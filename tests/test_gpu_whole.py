@@ -69,3 +69,23 @@ def test_reference_fixture_logits_fp32(reference_fixture):
                 logits = runner.step([StepEntry(seq, [case["output"][step]], [0])]).cpu().numpy()[0]
         seq.release()
         assert runner.cache.free_pages() == [12]
+
+
+def test_checkpoint_stored_in_32_bit_computed_in_bfloat16(tmp_path):
+    """A tensor stored in 32-bit stays so: bfloat16 activations meet float32 weights (no rounding of the weights)."""
+    import torch
+    from sprout_lm_amd.engine import StepEntry
+    from tests.plain import qwen2_plain as P
+    folder = H.make_model_folder(str(tmp_path), "B", storage=torch.float32)
+    runner = make_runner(folder, "B", "bfloat16")
+    assert runner.parts.blocks[0].mixer.w_qkv.dtype == torch.float32
+    cfg, w = P.load_folder(folder, "float32")              # the plain side keeps the float32 values too
+    tokens = H.random_tokens(384, 45, 12)
+    want = P.forward_logits(w, cfg, tokens, store=P.bf16_round)
+    seq = runner.cache.create()
+    assert runner.cache.reserve(seq, 45)
+    got = runner.step([StepEntry(seq, tokens[:30], list(range(30)))]).cpu().numpy()
+    got = np.concatenate([got, runner.step([StepEntry(seq, tokens[30:], list(range(15)))]).cpu().numpy()])
+    assert np.abs(got - want).max() <= H.tolerance("bfloat16", want)
+    rounded = P.forward_logits(P.load_folder(folder, "bfloat16")[1], cfg, tokens, store=P.bf16_round)
+    assert np.abs(got - want).max() < np.abs(got - rounded).max()    # closer to the unrounded weights
