@@ -262,7 +262,9 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
   uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
   uint16_t* vs = ks + kStageKeys * KP;
 
-  const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
+  // tiles are listed in order of position; the last ones walk the most keys, so they start first
+  const int tile = gridDim.x - 1 - blockIdx.x;
+  const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
   const int h = blockIdx.y, g = h / (nq / nkv);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
