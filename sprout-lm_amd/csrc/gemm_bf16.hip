@@ -5,12 +5,11 @@
 // instruction), the few activations wait in LDS, and the product runs on 16x16x32 MFMA with the
 // weights as the A operand: D[n, t].  Small matrices are cut along K over several blocks, whose
 // partial sums are added into the float32 output with hardware atomics (accumulate mode only).
-#include "mfma.h"
+#include "gemm_epilogue.h"
 #include "sprout_hip.h"
 
 namespace sprout {
 
-enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2, kSilu = 3 };   // kSilu: tiled kernel only, see below
 
 template <int TN> struct SkinnyChunk { static constexpr int KC = TN >= 3 ? 448 : 512; };
 
@@ -158,6 +157,10 @@ int gemm_bf16_tiled(hipStream_t s, const void* a, const void* w, int bias_dtype,
                     int T, int N, int K);
 int gemm_decode_plain(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, int mode, void* out,
                       int T, int N, int K);
+bool gemm_pipe_takes(int T, int N, int K);
+int gemm_bf16_pipe(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                   int T, int N, int K);
+int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K);
 
 // mode 0 stores bfloat16 here; a float32 store of mode 0 is passed in as mode 2 by the caller.
 int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, int out_dtype,
@@ -166,14 +169,17 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
   if (K % 8 != 0) return 0;                               // rows of w must start on 16-byte boundaries
   if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) & 15) return 0;
   if (mode == kStore && out_dtype == kF32) mode = kStoreF32;
+  *handled = true;
   if (T <= 64) {
-    *handled = true;
-    // few rows: split K between the waves of a block (and between blocks when accumulating)
+    // Few rows.  Large accumulating products stream their weights through the pipelined tiles (K split over
+    // blocks); the others split K between the waves of a block, or, when very wide, stream rows per wave.
+    if (T > 16 && mode == kAccumulate && size_t(N) * K >= (size_t(6) << 20) && gemm_pipe_takes(T, N, K))
+      return gemm_bf16_pipe(s, a, w, bias_dtype, bias, mode, out, T, N, K);
     if ((N + 15) / 16 < 2048) return gemm_decode_plain(s, a, w, bias_dtype, bias, mode, out, T, N, K);
     if (bias && bias_dtype == kBF16) return skinny_shape<bf16_t>(s, a, w, bias, mode, out, T, N, K);
     return skinny_shape<float>(s, a, w, bias, mode, out, T, N, K);
   }
-  *handled = true;
+  if (gemm_pipe_takes(T, N, K)) return gemm_bf16_pipe(s, a, w, bias_dtype, bias, mode, out, T, N, K);
   return gemm_bf16_tiled(s, a, w, bias_dtype, bias, mode, out, T, N, K);
 }
 
@@ -287,72 +293,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const uint16_t* __restr
     __syncthreads();
   }
 
-  if (MODE == kSilu) {
-    // tile column 0 of a wave holds gate rows, column 1 the matching up rows: out[t, n] = silu(gate) * up,
-    // both rounded to bfloat16 first, as where they are stored before the gated product
-    static_assert(MODE != kSilu || WN == 2, "the gated epilogue pairs two tile columns");
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-      const int t = t0 + (wm * WM + i) * 32 + li;
-      if (t >= T) continue;
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int n = blockIdx.x * (BN / 2) + wn * 32 + 8 * rg + 4 * lk;
-        if (n >= N) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float g = to_float(bf16_t{f32_to_bf16_bits(acc[i][0][4 * rg + r])});
-          const float u = to_float(bf16_t{f32_to_bf16_bits(acc[i][WN - 1][4 * rg + r])});
-          v[r] = g / (1.0f + __expf(-g)) * u;
-        }
-        uint16_t* dst = reinterpret_cast<uint16_t*>(out) + size_t(t) * N + n;
-        if (n + 4 <= N && (N & 3) == 0) *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-        else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = f32_to_bf16_bits(v[r]);
-      }
-    }
-    return;
-  }
-
-  // lane holds out[t = tile row li][n = tile column 8 * (r / 4) + 4 * lk + r % 4]: four consecutive n per group
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    const int t = t0 + (wm * WM + i) * 32 + li;
-    if (t >= T) continue;
-#pragma unroll
-    for (int j = 0; j < WN; ++j) {
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int n = n0 + (wn * WN + j) * 32 + 8 * rg + 4 * lk;
-        if (n >= N) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          v[r] = acc[i][j][4 * rg + r] + ((bias && blockIdx.z == 0 && n + r < N) ? to_float(bias[n + r]) : 0.f);
-        const size_t o = size_t(t) * N + n;
-        const bool whole = n + 4 <= N && (N & 3) == 0;
-        if (MODE == kStore) {
-          uint16_t* dst = reinterpret_cast<uint16_t*>(out) + o;
-          if (whole) *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-          else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = f32_to_bf16_bits(v[r]);
-        } else if (MODE == kStoreF32) {
-          float* dst = reinterpret_cast<float*>(out) + o;
-          if (whole) *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-          else for (int r = 0; r < 4 && n + r < N; ++r) dst[r] = v[r];
-        } else {
-          float* dst = reinterpret_cast<float*>(out) + o;
-          if (gridDim.z > 1) {
-            for (int r = 0; r < 4 && n + r < N; ++r) unsafeAtomicAdd(dst + r, v[r]);
-          } else if (whole) {
-            const float4 old = *reinterpret_cast<float4*>(dst);
-            *reinterpret_cast<float4*>(dst) = make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
-          } else {
-            for (int r = 0; r < 4 && n + r < N; ++r) dst[r] += v[r];
-          }
-        }
-      }
-    }
-  }
+  static_assert(4 * 32 * (32 * WN + 4) * sizeof(float) <= 2 * BUF * sizeof(uint16_t), "the turning buffer must fit");
+  tile_epilogue<WM, WN, MODE, TB>(acc, reinterpret_cast<float*>(tiles_lds), bias, out, T, N, t0, n0);
 }
 
 template <int WM, int WN, int TBK, int MODE, typename TB>
@@ -403,7 +345,7 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
   // Splitting K pays only while the atomics stay few: T * N * splits float atomics cost more than
   // the product itself once T is in the thousands (measured 352 us against 44 us at 2048 x 896 x 4864).
   auto splits_for = [&](int nblocks) {
-    if (mode != kAccumulate || size_t(T) * N > (size_t(1) << 18)) return 1;
+    if (mode != kAccumulate || size_t(T) * N > (size_t(1) << 20)) return 1;
     return max(1, min((768 + nblocks - 1) / nblocks, K / 512));
   };
   if (blocks(256, 128) >= 2048) return launch_tiled<4, 2, TB>(s, x, w, bias, mode, out, T, N, K, 1);
@@ -416,6 +358,7 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
 
 // out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for T > 64: 128-token tiles, 64 gate + 64 up rows per block.
 int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
+  if (gemm_pipe_takes(T, 2 * I, K)) return gemm_bf16_pipe_silu(s, x, w, out, T, I, K);
   dim3 grid((I + 63) / 64, (T + 127) / 128, 1);
   return launch_tiled_mode<2, 2, 64, kSilu, float>(s, grid, (const uint16_t*)x, (const uint16_t*)w, nullptr, out, T, I, K,
                                                     (K + 63) / 64 * 64);

@@ -320,6 +320,7 @@ extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual
 
 namespace sprout {
 int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K);
+bool gemm_pipe_takes(int T, int N, int K);
 }
 
 extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
@@ -392,7 +393,9 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
   SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr),
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
-  if (T > 64) return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K);
+  // many tokens, or a few with whole steps of 64 along K: the tiled kernels stream the weights better
+  if (T > 64 || (T > 16 && !residual && gemm_pipe_takes(T, 2 * I, K)))
+    return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.out = out;

@@ -19,7 +19,9 @@ def bf16(x):
 
 @pytest.mark.parametrize("T,N,K", [(1, 1, 1), (1, 37, 33), (3, 130, 31), (5, 64, 1025), (17, 151, 96), (64, 100, 70),
                                    (77, 300, 129), (200, 96, 224), (130, 257, 511), (129, 257, 200), (300, 331, 240),
-                                   (513, 1152, 896), (2, 896, 4864), (40, 640, 1000), (64, 151, 72), (1000, 130, 136)])
+                                   (513, 1152, 896), (2, 896, 4864), (40, 640, 1000), (64, 151, 72), (1000, 130, 136),
+                                   (130, 257, 64), (200, 96, 192), (129, 300, 1024), (1000, 130, 128), (300, 331, 320),
+                                   (700, 896, 4864), (65, 2100, 448)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
@@ -314,8 +316,7 @@ def _normed(res, w, eps):
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     from sprout_lm_amd import ops
-    if not ops.fused_supported(ops.FUSED_ROPE, T, (nq + 2 * nkv) * hd, K, hd, hd, norm):
-        pytest.skip("shape not taken by the fused kernel")
+    taken = ops.fused_supported(ops.FUSED_ROPE, T, (nq + 2 * nkv) * hd, K, hd, hd, norm)
     rng = np.random.default_rng(T * 7 + hd)
     N, pages, theta, eps = (nq + 2 * nkv) * hd, 40, 10000.0, 1e-5
     w = bf16(rng.standard_normal((N, K)) / math.sqrt(K))
@@ -332,8 +333,13 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     vp = torch.zeros(pages, nkv, hd, page, dtype=torch.bfloat16, device=DEV)
     q_out = torch.full((T, nq * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
     args = dict(residual=t(res), norm_weight=t(nw, torch.bfloat16), eps=eps) if norm else dict(x=t(x, torch.bfloat16))
-    ops.qkv_rope_cache(t(w, torch.bfloat16), t(b, torch.bfloat16), q_out, t(pos, torch.int32), inv, hd, t(slots, torch.int32),
-                       kp, vp, nq, nkv, hd, **args)
+    call = lambda: ops.qkv_rope_cache(t(w, torch.bfloat16), t(b, torch.bfloat16), q_out, t(pos, torch.int32), inv, hd,
+                                      t(slots, torch.int32), kp, vp, nq, nkv, hd, **args)
+    if not taken:       # a shape the kernel does not take is refused, never computed wrongly
+        with pytest.raises(ops.KernelError):
+            call()
+        return
+    call()
     qkv = bf16(x.astype(np.float64) @ w.astype(np.float64).T + b)
     want = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, hd, theta)
     got_q = q_out.float().cpu().numpy()
@@ -356,8 +362,7 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
-    if not ops.fused_supported(ops.FUSED_SILU, T, 2 * I, K, norm=norm):
-        pytest.skip("shape not taken by the fused kernel")
+    taken = ops.fused_supported(ops.FUSED_SILU, T, 2 * I, K, norm=norm)
     rng = np.random.default_rng(T + I)
     eps = 1e-6
     w = bf16(rng.standard_normal((2 * I, K)) / math.sqrt(K) * 2)
@@ -366,6 +371,10 @@ def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     x = _normed(res, nw, eps) if norm else bf16(res)
     args = dict(residual=t(res), norm_weight=t(nw), eps=eps) if norm else dict(x=t(x, torch.bfloat16))
     out = torch.empty(T, I, dtype=torch.bfloat16, device=DEV)
+    if not taken:
+        with pytest.raises(ops.KernelError):
+            ops.gate_up_silu(t(w, torch.bfloat16), out, **args)
+        return
     ops.gate_up_silu(t(w, torch.bfloat16), out, **args)
     gu = bf16(x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float64)
     g, u = gu[:, :I], gu[:, I:]
