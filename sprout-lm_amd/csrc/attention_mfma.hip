@@ -14,6 +14,8 @@
 // the block that finishes last do the merge needs a device-wide fence in every block, whose cache
 // write-back cost more than the second launch: measured 2.0 ms against 1.4 ms per step.)
 // Keys are always cut at the same places, so a position's result does not depend on the batch.
+#include <type_traits>
+
 #include "mfma.h"
 #include "sprout_hip.h"
 
@@ -72,6 +74,24 @@ __device__ __forceinline__ void load_step(KVStep<DT>& r, const PagedKV& kv, int 
 }
 
 constexpr float kNoKeyYet = -1.0e30f;   // running maximum before any key: finite, so that no inf - inf arises
+// The running maximum of a row follows the true maximum only when that has grown by more than this (in
+// log2 units): until then the probabilities are taken against the older maximum and are at most 2^8, which
+// float32 sums and bfloat16 operands hold as exactly as values below 1, and the accumulators are not rescaled.
+constexpr float kRescaleStep = 8.0f;
+
+// max(a, b) as the median of (a, b, +inf): one instruction, where fmaxf of an MFMA result costs a
+// canonicalising self-maximum more.  (Not inline assembly: the compiler must see who reads MFMA and
+// lane-swap results, to keep the wait states those need.)
+__device__ __forceinline__ float vmax(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
+__device__ __forceinline__ float vmax3(float a, float b, float c) { return vmax(vmax(a, b), c); }
+// Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48, in the vector unit (no trip through LDS).
+__device__ __forceinline__ float max_over_quarters(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto h = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const unsigned v = __float_as_uint(vmax(__uint_as_float(h[0]), __uint_as_float(h[1])));
+  const auto f = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return vmax(__uint_as_float(f[0]), __uint_as_float(f[1]));
+}
 
 // Scores, running softmax and P.V of one loaded step for NQT tiles of 16 rows.
 // qpos[qt]: position of this lane's row (column l % 16 of tile qt), or -1 for a row that does not exist.
@@ -99,22 +119,33 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     if (MASKED) {
+      // visible keys of this lane's row: lo .. lo + span (none when span < 0), tested with one unsigned compare
+      const int hi = qpos[qt];
+      const int lo = window > 0 ? max(k_lo, hi - window + 1) : k_lo;
+      const int span = hi - lo;
+      const unsigned limit = span >= 0 ? unsigned(span) : 0u;
+      const int base = span >= 0 ? lo : key0 + 64;          // key - base < 0 for every key of the step: none passes
+      const int first = key0 + 4 * lj - base;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const int key = key0 + 16 * kt + 4 * lj + r4;
-          const bool visible = key <= qpos[qt] && key >= k_lo && (window <= 0 || qpos[qt] - key < window);
-          if (!visible) s[qt][kt][r4] = -INFINITY;
-        }
+        for (int r4 = 0; r4 < 4; ++r4)
+          s[qt][kt][r4] = unsigned(first + 16 * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
     }
-    float raw = fmaxf(fmaxf(fmaxf(s[qt][0][0], s[qt][0][1]), fmaxf(s[qt][0][2], s[qt][0][3])),
-                      fmaxf(fmaxf(s[qt][1][0], s[qt][1][1]), fmaxf(s[qt][1][2], s[qt][1][3])));
-    raw = fmaxf(raw, __shfl_xor(raw, 16, 64));
-    raw = fmaxf(raw, __shfl_xor(raw, 32, 64));
-    const float mx = fmaxf(m[qt], raw * scale2);            // finite: m starts finite
-    const float alpha = __builtin_amdgcn_exp2f(m[qt] - mx);
-    m[qt] = mx;
+    float raw = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
+    raw = vmax3(raw, s[qt][0][3], s[qt][1][0]);
+    raw = vmax3(raw, s[qt][1][1], s[qt][1][2]);
+    raw = max_over_quarters(vmax(raw, s[qt][1][3]));
+    const float top = raw * scale2;                          // -inf when the row sees no key of the step
+    if (__builtin_amdgcn_ballot_w64(top > m[qt] + kRescaleStep) != 0) {
+      const float mx = top > m[qt] + kRescaleStep ? top : m[qt];   // finite: m starts finite
+      const float alpha = __builtin_amdgcn_exp2f(m[qt] - mx);
+      m[qt] = mx;
+      lsum[qt] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha;
+    }
+    const float mx = m[qt];
     float p[2][4], sum = 0.f;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
@@ -123,15 +154,13 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
         p[kt][r4] = __builtin_amdgcn_exp2f(fmaf(s[qt][kt][r4], scale2, -mx));   // exp2(-inf) = 0 for masked keys
         sum += p[kt][r4];
       }
-    lsum[qt] = fmaf(lsum[qt], alpha, sum);
+    lsum[qt] += sum;
     const uint4 pb = make_uint4(pack_bf16x2(p[0][0], p[0][1]), pack_bf16x2(p[0][2], p[0][3]),
                                 pack_bf16x2(p[1][0], p[1][1]), pack_bf16x2(p[1][2], p[1][3]));
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      floatx4 acc = o[qt][dt];
-      acc *= alpha;
       const uint4 a = make_uint4(r.va[dt][0].x, r.va[dt][0].y, r.va[dt][1].x, r.va[dt][1].y);
-      o[qt][dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+      o[qt][dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), o[qt][dt]);
     }
   }
 }
@@ -250,7 +279,7 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     int window, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
-  constexpr int VP = kStageKeys + 4;          // value row pitch: the stage's keys + 8 bytes of padding
+  constexpr int VP = kStageKeys + 8;          // value row pitch: the stage's keys + 16 bytes of padding
   constexpr int KCHUNKS = kStageKeys * (HD / 8);      // 16-byte pieces of the stage's keys ...
   const int page_size = 1 << page_shift, page_mask = page_size - 1;   // pages are a power of two of tokens
   constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
@@ -279,8 +308,12 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
   const bool table_in_lds = n_pages <= kMaxTableLds;
   if (table_in_lds)
     for (int i = threadIdx.x; i < n_pages; i += 256) s_table[i] = table[first_page + i];
-  auto page_at = [&](int key) {
-    const int page = table_in_lds ? s_table[(key >> page_shift) - first_page] : table[key >> page_shift];
+  // where the page numbers are read from is a compile-time choice of the caller (a run-time choice
+  // between LDS and memory would turn every read into a flat load)
+  auto page_at = [&](int key, auto in_lds) {
+    int page;
+    if constexpr (decltype(in_lds)::value) page = s_table[(key >> page_shift) - first_page];
+    else page = table[key >> page_shift];
     return min(max(page, 0), num_pages - 1);
   };
   const size_t heads = size_t(nkv);
@@ -307,21 +340,25 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     __syncthreads();   // the page numbers are in LDS; the last stage has been used
     const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
     uint4 stage[PER_THREAD];
+    auto fetch = [&](auto in_lds) {
 #pragma unroll
-    for (int u = 0; u < PER_THREAD; ++u) {
-      const int i = threadIdx.x + 256 * u;
-      if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
-        const int r = i / (HD / 8), c = i % (HD / 8);
-        int key = key0 + r;
-        if (!interior) key = min(max(key, k_lo), k_hi);
-        stage[u] = ldg128(kbase + (((size_t(page_at(key)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
-      } else {                                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
-        const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
-        int kb = key0 + 8 * c;
-        if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
-        stage[u] = ldg128(vbase + ((size_t(page_at(kb)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
+      for (int u = 0; u < PER_THREAD; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
+          const int r = i / (HD / 8), c = i % (HD / 8);
+          int key = key0 + r;
+          if (!interior) key = min(max(key, k_lo), k_hi);
+          stage[u] = ldg128(kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
+        } else {                                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
+          const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
+          int kb = key0 + 8 * c;
+          if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+          stage[u] = ldg128(vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
+        }
       }
-    }
+    };
+    if (table_in_lds) fetch(std::true_type{});
+    else fetch(std::false_type{});
 #pragma unroll
     for (int u = 0; u < PER_THREAD; ++u) {
       const int i = threadIdx.x + 256 * u;
@@ -330,9 +367,7 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
         *reinterpret_cast<uint4*>(&ks[r * KP + 8 * c]) = stage[u];
       } else {
         const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
-        uint2* dst = reinterpret_cast<uint2*>(&vs[d * VP + 8 * c]);   // rows are 8-byte aligned
-        dst[0] = make_uint2(stage[u].x, stage[u].y);
-        dst[1] = make_uint2(stage[u].z, stage[u].w);
+        *reinterpret_cast<uint4*>(&vs[d * VP + 8 * c]) = stage[u];
       }
     }
     __syncthreads();

@@ -16,6 +16,9 @@ ARCH = "gfx950"
 # -packed-fp32-ops is switched off: the compiler must not form packed float32 instructions.
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-result"]
+# Attention rescales its MFMA accumulators with vector instructions at every step; kept in AGPRs each
+# such step would cost a move out and a move back, so these kernels take the VGPR form of MFMA.
+FILE_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources() -> list[str]:
@@ -30,6 +33,7 @@ def source_digest() -> str:
             with open(os.path.join(HERE, name), "rb") as f:
                 h.update(f.read())
     h.update(" ".join(FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()
 
 
@@ -63,7 +67,7 @@ def build(folder: str | None = None, verbose: bool = True, jobs: int | None = No
 
     def compile_one(name: str) -> str:
         obj = os.path.join(work, name[:-4] + ".o")
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(HERE, name), "-o", obj]
+        cmd = [hipcc, *FLAGS, *FILE_FLAGS.get(name, []), "-c", os.path.join(HERE, name), "-o", obj]
         t0 = time.time()
         done = subprocess.run(cmd, capture_output=True, text=True)
         if done.returncode != 0:
