@@ -11,11 +11,12 @@ bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
 size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx);
+size_t attention_prefill_workspace_floats(int n_tiles, int nq, int hd, int page_size, int max_tile_ctx);
 int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
-                   int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int hd, int page_size,
-                   int num_pages, int window, float scale);
+                   int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq, int nkv, int hd,
+                   int page_size, int num_pages, int window, float scale);
 }  // namespace sprout
 
 using namespace sprout;
@@ -40,17 +41,25 @@ extern "C" int sp_attention_plan(int dtype, int hd, int page_size, int nq, int n
   return 0;
 }
 
+static int64_t workspace_floats_of(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx,
+                                   int n_tiles, int max_tile_ctx) {
+  const size_t decode = attention_mfma_decode_supports(nq, nkv)
+                            ? attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx) : 0;
+  return (int64_t)(decode + attention_prefill_workspace_floats(n_tiles, nq, hd, page_size, max_tile_ctx));
+}
+
 extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
-                                                 int n_decode, int max_decode_ctx) {
-  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind) || !attention_mfma_decode_supports(nq, nkv)) return 0;
-  return (int64_t)attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx);
+                                                 int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx) {
+  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind)) return 0;
+  return workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, n_tiles, max_tile_ctx);
 }
 
 extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                             const void* v_pool, const int32_t* block_tables, int max_blocks,
                             const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
-                            const int32_t* tiles, int n_tiles, int tile_q, const int32_t* decode_seqs, int n_decode,
-                            int max_decode_ctx, float* workspace, int64_t workspace_floats, void* out, int nq,
+                            const int32_t* tiles, int n_tiles, int tile_q, int max_tile_ctx,
+                            const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
+                            int64_t workspace_floats, void* out, int nq,
                             int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind) {
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
@@ -71,11 +80,12 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   }
   SP_REQUIRE(max_decode_ctx >= 0 && max_decode_ctx <= max_blocks * page_size,
              "sp_attention: decode context %d exceeds the block tables", max_decode_ctx);
-  const int64_t need = (int64_t)attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx);
+  SP_REQUIRE(max_tile_ctx >= 0, "sp_attention: negative context length");
+  const int64_t need = workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, n_tiles, max_tile_ctx);
   SP_REQUIRE(need == 0 || (workspace && workspace_floats >= need),
              "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
              (long long)need);
   return attention_mfma(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
-                        n_tiles, decode_seqs, n_decode, max_decode_ctx, workspace, out, nq, nkv, hd, page_size,
-                        num_pages, window, scale);
+                        n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, workspace, out, nq, nkv, hd,
+                        page_size, num_pages, window, scale);
 }

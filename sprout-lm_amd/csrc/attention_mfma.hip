@@ -275,7 +275,8 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
-    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_shift, int num_pages,
+    const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int n_splits, int stages_per_split, int nq, int nkv, int page_shift, int num_pages,
     int window, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
@@ -336,7 +337,15 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int key0 = (k_lo / kStageKeys) * kStageKeys; key0 <= k_hi; key0 += kStageKeys) {
+  // With n_splits > 1 the stages of a tile are shared out between gridDim.z blocks, stages_per_split each
+  // (the last block takes what is left, however long the sequence), and the blocks leave partial results.
+  const int split = blockIdx.z;
+  int range_lo = (k_lo / kStageKeys) * kStageKeys, range_hi = k_hi;
+  if (n_splits > 1) {
+    range_lo = max(range_lo, split * stages_per_split * kStageKeys);
+    if (split + 1 < n_splits) range_hi = min(range_hi, (split + 1) * stages_per_split * kStageKeys - 1);
+  }
+  for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
     __syncthreads();   // the page numbers are in LDS; the last stage has been used
     const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
     uint4 stage[PER_THREAD];
@@ -422,9 +431,51 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) num[r4] += f * src[d + r4];
     }
+    if (n_splits > 1) {
+      // partial result of this block's keys: sums against the maximum mx, for the merge kernel
+      const size_t slot = ((size_t(tile) * (16 * NQT) + row) * nq + h) * n_splits + split;
+      *reinterpret_cast<float4*>(part_o + slot * HD + d) = make_float4(num[0], num[1], num[2], num[3]);
+      if (d == 0) *reinterpret_cast<float2*>(part_ml + 2 * slot) = make_float2(mx, den);
+      continue;
+    }
     const float inv = den > 0.f ? 1.0f / den : 0.f;
     uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD + d;
     *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
+  }
+}
+
+// Merges the partial results of the staged kernel's key splits: one wave per (query row, head).
+// part_o [tile][row][head][split][HD], part_ml [tile][row][head][split][2] = (maximum in log2 units, sum).
+template <int DT, int NQT>
+__global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ q_len, const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int n_splits,
+    int nq) {
+  constexpr int HD = 16 * DT, ROWS = 16 * NQT;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tile = blockIdx.x / (ROWS / 4), row = (blockIdx.x % (ROWS / 4)) * 4 + wave, h = blockIdx.y;
+  const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
+  if (q_off + row >= q_len[seq]) return;
+  const size_t base = ((size_t(tile) * ROWS + row) * nq + h) * n_splits;
+  float ms = kNoKeyYet, l = 0.f;
+  if (lane < n_splits) {
+    ms = part_ml[2 * (base + lane)];
+    l = part_ml[2 * (base + lane) + 1];
+  }
+  const float mx = wave_max(ms);
+  const float f = lane < n_splits ? exp2f(ms - mx) : 0.f;
+  const float den = wave_sum(f * l);
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  uint16_t* dst = out + size_t(q_start[seq] + q_off + row) * (size_t(nq) * HD) + h * HD;
+#pragma unroll
+  for (int j = 0; j < (HD + 63) / 64; ++j) {
+    const int d = lane + 64 * j;
+    float acc = 0.f;
+    for (int sp = 0; sp < n_splits; ++sp) {
+      const float fs = __shfl(f, sp, 64);
+      if (d < HD) acc = fmaf(fs, part_o[(base + sp) * HD + d], acc);
+    }
+    if (d < HD) dst[d] = f32_to_bf16_bits(acc * inv);
   }
 }
 
@@ -575,6 +626,24 @@ bool attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
 bool attention_mfma_decode_supports(int nq, int nkv) { return nq / nkv <= 16; }
 int attention_mfma_tile_q(int hd) { return 32; }
 
+constexpr int kMaxPrefillSplits = 32;   // the merge kernel holds one split per lane; 64 would do as well
+
+static bool staged_prefill(int page_size) { return page_size >= 8 && (page_size & (page_size - 1)) == 0; }
+
+// Blocks per tile and head along the keys.  A step with few queries over a long context (a portion of a long
+// prompt) has few tiles, each with a long walk: the walk is cut until the grid fills the chip about three times.
+int attention_prefill_splits(int n_tiles, int nq, int page_size, int max_tile_ctx) {
+  if (!staged_prefill(page_size)) return 1;
+  const int blocks = n_tiles * nq, stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
+  if (blocks <= 0 || blocks >= 512 || stages <= 4) return 1;
+  return max(1, min(min((768 + blocks - 1) / blocks, stages / 2), kMaxPrefillSplits));
+}
+
+size_t attention_prefill_workspace_floats(int n_tiles, int nq, int hd, int page_size, int max_tile_ctx) {
+  const size_t splits = attention_prefill_splits(n_tiles, nq, page_size, max_tile_ctx);
+  return splits <= 1 ? 0 : size_t(n_tiles) * 32 * nq * splits * (hd + 2);
+}
+
 size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx) {
   const size_t splits = (max_ctx + kDecodeChunk - 1) / kDecodeChunk;
   return splits <= 1 ? 0 : size_t(n_decode) * nq * splits * (hd + 2);
@@ -584,19 +653,31 @@ template <int DT>
 static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                        const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                        const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs,
-                       int n_decode, int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int page_size,
-                       int num_pages, int window, float scale) {
+                       int n_decode, int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq,
+                       int nkv, int page_size, int num_pages, int window, float scale) {
   constexpr int HD = 16 * DT;
   constexpr int NQT = 2;
   const float scale2 = scale * kLog2e;
   const uint16_t *qp = (const uint16_t*)q, *kp = (const uint16_t*)k_pool, *vp = (const uint16_t*)v_pool;
+  // the workspace holds the decode partials first, then the prefill partials
+  float* prefill_ws = workspace ? workspace + attention_decode_workspace_floats(n_decode, nq, HD, max_decode_ctx) : nullptr;
   if (n_tiles > 0) {
-    if (page_size >= 8 && (page_size & (page_size - 1)) == 0) {
+    if (staged_prefill(page_size)) {
       int page_shift = 0;
       while ((1 << page_shift) < page_size) ++page_shift;
-      attention_prefill_staged_kernel<DT, NQT><<<dim3(n_tiles, nq), 256, 0, s>>>(
-          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
-          page_shift, num_pages, window, scale2);
+      const int splits = attention_prefill_splits(n_tiles, nq, page_size, max_tile_ctx);
+      const int stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
+      const int per_split = (stages + splits - 1) / splits;
+      float* part_o = splits > 1 ? prefill_ws : nullptr;
+      float* part_ml = splits > 1 ? prefill_ws + size_t(n_tiles) * 16 * NQT * nq * splits * HD : nullptr;
+      attention_prefill_staged_kernel<DT, NQT><<<dim3(n_tiles, nq, splits), 256, 0, s>>>(
+          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, part_o,
+          part_ml, splits, per_split, nq, nkv, page_shift, num_pages, window, scale2);
+      if (splits > 1) {
+        if (check_launch("sp_attention (prefill)")) return 1;
+        attention_prefill_merge_kernel<DT, NQT><<<dim3(n_tiles * (16 * NQT / 4), nq), 256, 0, s>>>(
+            part_o, part_ml, q_start, q_len, tiles, (uint16_t*)out, splits, nq);
+      }
     } else {
       attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
@@ -624,13 +705,13 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
 int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
-                   int max_decode_ctx, float* workspace, void* out, int nq, int nkv, int hd, int page_size,
-                   int num_pages, int window, float scale) {
+                   int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq, int nkv, int hd,
+                   int page_size, int num_pages, int window, float scale) {
 #define SP_MFMA(DT)                                                                                              \
   case DT:                                                                                                       \
     return launch_mfma<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len,    \
-                           tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, workspace, out, nq, nkv,       \
-                           page_size, num_pages, window, scale)
+                           tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, workspace, out,  \
+                           nq, nkv, page_size, num_pages, window, scale)
   switch (hd / 16) {
     SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
   }

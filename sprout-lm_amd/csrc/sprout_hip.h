@@ -51,16 +51,18 @@ int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, 
 // sp_attention_plan tells how the caller must list the work: tiles [n_tiles][2] = (sequence, first
 // query of the tile within the sequence's tokens) of plan[0] queries each, over every sequence
 // (plan[1] == 1) or over the sequences with more than one query only, the others being listed in
-// decode_seqs (plan[1] == 0).  max_decode_ctx: largest ctx_len among decode_seqs.
+// decode_seqs (plan[1] == 0).  max_decode_ctx: largest ctx_len among decode_seqs; max_tile_ctx: largest
+// ctx_len among the sequences of the tile list (it only guides how a long walk over the keys is shared out
+// between blocks: a smaller value than the truth costs time, not correctness).
 // window <= 0: all keys; else keys with position - key < window.
 // workspace: sp_attention_workspace_floats(...) floats of scratch for partial results.
 int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind, int* plan);
 int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
-                                      int n_decode, int max_decode_ctx);
+                                      int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx);
 int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                  const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                  const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, int tile_q,
-                 const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
+                 int max_tile_ctx, const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
                  int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size, int num_pages,
                  int window, float scale, int kernel_kind);
 

@@ -68,7 +68,7 @@ class _DecodeGraph:
         lists = {f"tiles_multi_{t}": empty for t in ops.kernels.TILE_SIZES}
         lists.update({f"tiles_all_{t}": (every, S) for t in ops.kernels.TILE_SIZES})
         lists["decode_seqs"] = (view("decode_seqs"), S)
-        ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, S, lists, ctx_bucket)
+        ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, S, lists, ctx_bucket, ctx_bucket)
         ctx.group_tables = [view(f"tables{g}").view(S, self.max_blocks) for g in range(G)]
         ctx.group_slots = [view(f"slots{g}") for g in range(G)]
         ctx.n_tokens = ctx.n_seqs = ctx.n_logits = S

@@ -9,6 +9,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.spec import PagedKVSpec
 from ..config.base import token_id_list
+from .. import ops
 from ..models.plan import ModelPlan
 from ..registry import build_model_plan, load_config
 from ..weights.loader import load_named_tensors
@@ -167,16 +168,17 @@ class ModelRunner:
 
     def forward(self, ctx) -> torch.Tensor:
         T, H = ctx.n_tokens, self.hidden_size
-        residual = ctx.buffer("residual", (T, H), torch.float32)
-        self.parts.embedding.forward(ctx, ctx.token_ids, residual)
-        for call in self.plan.schedule:
-            self.parts.blocks[call.layer].forward(ctx, residual, self._slot_view(ctx, call))
-        n = ctx.n_logits
-        logits = ctx.buffer("logits", (n, self.vocab_size), torch.float32)
-        if n:
-            normed = ctx.buffer("final_normed", (n, H), self.dtype)
-            self.parts.final_norm.forward(ctx, residual, normed, rows=ctx.logit_rows)
-            self.parts.head.forward(ctx, normed, logits)
+        with ops.stream_scope():       # one stream lookup for the step's launches
+            residual = ctx.buffer("residual", (T, H), torch.float32)
+            self.parts.embedding.forward(ctx, ctx.token_ids, residual)
+            for call in self.plan.schedule:
+                self.parts.blocks[call.layer].forward(ctx, residual, self._slot_view(ctx, call))
+            n = ctx.n_logits
+            logits = ctx.buffer("logits", (n, self.vocab_size), torch.float32)
+            if n:
+                normed = ctx.buffer("final_normed", (n, H), self.dtype)
+                self.parts.final_norm.forward(ctx, residual, normed, rows=ctx.logit_rows)
+                self.parts.head.forward(ctx, normed, logits)
         return logits
 
     # ------------------------------------------------------------------ sizes

@@ -2,8 +2,8 @@
 and launches on torch's current stream."""
 from .kernels import (FUSED_ROPE, FUSED_SILU, AttentionBatch, attention, attention_lists, attention_plan, cast,
                       fused_supported, gate_up_silu, qkv_rope_cache, embed, gemm, rmsnorm, rope_cache, sample,
-                      sample_workspace_floats, silu_mul)
+                      sample_workspace_floats, silu_mul, stream_scope)
 from .library import KernelError, library
 
 __all__ = ["FUSED_ROPE", "FUSED_SILU", "fused_supported", "gate_up_silu", "qkv_rope_cache", "AttentionBatch", "attention", "attention_lists", "attention_plan", "cast", "embed", "gemm", "rmsnorm", "rope_cache", "sample",
-           "sample_workspace_floats", "silu_mul", "KernelError", "library"]
+           "sample_workspace_floats", "silu_mul", "stream_scope", "KernelError", "library"]

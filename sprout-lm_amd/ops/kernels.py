@@ -29,8 +29,30 @@ def _ints(t: torch.Tensor, n: int, what: str) -> None:
         raise KernelError(f"{what}: expected at least {n} int32 values, got {t.numel()} of {t.dtype}.")
 
 
+_scope_stream: int | None = None    # the stream of the enclosing stream_scope, if any
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return torch.cuda.current_stream().cuda_stream if _scope_stream is None else _scope_stream
+
+
+class stream_scope:
+    """Looks the current HIP stream up once for every launch inside the `with` block.
+
+    The lookup costs about as much as a launch itself, and a model step launches some two hundred
+    kernels.  Entered anew inside a graph capture, it picks up the capturing stream.
+    """
+
+    def __enter__(self):
+        global _scope_stream
+        self._outer = _scope_stream
+        _scope_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _scope_stream
+        _scope_stream = self._outer
+        return False
 
 
 def _ptr(t):
@@ -145,10 +167,11 @@ def attention_lists(q_lens) -> dict:
 class AttentionBatch:
     """The device-side description of a step's sequences that `attention` reads."""
 
-    def __init__(self, q_start, q_len, ctx_len, n_seqs: int, lists: dict, max_decode_ctx: int):
-        """`lists`: name -> (device int32 tensor, number of entries), names as in `attention_lists`."""
+    def __init__(self, q_start, q_len, ctx_len, n_seqs: int, lists: dict, max_decode_ctx: int, max_ctx: int):
+        """`lists`: name -> (device int32 tensor, number of entries), names as in `attention_lists`;
+        `max_decode_ctx`, `max_ctx`: the longest context among one-query sequences, and among all."""
         self.q_start, self.q_len, self.ctx_len, self.n_seqs = q_start, q_len, ctx_len, n_seqs
-        self.lists, self.max_decode_ctx = lists, max_decode_ctx
+        self.lists, self.max_decode_ctx, self.max_ctx = lists, max_decode_ctx, max_ctx
 
     @classmethod
     def build(cls, q_lens, ctx_lens, device) -> "AttentionBatch":
@@ -158,7 +181,8 @@ class AttentionBatch:
         starts = np.concatenate([[0], np.cumsum(q_lens)[:-1]]) if len(q_lens) else np.zeros(0)
         lists = {k: (to(v), len(v)) for k, v in attention_lists(q_lens).items()}
         decode_ctx = [c for c, q in zip(ctx_lens, q_lens) if q == 1]
-        return cls(to(starts), to(q_lens), to(ctx_lens), len(q_lens), lists, max(decode_ctx, default=0))
+        return cls(to(starts), to(q_lens), to(ctx_lens), len(q_lens), lists, max(decode_ctx, default=0),
+                   max((int(c) for c in ctx_lens), default=0))
 
 
 def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: int, kind: int = 0) -> tuple[int, bool]:
@@ -203,7 +227,9 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         _ints(decode, n_decode, "decode_seqs")
         if max_decode_ctx > block_tables.shape[1] * page_size:
             raise KernelError("attention: a decode context is longer than its block table")
-    need = library().sp_attention_workspace_floats(_code(q, "q"), hd, page_size, nq, nkv, kind, n_decode, max_decode_ctx)
+    max_tile_ctx = min(batch.max_ctx, block_tables.shape[1] * page_size) if n_tiles else 0
+    need = library().sp_attention_workspace_floats(_code(q, "q"), hd, page_size, nq, nkv, kind, n_decode, max_decode_ctx,
+                                                   n_tiles, max_tile_ctx)
     ws = None
     if need:
         ws = workspace(need) if workspace is not None else torch.empty(need, dtype=torch.float32, device=q.device)
@@ -212,7 +238,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
                                  batch.q_len.data_ptr(), batch.ctx_len.data_ptr(), _ptr(tiles) if n_tiles else None,
-                                 n_tiles, tile_q, _ptr(decode) if n_decode else None, n_decode, max_decode_ctx, _ptr(ws),
+                                 n_tiles, tile_q, max_tile_ctx, _ptr(decode) if n_decode else None, n_decode,
+                                 max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
                                  float(scale), kind))
 

@@ -23,8 +23,8 @@ def _declare(lib):
         "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
                           c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
-                         c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int, c_int,
-                         c_int, c_float, c_int],
+                         c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
+                         c_int, c_int, c_float, c_int],
         "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
         "sp_fused_supported": [c_int] * 7,
         "sp_gemm_decode": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_void, c_int,
@@ -37,7 +37,7 @@ def _declare(lib):
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
     }
-    lib.sp_attention_workspace_floats.argtypes = [c_int] * 8
+    lib.sp_attention_workspace_floats.argtypes = [c_int] * 10
     lib.sp_attention_workspace_floats.restype = c_i64
     for name, argtypes in sig.items():
         fn = getattr(lib, name)

@@ -252,6 +252,25 @@ def test_attention_finds_one_far_key_among_hundreds(dtype, kind, far):
     assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 0)])
+@pytest.mark.parametrize("nq,nkv,hd,page", [(4, 2, 64, 16), (3, 1, 32, 8), (6, 3, 80, 32), (8, 2, 128, 16)])
+@pytest.mark.parametrize("window", [None, 300])
+def test_attention_few_queries_over_a_long_context(dtype, kind, nq, nkv, hd, page, window):
+    """A portion of a long prompt beside short sequences: few tiles with a long walk over the keys, which
+    the bfloat16 kernel shares out between several blocks per tile and merges afterwards."""
+    seqs = [(3000, 40), (90, 90), (700, 1), (1537, 17), (129, 2)]
+    got, want = run_attention(dtype, nq, nkv, hd, page, seqs, window=window, kind=kind, seed=hd)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("far", [0, 127, 128, 1000, 2047, 2999])
+def test_attention_split_walk_finds_one_far_key(far):
+    got, want = run_attention(torch.bfloat16, 4, 2, 64, 16, [(3000, 1), (3000, 9)], kind=0, spike=(1, far), seed=far)
+    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+
+
 def test_attention_refuses_what_it_cannot_take():
     from sprout_lm_amd import ops
     q = torch.zeros(1, 4 * 16, device=DEV)
