@@ -17,6 +17,8 @@ class EngineOptions:
     prefill_chunk_size  most prompt tokens of one request in one step
     prefix_caching      share full prompt pages between requests
     record_trace        keep every event in `engine.trace`
+    decode_lookahead    launch the next step of decoded tokens before the running one has been read back
+                        (not in the reference; off: every step waits for its tokens first)
     """
 
     block_size: int = 16
@@ -26,11 +28,12 @@ class EngineOptions:
     prefill_chunk_size: int = 512
     prefix_caching: bool = True
     record_trace: bool = False
+    decode_lookahead: bool = True
 
     def __post_init__(self):
         for f in fields(self):
             value = getattr(self, f.name)
-            if f.name in ("prefix_caching", "record_trace"):
+            if f.name in ("prefix_caching", "record_trace", "decode_lookahead"):
                 if not isinstance(value, bool):
                     raise ConfigError(f"{f.name} must be a boolean.")
             elif isinstance(value, bool) or not isinstance(value, int) or value <= 0:

@@ -108,7 +108,30 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict
 
 }  // namespace sprout
 
+namespace sprout {
+// tokens[i] = previous[source[i]] where source[i] >= 0 (a token that an earlier step sampled and the host
+// has not read yet); an invalid token (the sampler's mark for non-finite logits) becomes 0: the step's
+// result is thrown away by the host, but its kernels must not index with it.
+__global__ void feed_tokens_kernel(int32_t* __restrict__ tokens, const int32_t* __restrict__ previous,
+                                   const int32_t* __restrict__ source, int n, int vocab) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int from = source[i];
+  if (from < 0) return;
+  const int token = previous[from];
+  tokens[i] = token >= 0 && token < vocab ? token : 0;
+}
+}  // namespace sprout
+
 using namespace sprout;
+
+extern "C" int sp_feed_tokens(void* stream, int32_t* tokens, const int32_t* previous, const int32_t* source, int n,
+                              int vocab) {
+  SP_REQUIRE(n >= 0 && vocab > 0 && tokens && previous && source, "sp_feed_tokens: bad arguments");
+  if (n == 0) return 0;
+  feed_tokens_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(tokens, previous, source, n, vocab);
+  return check_launch("sp_feed_tokens");
+}
 
 extern "C" int sp_embed(void* stream, int table_dtype, const void* table, const int32_t* tokens,
                         float* residual, int T, int H, int V) {

@@ -72,6 +72,11 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 // dst (dst_dtype) = src (src_dtype), n elements
 int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n);
 
+// tokens[i] = previous[source[i]] for every i < n with source[i] >= 0 (others are left as they are):
+// feeds tokens sampled by a step that the host has not read yet into the next step.  previous holds at
+// least max(source) + 1 entries; a value outside [0, vocab) is replaced by 0.
+int sp_feed_tokens(void* stream, int32_t* tokens, const int32_t* previous, const int32_t* source, int n, int vocab);
+
 // Greedy / temperature sampling of R rows of float32 logits [R, V].
 // temperature[r] == 0: lowest index of the maximum.  Else argmax of logits / temperature + Gumbel noise
 // from a counter generator keyed by (seed[r], counter[r], column).

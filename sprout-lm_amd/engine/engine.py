@@ -52,6 +52,7 @@ class Engine:
         self.sampler = sampler     # None: the model samples on the device (`step_and_sample`)
         self.scheduler = Scheduler(cache, self.options, model.vocab_size, model.max_positions, model.stop_token_ids)
         self._auto_ids = itertools.count()
+        self._ahead = None      # (work, handle) of a step launched before its predecessor was read back
 
     @classmethod
     def from_folder(cls, folder: str, dtype="bfloat16", options: EngineOptions | None = None, **overrides) -> "Engine":
@@ -98,27 +99,75 @@ class Engine:
         return self.scheduler.result(id)
 
     def step(self) -> StepReport:
-        """One scheduling iteration: plan, run the batch, sample, book (src/engine.ts:127-189)."""
-        work = self.scheduler.plan()
+        """One scheduling iteration: plan, run the batch, sample, book (src/engine.ts:127-189).
+
+        A step of decoded tokens is launched and, before its tokens are read back, the step after it is
+        planned and launched as well where the scheduler can foresee it (`plan_ahead`): the host then
+        plans one step while the GPU computes the other.  That step is booked by the next call.
+        """
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and not any(w.request.status == "running" for w in ahead[0]):
+            self._discard(ahead)    # every request of it has ended meanwhile: nothing to book
+            ahead = None
+        if ahead is not None:
+            work, pending = ahead
+            self.scheduler.begin_ahead()
+        else:
+            work, pending = self.scheduler.plan(), None
         sampled: dict[str, int] = {}
         reports = []
         if work:
-            entries = [StepEntry(w.request.seq, w.tokens, [len(w.tokens) - 1] if w.samples else []) for w in work]
+            sampling = [w for w in work if w.samples]
             try:
-                sampling = [w for w in work if w.samples]
-                params = [w.request.params for w in sampling]
-                counters = [len(w.request.output) for w in sampling]
-                if self.sampler is None:
+                if pending is None:
+                    entries = [StepEntry(w.request.seq, w.tokens, [len(w.tokens) - 1] if w.samples else []) for w in work]
+                    params = [w.request.params for w in sampling]
+                    counters = [len(w.request.output) for w in sampling]
+                    launch = getattr(self.model, "launch_decode", None) if self.sampler is None else None
+                    if launch is not None:
+                        pending = launch(entries, params, counters)
+                if pending is not None:
+                    self._launch_ahead(work, pending)
+                    tokens = self.model.finish_decode(pending)
+                elif self.sampler is None:
                     tokens = self.model.step_and_sample(entries, params, counters)
                 else:
                     tokens = self.sampler.sample(self.model.step(entries), params, counters)
             except Exception as error:
+                if self._ahead is not None:
+                    self._discard(self._ahead)
+                    self._ahead = None
                 self.scheduler.fail_all(str(error))
                 raise
             sampled = {w.request.id: t for w, t in zip(sampling, tokens)}
             reports = [w.report() for w in work]
         events = self.scheduler.complete(work, sampled)
         return StepReport(self.scheduler.tick, reports, events, self.cache)
+
+    @staticmethod
+    def _discard(ahead) -> None:
+        """Wait for a launched step whose result nobody wants: what it reads and writes (cache pages, the
+        recorded graph and its buffers) must not be given back or destroyed under it."""
+        try:
+            ahead[1].result()
+        except Exception:
+            pass
+
+    def _launch_ahead(self, work, pending) -> None:
+        """Plan and launch the step after `work` (which runs as `pending`) if it can be foreseen."""
+        if not self.options.decode_lookahead:
+            return
+        following = self.scheduler.plan_ahead(work)
+        if not following:
+            return
+        row = {w.request.id: i for i, w in enumerate(work)}
+        entries = [StepEntry(w.request.seq, [None], [0]) for w in following]
+        sources = [row[w.request.id] for w in following]
+        params = [w.request.params for w in following]
+        counters = [len(w.request.output) + 1 for w in following]     # the running step's token comes first
+        launched = self.model.launch_decode(entries, params, counters, feed=(pending, sources))
+        if launched is not None:
+            self._ahead = (following, launched)
 
     # ------------------------------------------------------------------ conveniences
     def generate(self, prompts, max_new_tokens: int = 16, temperature: float = 0.0, seed: int = 0,
@@ -162,4 +211,12 @@ class Engine:
                 "evictions": self.cache.evictions}
 
     def close(self) -> None:
+        if self._ahead is not None:
+            self._discard(self._ahead)
+            self._ahead = None
         self.scheduler.fail_all("closed")
+
+    def __del__(self):
+        ahead = getattr(self, "_ahead", None)
+        if ahead is not None:
+            self._discard(ahead)

@@ -12,6 +12,9 @@ power-of-two context.  Nothing in a graph depends on the values of a step.
 """
 from __future__ import annotations
 
+import gc
+import weakref
+
 import numpy as np
 import torch
 
@@ -27,7 +30,10 @@ class _DecodeGraph:
     """Static buffers and the recorded graph of one (sequences, context) bucket."""
 
     def __init__(self, runner, n_seqs: int, ctx_bucket: int):
-        self.runner, self.S = runner, n_seqs
+        # the runner owns the graphs; a strong reference back would make a cycle that only the garbage
+        # collector frees, at a moment of its own choosing (see _record)
+        self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
+        self.S = n_seqs
         cache = runner.cache
         bs = cache.block_size
         self.max_blocks = -(-ctx_bucket // bs)
@@ -35,7 +41,7 @@ class _DecodeGraph:
         S, G = n_seqs, len(cache.groups)
         # layout of the int32 staging buffer
         names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots",
-                 "seq_of_token", "decode_seqs", "counter", "temperature"]
+                 "seq_of_token", "decode_seqs", "counter", "temperature", "feed_source"]
         self.offsets, total = {}, 0
         for name in names:
             self.offsets[name] = (total, S)
@@ -57,6 +63,7 @@ class _DecodeGraph:
         for name in ("q_start", "logit_rows", "seq_of_token", "decode_seqs"):
             self.h[name][:] = arange
         self.h["q_len"][:] = 1
+        self.h["feed_source"][:] = -1
 
         # buffers of its own: a graph holds their addresses, so they must never be reallocated
         ctx = StepContext(Workspace(runner.device), runner.dtype, runner.attention_kind)
@@ -77,6 +84,8 @@ class _DecodeGraph:
         self.temperature = view("temperature").view(torch.float32)
         self.seed = view("seed").view(torch.int64)
         self.counter = view("counter")
+        self.feed_source = view("feed_source")
+        self.copied = None         # event: the staging buffer of the last launch has reached the device
         self.sampled = torch.zeros(S, dtype=torch.int32, device=runner.device)
         self.sample_ws = torch.empty(max(1, ops.sample_workspace_floats(S, runner.vocab_size)), dtype=torch.float32,
                                      device=runner.device)
@@ -85,15 +94,20 @@ class _DecodeGraph:
         self._filled = -1          # number of real sequences at the last fill
         self._rows = [None] * S    # per row: which sequence and how many pages its table row holds
 
-    def fill(self, entries, params, counters) -> None:
+    def fill(self, entries, params, counters, sources=None) -> None:
         """Write this step's values into the pinned staging buffer.
 
         Block-table rows are rewritten only when a row's sequence or its number of pages has changed
-        since the last step (a steady decode batch gains a page every `block_size` steps)."""
+        since the last step (a steady decode batch gains a page every `block_size` steps).
+        `sources[i] >= 0`: entry i's token is row sources[i] of an earlier step's sampled tokens, which
+        the host does not know yet (its `tokens[0]` is None)."""
         cache, h, n, S = self.runner.cache, self.h, len(entries), self.S
         bs = cache.block_size
+        if self.copied is not None:
+            self.copied.synchronize()      # the last launch's upload may still be reading the staging buffer
         lengths = np.fromiter((e.seq.length for e in entries), dtype=np.int32, count=n)
-        h["token_ids"][:n] = [e.tokens[0] for e in entries]
+        h["token_ids"][:n] = [e.tokens[0] or 0 for e in entries]
+        h["feed_source"][:n] = -1 if sources is None else sources
         h["positions"][:n] = lengths
         h["ctx_len"][:n] = lengths + 1
         h["state_slots"][:n] = [e.seq.state_slot for e in entries]
@@ -103,6 +117,7 @@ class _DecodeGraph:
         if n != self._filled:
             for name in ("token_ids", "positions", "state_slots", "temperature"):
                 h[name][n:] = 0
+            h["feed_source"][n:] = -1
             h["ctx_len"][n:] = 1
             self._rows = [None] * S
         last_block = lengths // bs
@@ -126,8 +141,15 @@ class _DecodeGraph:
             slots[:n] = pages * bs + lengths % bs
         self._filled = n
 
-    def launch(self) -> None:
+    def launch(self, previous=None) -> None:
+        """Upload the staging buffer and run the step; `previous`: the device tensor of sampled tokens that
+        `feed_source` indexes."""
         self.dev.copy_(self.host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+        if previous is not None:
+            ops.feed_tokens(self.ctx.token_ids, previous, self.feed_source, self.runner.vocab_size)
         if self.graph is None:
             self._record()
         else:
@@ -143,10 +165,18 @@ class _DecodeGraph:
         torch.cuda.current_stream().synchronize()
         self.ctx.workspace.frozen = True
         graph = torch.cuda.CUDAGraph()
+        # No garbage collection while the stream is capturing: a dead cycle that holds GPU objects (an older
+        # engine's graphs, events, pinned buffers) would be destroyed in the middle of the capture, and what
+        # their destructors call is not allowed then (the process aborts).  Collect first, then hold it off.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
         try:
             with torch.cuda.graph(graph):
                 self._body()
         finally:
+            if collecting:
+                gc.enable()
             self.ctx.workspace.frozen = False
         self.graph = graph
         # the eager run above already produced this step's results; replaying would only repeat it
@@ -154,7 +184,7 @@ class _DecodeGraph:
 
 class DecodeGraphs:
     def __init__(self, runner, max_graphs: int = 32):
-        self.runner = runner
+        self.runner = weakref.proxy(runner)
         self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
         self.max_graphs = max_graphs
         self.replays = 0
@@ -164,8 +194,13 @@ class DecodeGraphs:
         return (runner.parts.graph_safe and not runner.cache.state_groups and len(entries) > 0
                 and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries))
 
-    def run(self, entries, params, counters) -> list[int]:
-        """One decode step of `entries` with sampling; returns the sampled token ids."""
+    def launch(self, entries, params, counters, feed=None) -> "PendingDecode":
+        """Start one decode step of `entries` with sampling and return without waiting for it.
+
+        `feed`: (an earlier, possibly unfinished PendingDecode, for every entry the row of its token among
+        that step's entries or -1).  Entries with a row >= 0 carry `tokens == [None]`: the token goes from
+        step to step on the device.  The sequences' lengths are advanced before the call returns.
+        """
         runner = self.runner
         n = len(entries)
         S = _bucket(n)
@@ -177,10 +212,39 @@ class DecodeGraphs:
             if len(self.graphs) >= self.max_graphs:
                 self.graphs.pop(next(iter(self.graphs)))
             state = self.graphs[key] = _DecodeGraph(runner, S, ctx_bucket)
-        state.fill(entries, params, counters)
-        state.launch()
+        previous, sources = (None, None) if feed is None else (feed[0].sampled, feed[1])
+        state.fill(entries, params, counters, sources)
+        state.launch(previous)
         self.replays += 1
-        tokens = state.sampled[:n].tolist()      # waits for the step
+        pending = PendingDecode(state.sampled, n, self._host_tokens(S))
         for e in entries:
             runner.cache.commit(e.seq, e.seq.length + 1)
-        return tokens
+        return pending
+
+    def run(self, entries, params, counters) -> list[int]:
+        """One decode step of `entries` with sampling; returns the sampled token ids."""
+        return self.launch(entries, params, counters).result()
+
+    def _host_tokens(self, n: int) -> torch.Tensor:
+        """A pinned buffer for a step's sampled tokens; a few are kept and handed out in turn (a step's
+        buffer is read before the step after next is launched)."""
+        if not hasattr(self, "_pinned") or self._pinned[0].numel() < n:
+            self._pinned = [torch.zeros(max(n, 64), dtype=torch.int32, pin_memory=True) for _ in range(4)]
+            self._turn = 0
+        self._turn = (self._turn + 1) % len(self._pinned)
+        return self._pinned[self._turn]
+
+
+class PendingDecode:
+    """A launched decode step: the sampled tokens are on their way to the host."""
+
+    def __init__(self, sampled: torch.Tensor, n: int, host: torch.Tensor):
+        self.sampled, self.n = sampled, n       # the step's device buffer: valid until the same graph runs again
+        self._host = host
+        host[:n].copy_(sampled[:n], non_blocking=True)
+        self._done = torch.cuda.Event()
+        self._done.record()
+
+    def result(self) -> list[int]:
+        self._done.synchronize()
+        return self._host[:self.n].tolist()

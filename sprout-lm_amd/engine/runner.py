@@ -111,12 +111,15 @@ class ModelRunner:
                 if needed:
                     raise ValueError("Pages for the entry's tokens were not reserved before the step.")
 
-    def validate_decode(self, entries: list[StepEntry]) -> None:
-        """The checks of `validate` for a step of single tokens, in one pass."""
+    def validate_decode(self, entries: list[StepEntry], sources=None) -> None:
+        """The checks of `validate` for a step of single tokens, in one pass.  An entry whose token is still
+        on the device (`sources[i] >= 0`) brings None in its place."""
         seen = set()
         bs, limit, vocab = self.cache.block_size, self.max_positions, self.vocab_size
-        for e in entries:
+        for i, e in enumerate(entries):
             seq, token = e.seq, e.tokens[0]
+            if token is None and sources is not None and sources[i] >= 0:
+                token = 0
             if id(seq) in seen:
                 raise ValueError("A request appears twice in one step.")
             seen.add(id(seq))
@@ -151,20 +154,38 @@ class ModelRunner:
 
         Steps in which every request brings one token are replayed from a recorded HIP graph.
         """
-        from ..sampling.sampler import NonFiniteLogits, Sampler
-        if self.use_graphs:
-            if self._graphs is None:
-                from .graphs import DecodeGraphs
-                self._graphs = DecodeGraphs(self)
-            if self._graphs.usable(entries):
-                self.validate_decode(entries)
-                tokens = self._graphs.run(entries, params, counters)
-                if any(t < 0 or t >= self.vocab_size for t in tokens):
-                    raise NonFiniteLogits("Non-finite logits: the model produced NaN or infinity.")
-                return tokens
+        from ..sampling.sampler import Sampler
+        pending = self.launch_decode(entries, params, counters)
+        if pending is not None:
+            return self.finish_decode(pending)
         if self._sampler is None:
             self._sampler = Sampler(self.device, self.vocab_size)
         return self._sampler.sample(self.step(entries), params, counters)
+
+    def launch_decode(self, entries: list[StepEntry], params, counters, feed=None):
+        """Start a step in which every request brings one token, without waiting for its result.
+
+        Returns a handle for `finish_decode`, or None if the step cannot run from a recorded graph (then
+        nothing has been launched).  `feed`: (handle of an earlier step, row of each entry's token among that
+        step's entries or -1): tokens the host has not seen go from step to step on the device.
+        """
+        if not self.use_graphs:
+            return None
+        if self._graphs is None:
+            from .graphs import DecodeGraphs
+            self._graphs = DecodeGraphs(self)
+        if not self._graphs.usable(entries):
+            return None
+        self.validate_decode(entries, None if feed is None else feed[1])
+        return self._graphs.launch(entries, params, counters, feed)
+
+    def finish_decode(self, pending) -> list[int]:
+        """Wait for a launched decode step; returns its sampled token ids."""
+        from ..sampling.sampler import NonFiniteLogits
+        tokens = pending.result()
+        if any(t < 0 or t >= self.vocab_size for t in tokens):
+            raise NonFiniteLogits("Non-finite logits: the model produced NaN or infinity.")
+        return tokens
 
     def forward(self, ctx) -> torch.Tensor:
         T, H = ctx.n_tokens, self.hidden_size

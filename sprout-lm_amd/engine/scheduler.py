@@ -9,7 +9,9 @@ token while it computes, all pages of a step are settled here before anything is
 request that is preempted while the step is planned brings no tokens to that step.
 
 The scheduler decides and keeps the books; it launches nothing.  `plan()` returns the work of the
-next step, the caller runs it and reports the sampled tokens to `complete()`.
+next step, the caller runs it and reports the sampled tokens to `complete()`.  While a step of decoded
+tokens runs, `plan_ahead()` may already settle the step after it, so that the host's work for one step
+overlaps the GPU's work for the other (no counterpart in the reference, whose steps are synchronous).
 """
 from __future__ import annotations
 
@@ -164,6 +166,39 @@ class Scheduler:
             planned[request.id] = Work(request, phase, start, tokens, samples=start + count == total)
             budget -= count
         return [planned[r.id] for r in batch if r.id in planned]
+
+    def plan_ahead(self, running: list[Work]) -> list[Work] | None:
+        """The step after `running`, planned while that step is still being computed.
+
+        Possible only where the next step can be foreseen without the tokens on their way: `running` is a
+        step of single decoded tokens of every active request, nobody waits for admission, and every
+        request that goes on has a page for one more token (nothing is preempted on a guess).  A request
+        that will reach its token limit is left out; one that turns out to have stopped at an end token is
+        not known yet and is included: its share of the step is computed in vain and ignored by
+        `complete`.  The tokens of the returned work are [None]: they are not known on the host.
+        Returns None when the caller should wait for the running step and `plan()` as usual.
+        """
+        if self.waiting or not running:
+            return None
+        if any(w.phase != "decode" or not w.samples for w in running):
+            return None
+        alive = [w.request for w in running if w.request.status == "running"]
+        if len(alive) != len(self.active) or any(r.id not in self.active for r in alive):
+            return None
+        if any(r.seq.length != r.history_length() for r in alive):
+            return None        # `running` has not been launched: its tokens are not in the cache yet
+        ahead = [r for r in alive if len(r.output) + 1 < r.max_new_tokens]
+        if not ahead:
+            return None
+        for r in ahead:
+            if not self.cache.reserve(r.seq, r.seq.length + 1):
+                return None
+        return [Work(r, "decode", r.seq.length, [None], samples=True) for r in ahead]
+
+    def begin_ahead(self) -> None:
+        """A step planned by `plan_ahead` becomes the current one (what `plan()` does besides choosing)."""
+        self.tick += 1
+        self._step_events = []
 
     def complete(self, work: list[Work], sampled: dict[str, int]) -> list[dict]:
         """Book a finished step: lengths have advanced; `sampled` maps request id -> new token."""

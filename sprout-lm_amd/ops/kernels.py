@@ -244,6 +244,13 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  float(scale), kind))
 
 
+def feed_tokens(tokens: torch.Tensor, previous: torch.Tensor, source: torch.Tensor, vocab: int) -> None:
+    """tokens[i] = previous[source[i]] where source[i] >= 0: tokens of a step the host has not read yet."""
+    n = tokens.numel()
+    _ints(tokens, n, "tokens"); _ints(source, n, "token sources"); _ints(previous, 1, "sampled tokens")
+    check(library().sp_feed_tokens(_stream(), tokens.data_ptr(), previous.data_ptr(), source.data_ptr(), n, int(vocab)))
+
+
 FUSED_ROPE, FUSED_SILU = 3, 4
 
 

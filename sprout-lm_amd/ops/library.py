@@ -36,6 +36,7 @@ def _declare(lib):
         "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
+        "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],
     }
     lib.sp_attention_workspace_floats.argtypes = [c_int] * 10
     lib.sp_attention_workspace_floats.restype = c_i64

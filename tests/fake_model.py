@@ -24,6 +24,7 @@ class FakeRunner:
         self.cache = CacheManager([PagedKVSpec(1, 8)] * layers, block_size, num_blocks, max_sequences, prefix_caching)
         self.slots = {}          # (page, offset) -> (token, position)
         self.steps = []          # tokens per step
+        self.fed = 0             # tokens that went from one step to the next without the host seeing them
         self._memo = {}
 
     def logits_of(self, history) -> np.ndarray:
@@ -52,11 +53,35 @@ class FakeRunner:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
         return np.stack(rows) if rows else np.zeros((0, self.vocab_size), np.float32)
 
+    # ---- the runner's own sampling entry points (greedy), as the engine uses them without a sampler
+    def step_and_sample(self, entries, params, counters):
+        return [int(np.argmax(row)) for row in self.step(entries)]
+
+    def launch_decode(self, entries, params, counters, feed=None):
+        """A step of single tokens that is "launched": computed at once here, read back by finish_decode.
+        A token the host does not know yet (None) is taken from the earlier step's result, as the device does."""
+        if any(len(e.tokens) != 1 or len(e.want) != 1 for e in entries):
+            return None
+        for i, e in enumerate(entries):
+            if e.tokens[0] is None:
+                assert feed is not None and feed[1][i] >= 0, "an unknown token needs a source"
+                e.tokens[0] = feed[0].tokens[feed[1][i]]
+                self.fed += 1
+        return _Launched(self.step_and_sample(entries, params, counters))
+
+    def finish_decode(self, launched):
+        return list(launched.tokens)
+
     def greedy(self, prompt, steps):
         out = []
         for _ in range(steps):
             out.append(int(np.argmax(self.logits_of(list(prompt) + out))))
         return out
+
+
+class _Launched:
+    def __init__(self, tokens):
+        self.tokens = tokens
 
 
 class ArgmaxSampler:

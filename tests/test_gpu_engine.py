@@ -178,6 +178,80 @@ def test_graph_replays_equal_eager_steps(folders):
     assert graphed == eager
 
 
+def test_lookahead_equals_synchronous_steps(folders):
+    """The next decode step launched before the running one is read back (tokens go from step to step on the
+    device) gives every request the tokens of steps that each wait for their result: greedy and with
+    temperature, requests of different lengths, one arriving under way."""
+    from sprout_lm_amd.engine import Engine
+    name = "A"
+    vocab = H.CONFIGS[name]["vocab_size"]
+    prompts = [H.random_tokens(vocab, n, 40 + i) for i, n in enumerate((6, 19, 33, 4))]
+
+    def run(lookahead):
+        engine = Engine.from_folder(folders[name], "bfloat16", block_size=16, num_blocks=48, max_sequences=4,
+                                    max_batch_tokens=32, prefill_chunk_size=16, decode_lookahead=lookahead)
+        engine.add("r0", prompts[0], 40, ignore_eos=True)
+        engine.add("r1", prompts[1], 22, temperature=0.7, seed=11, ignore_eos=True)
+        engine.add("r2", prompts[2], 9, ignore_eos=True)
+        steps = ahead = 0
+        while engine.pending:
+            steps += 1
+            if steps == 25:
+                engine.add("r3", prompts[3], 14, ignore_eos=True)
+            engine.step()
+            ahead += engine._ahead is not None
+        return [engine.result(f"r{i}")["output"] for i in range(4)], ahead
+
+    sync, none = run(False)
+    overlapped, launched = run(True)
+    assert none == 0 and launched > 20
+    assert overlapped == sync
+
+
+def test_lookahead_steps_give_the_tokens_of_synchronous_steps(folders):
+    """With the next decode step launched before the running one is read back (tokens go from step to step on
+    the device) every request gets the tokens it gets when each step waits for its result: greedy and with
+    temperature, with an end token that stops one request early, arrivals, a cancellation, and context buckets
+    that change under way."""
+    from sprout_lm_amd.engine import Engine
+    name = "C"
+    vocab = H.CONFIGS[name]["vocab_size"]
+    folder = H.make_model_folder(os.path.dirname(folders["A"]), name)
+    prompts = [H.random_tokens(vocab, n, 90 + i) for i, n in enumerate((5, 30, 250, 9, 17))]
+
+    def run(lookahead, stop=None):
+        engine = Engine.from_folder(folder, "bfloat16", block_size=16, num_blocks=64, max_sequences=4,
+                                    max_batch_tokens=64, prefill_chunk_size=32, decode_lookahead=lookahead)
+        engine.add("r0", prompts[0], 60, ignore_eos=True)
+        engine.add("r1", prompts[1], 40, stop_token_ids=None if stop is None else [stop])
+        engine.add("r2", prompts[2], 25, temperature=0.9, seed=3, ignore_eos=True)     # crosses 256 keys
+        steps, ahead = 0, 0
+        while engine.pending:
+            steps += 1
+            if steps == 20:
+                engine.add("r3", prompts[3], 30, ignore_eos=True)
+            if steps == 30:
+                engine.cancel("r0")
+                engine.add("r4", prompts[4], 12, temperature=0.5, seed=1, ignore_eos=True)
+            engine.step()
+            ahead += engine._ahead is not None
+        engine.cache.clear_prefixes()
+        assert engine.cache.free_pages() == [64] * len(engine.cache.free_pages())
+        return {f"r{i}": engine.result(f"r{i}") for i in range(5)}, ahead
+
+    first, _ = run(False)
+    stop = first["r1"]["output"][11]
+    sync, none = run(False, stop)
+    ahead, launched = run(True, stop)
+    assert none == 0 and launched > 30
+    assert sync["r1"]["finish_reason"] == "eos" and len(sync["r1"]["output"]) <= 12
+    for k in ("r1", "r2", "r3", "r4"):
+        assert ahead[k]["output"] == sync[k]["output"] and ahead[k]["finish_reason"] == sync[k]["finish_reason"], k
+    assert ahead["r0"]["status"] == "cancelled"
+    n = min(len(ahead["r0"]["output"]), len(sync["r0"]["output"]))
+    assert n > 5 and ahead["r0"]["output"][:n] == sync["r0"]["output"][:n]
+
+
 def test_real_layer_sizes_both_dtypes(tmp_path):
     """Two layers with the sizes of Qwen2.5-0.5B (hidden 896, 14 heads in 2 groups of head size 64, inner 4864,
     vocabulary 151936, tied): whole prompt, portions and single tokens against the plain implementation."""

@@ -189,3 +189,97 @@ def test_generate_returns_outputs_in_order():
     engine = make(max_sequences=2)
     prompts = [prompt("one"), prompt("second"), prompt("3")]
     assert engine.generate(prompts, max_new_tokens=3) == [engine.model.greedy(p, 3) for p in prompts]
+
+
+# ---- the next decode step launched before the running one is read back ---------------------------------
+
+def make_lookahead(lookahead=True, **kw):
+    runner = FakeRunner(kw.pop("block_size", 4), kw.pop("num_blocks", 64), kw.pop("max_sequences", 4), True, kw.pop("eos", ()))
+    kw.setdefault("max_batch_tokens", 8)
+    kw.setdefault("prefill_chunk_size", 4)
+    return Engine(runner, record_trace=True, decode_lookahead=lookahead, **kw)
+
+
+def test_lookahead_changes_no_output_and_feeds_tokens_on_the_device():
+    prompts = {"a": prompt("alpha"), "b": prompt("be"), "c": prompt("gamma ray")}
+    limits = {"a": 9, "b": 3, "c": 14}
+    probe = make_lookahead(False)
+    stop = probe.model.greedy(prompts["a"], 5)[4]          # request a ends early at an end token
+    outputs = {}
+    for lookahead in (False, True):
+        engine = make_lookahead(lookahead)
+        for id, p in prompts.items():
+            engine.add(id, p, limits[id], stop_token_ids=[stop] if id == "a" else None)
+        reports = drain(engine)
+        outputs[lookahead] = {id: engine.result(id) for id in prompts}
+        assert (engine.model.fed > 0) == lookahead
+        assert engine._ahead is None or not any(w.request.status == "running" for w in engine._ahead[0])
+        engine.cache.clear_prefixes()
+        assert engine.cache.free_pages() == [engine.options.num_blocks]
+        ticks = [r.tick for r in reports]
+        assert ticks == sorted(set(ticks))
+    for id in prompts:
+        assert outputs[True][id]["output"] == outputs[False][id]["output"]
+        assert outputs[True][id]["finish_reason"] == outputs[False][id]["finish_reason"]
+    assert outputs[True]["a"]["finish_reason"] == "eos" and outputs[True]["b"]["finish_reason"] == "length"
+    assert outputs[True]["c"]["output"] == probe.model.greedy(prompts["c"], limits["c"])
+    want = probe.model.greedy(prompts["a"], limits["a"])
+    assert outputs[True]["a"]["output"] == want[:want.index(stop) + 1]
+
+
+def test_lookahead_with_cancellation_and_a_late_request():
+    engine = make_lookahead(True, block_size=2)
+    pa, pb, pc = prompt("abc"), prompt("defg"), prompt("hi")
+    engine.add("A", pa, 12)
+    engine.add("B", pb, 12)
+    while not (engine.result("A")["output"] and engine.result("B")["output"]):
+        engine.step()
+    engine.step()
+    assert engine._ahead is not None                      # a step is in flight beyond the one just booked
+    assert engine.cancel("A")                             # ... with a share for A, which is thrown away
+    engine.add("C", pc, 4)                                # joins after the step in flight
+    drain(engine)
+    assert engine.result("A")["status"] == "cancelled"
+    assert engine.result("B")["output"] == engine.model.greedy(pb, 12)
+    assert engine.result("C")["output"] == engine.model.greedy(pc, 4)
+    engine.cache.clear_prefixes()
+    assert engine.cache.free_pages() == [engine.options.num_blocks]
+
+
+def test_plan_ahead_only_where_the_next_step_is_certain():
+    # somebody waits for admission: the next step is not certain, every step is read back first
+    engine = make_lookahead(True, max_sequences=1)
+    engine.add("A", prompt("abc"), 6)
+    engine.add("B", prompt("de"), 3)
+    while engine.result("A")["status"] != "finished":
+        engine.step()
+        assert engine._ahead is None
+    drain(engine)
+    assert engine.model.fed > 0                           # B, alone at the end, did run ahead
+    # a prompt portion in the batch: not a step of decoded tokens only
+    engine = make_lookahead(True)
+    engine.add("A", prompt("ab"), 8)
+    engine.step(); engine.step()
+    engine.add("late", prompt("a long prompt that takes several portions"), 2)
+    engine.step()                                         # books the step in flight
+    while not engine.result("late")["output"]:
+        engine.step()
+        assert engine._ahead is None
+    drain(engine)
+    assert engine.result("A")["output"] == engine.model.greedy(prompt("ab"), 8)
+    # no free page for the token after next: nothing is preempted on a guess, the ordinary plan decides
+    engine = make_lookahead(True, block_size=2, num_blocks=5, max_sequences=2)
+    pa, pb = prompt("abc"), prompt("de")
+    engine.add("A", pa, 8)
+    engine.add("B", pb, 8)
+    reports = drain(engine)
+    assert engine.result("A")["output"] == engine.model.greedy(pa, 8)
+    assert engine.result("B")["output"] == engine.model.greedy(pb, 8)
+    assert engine.stats()["preemptions"] > 0
+    assert all(e["type"] != "preempted" or e["id"] == "B" for r in reports for e in r.events)
+    # the scheduler itself refuses a step that has not been launched (its tokens are not in the cache yet)
+    engine = make_lookahead(False)
+    engine.add("A", prompt("ab"), 8)
+    engine.step(); engine.step()
+    work = engine.scheduler.plan()
+    assert [w.phase for w in work] == ["decode"] and engine.scheduler.plan_ahead(work) is None
