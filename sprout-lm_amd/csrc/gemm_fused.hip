@@ -92,6 +92,29 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   load_weights(wave);
   __builtin_amdgcn_sched_barrier(0);   // keep these loads ahead of the prologue
 
+  // What the epilogue reads per output (bias, position, rotation frequency, cache slot) is requested now
+  // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
+  // thread -> (token et of a tile, row ei of the tile), as in the epilogue below
+  const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
+  float bias_of[2] = {0.f, 0.f};
+  if (a.bias && blockIdx.y == 0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (row0[i] + ei < a.N) bias_of[i] = load_param(a.bias, a.bias_bf16, row0[i] + ei);
+  }
+  int position_of[TN], slot_of[TN];
+  float frequency = 0.f;
+  if (EPI == kEpiRope) {
+    const int d = row0[0] % a.hd + ei;
+    if (d < a.rotary_dim / 2) frequency = a.inv_freq[d];
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      const int t = min(tn * 16 + et, a.T - 1);
+      position_of[tn] = a.positions[t];
+      slot_of[tn] = a.slot_mapping[t];
+    }
+  }
+
   if (NORM) {
     // RMSNorm of up to 16 tokens: 16 threads per token, each owning every 16th group of four columns,
     // so that a token's loads are all in flight together and its sum closes with four lane exchanges.
@@ -198,7 +221,6 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   __syncthreads();
 
   // thread -> (token t of the tile, row i of the tile); the MFMA lane that holds it is (i / 4) * 16 + t, element i % 4
-  const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
   const int src_lane = (ei >> 2) * 16 + et, src_r = ei & 3;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
@@ -209,9 +231,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       float sum = 0.f;
 #pragma unroll
       for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * 2 + i) * TN + tn) * 64 + src_lane])[src_r];
-      const int n = row0[i] + ei;
-      if (a.bias && blockIdx.y == 0 && n < a.N) sum += load_param(a.bias, a.bias_bf16, n);
-      v[i] = sum;
+      v[i] = sum + bias_of[i];
     }
     if (t >= a.T) continue;
     if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
@@ -239,7 +259,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       const int half = a.hd / 2;
       if (head < a.nq + a.nkv && d < a.rotary_dim / 2 && half == a.rotary_dim / 2) {
         float sn, cs;
-        sincosf(float(a.positions[t]) * a.inv_freq[d], &sn, &cs);
+        sincosf(float(position_of[tn]) * frequency, &sn, &cs);
         const float rl = lo * cs - hi * sn, rh = hi * cs + lo * sn;
         lo = rl;
         hi = rh;
@@ -250,7 +270,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         q[d] = blo;
         q[d + half] = bhi;
       } else {
-        const int slot = a.slot_mapping[t];
+        const int slot = slot_of[tn];
         if (slot >= 0) {
           const int page = slot / a.page_size, off = slot % a.page_size;
           if (head < a.nq + a.nkv) {
