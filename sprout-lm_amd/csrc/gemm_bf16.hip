@@ -186,7 +186,8 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
 }  // namespace sprout
 
 // ------------------------------------------------------------------------------------------------
-// Tiled kernel (T > 64, prefill): both operands go through LDS in steps of 64 or 128 along K; 4 waves in a
+// Tiled kernel for the shapes that the pipelined kernel (gemm_pipe.hip) does not take: T > 64 with a K that is
+// no multiple of 64.  Both operands go through LDS in steps of 64 or 128 along K; 4 waves in a
 // 2 x 2 arrangement, each computing WM x WN tiles of 32 x 32 on 32x32x16 MFMA with the weights as the
 // A operand (D[n, t]), so that a lane ends with four consecutive n of one token and stores 8 or 16 bytes.
 // The next step is on its way from memory while one is multiplied.  Small accumulating products may be
@@ -356,7 +357,8 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
   return launch_tiled<1, 1, TB>(s, x, w, bias, mode, out, T, N, K, splits_for(blocks(64, 64)));
 }
 
-// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for T > 64: 128-token tiles, 64 gate + 64 up rows per block.
+// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T): the pipelined kernel where it takes the shape, else (T > 64)
+// this file's kernel with 128-token tiles, 64 gate + 64 up rows per block.
 int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
   if (gemm_pipe_takes(T, 2 * I, K)) return gemm_bf16_pipe_silu(s, x, w, out, T, I, K);
   dim3 grid((I + 63) / 64, (T + 127) / 128, 1);
