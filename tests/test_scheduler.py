@@ -283,3 +283,46 @@ def test_plan_ahead_only_where_the_next_step_is_certain():
     engine.step(); engine.step()
     work = engine.scheduler.plan()
     assert [w.phase for w in work] == ["decode"] and engine.scheduler.plan_ahead(work) is None
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_lookahead_under_random_arrivals_cancellations_and_pressure(seed):
+    """Requests arrive, stop at end tokens, are cancelled and preempted at random while steps run ahead: every
+    request that finishes has the tokens it would have had alone, and no page is lost."""
+    import random
+    rng = random.Random(seed)
+    num_blocks = rng.choice([6, 9, 16, 40])
+    engine = make_lookahead(True, block_size=rng.choice([2, 4]), num_blocks=num_blocks, max_sequences=rng.choice([2, 3, 4]),
+                            max_batch_tokens=rng.choice([6, 8, 16]), prefill_chunk_size=rng.choice([2, 4, 8]))
+    capacity = num_blocks * engine.options.block_size
+    plans, live, cancelled = {}, [], set()
+    next_id = steps = 0
+    while steps < 400 and (engine.pending or next_id < 12):
+        steps += 1
+        if next_id < 12 and rng.random() < 0.35:
+            p = [rng.randrange(50) for _ in range(rng.randrange(1, 9))]
+            limit = rng.randrange(1, 10)
+            if len(p) + limit - 1 <= min(capacity, engine.model.max_positions):
+                greedy = engine.model.greedy(p, limit)
+                stop = greedy[rng.randrange(limit)] if rng.random() < 0.4 else None
+                id = f"q{next_id}"
+                engine.add(id, p, limit, stop_token_ids=None if stop is None else [stop], ignore_eos=stop is None)
+                plans[id] = greedy[:greedy.index(stop) + 1] if stop is not None else greedy
+                live.append(id)
+            next_id += 1
+        if live and rng.random() < 0.05:
+            victim = rng.choice(live)
+            if engine.cancel(victim):
+                cancelled.add(victim)
+        report = engine.step()
+        assert all(p["refs"] >= 0 and p["active_refs"] >= 0 for p in report.memory["pages"])
+        live = [i for i in live if engine.result(i)["status"] in ("waiting", "running")]
+    assert not engine.pending
+    for id, want in plans.items():
+        result = engine.result(id)
+        if id in cancelled:
+            assert result["status"] == "cancelled" and result["output"] == want[:len(result["output"])]
+        else:
+            assert result["status"] == "finished" and result["output"] == want, id
+    engine.cache.clear_prefixes()
+    assert engine.cache.free_pages() == [num_blocks]
