@@ -72,8 +72,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
 
-  // The first weights are requested before anything else: they do not depend on the prologue, and
-  // their way from memory is the longest wait of the kernel.
+  // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
+  // of this wave together.
   constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
   const int steps = (k_end - k_begin + 63) / 64;
   uint4 wa[UN][2][2];
@@ -89,9 +89,47 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       }
     }
   };
+  // RMSNorm of up to 16 tokens: 16 threads per token, each owning every 16th group of four columns,
+  // so that a token's loads are all in flight together and its sum closes with four lane exchanges.
+  const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
+  const float* row = NORM ? a.residual + size_t(min(t, a.T - 1)) * a.K : nullptr;   // rows past T repeat the last one
+  float4 v[16], wn[16];
+  auto load_values = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int k = k0 + 4 * part + 64 * j;
+      v[j] = k < a.K ? *reinterpret_cast<const float4*>(row + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
+  auto load_norm_weights = [&](int k0) {   // one vector load per group of four columns
+    if (a.norm_w_bf16) {
+      const uint16_t* nw = reinterpret_cast<const uint16_t*>(a.norm_w);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int k = k0 + 4 * part + 64 * j;
+        const uint2 b = k < a.K ? *reinterpret_cast<const uint2*>(nw + k) : make_uint2(0, 0);
+        wn[j] = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
+                            __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
+      }
+    } else {
+      const float* nw = reinterpret_cast<const float*>(a.norm_w);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int k = k0 + 4 * part + 64 * j;
+        wn[j] = k < a.K ? *reinterpret_cast<const float4*>(nw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  };
+  // Loads return in the order of their requests.  The residual rows (close by, in L2) are therefore asked for
+  // before the weights (far, in memory): they arrive early, and the norm is computed while the weights are
+  // still on their way.  (With the weights first, the norm waited for them and stood between them and the
+  // products: it then cost as much as a kernel of its own.)
+  if (NORM) {
+    load_values(0);
+    load_norm_weights(0);
+  }
   load_weights(wave);
-  __builtin_amdgcn_sched_barrier(0);   // keep these loads ahead of the prologue
-
+  __builtin_amdgcn_sched_barrier(0);   // keep these requests ahead of everything below
   // What the epilogue reads per output (bias, position, rotation frequency, cache slot) is requested now
   // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
   // thread -> (token et of a tile, row ei of the tile), as in the epilogue below
@@ -116,41 +154,9 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   }
 
   if (NORM) {
-    // RMSNorm of up to 16 tokens: 16 threads per token, each owning every 16th group of four columns,
-    // so that a token's loads are all in flight together and its sum closes with four lane exchanges.
-    const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
-    const float* row = a.residual + size_t(min(t, a.T - 1)) * a.K;     // rows past T repeat the last one
-    float4 v[16], wn[16];
-    auto load_values = [&](int k0) {
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int k = k0 + 4 * part + 64 * j;
-        v[j] = k < a.K ? *reinterpret_cast<const float4*>(row + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    };
-    auto load_norm_weights = [&](int k0) {   // one vector load per group of four columns
-      if (a.norm_w_bf16) {
-        const uint16_t* nw = reinterpret_cast<const uint16_t*>(a.norm_w);
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int k = k0 + 4 * part + 64 * j;
-          const uint2 b = k < a.K ? *reinterpret_cast<const uint2*>(nw + k) : make_uint2(0, 0);
-          wn[j] = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
-                              __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
-        }
-      } else {
-        const float* nw = reinterpret_cast<const float*>(a.norm_w);
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int k = k0 + 4 * part + 64 * j;
-          wn[j] = k < a.K ? *reinterpret_cast<const float4*>(nw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-      }
-    };
     float sum = 0.f;
     for (int k0 = 0; k0 < a.K; k0 += 1024) {
-      load_values(k0);
-      if (a.K <= 1024) load_norm_weights(0);               // requested together with the values
+      if (k0 > 0) load_values(k0);                         // the first 1024 columns were requested above
 #pragma unroll
       for (int j = 0; j < 16; ++j) sum = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, sum))));
     }

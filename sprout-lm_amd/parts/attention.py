@@ -69,9 +69,9 @@ class Attention(Mixer):
                 and ops.fused_supported(ops.FUSED_ROPE, T, self.w_qkv.shape[0], self.hidden, self.head_dim,
                                         self.position.rotary_dim, norm))
 
-    # Folding the norm into the projection kernel saves a launch but puts the norm's memory round trip
-    # in front of every block; on MI355X both cost the same 3.3 us at hidden size 896, so it is off.
-    fuse_input_norm = False
+    # Folding the norm into the projection kernel (up to 16 tokens) saves a launch; the kernel asks for the
+    # residual rows before its weights, so the norm is computed while the weights are on their way.
+    fuse_input_norm = True
 
     def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
         T = residual.shape[0]
