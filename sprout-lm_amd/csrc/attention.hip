@@ -70,8 +70,7 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   sp_attention_plan(dtype, hd, page_size, nq, nkv, kernel_kind, plan);
   SP_REQUIRE(tile_q == plan[0], "sp_attention: tiles were built for %d queries, the kernel takes %d", tile_q, plan[0]);
   SP_REQUIRE(plan[1] == 0 || n_decode == 0, "sp_attention: this kernel takes every sequence in the tile list");
-  SP_REQUIRE(n_tiles >= 0 && n_decode >= 0 && (n_tiles == 0 || tiles) && (n_decode == 0 || decode_seqs),
-             "sp_attention: missing tile or sequence list");
+  SP_REQUIRE(n_tiles >= 0 && n_decode >= 0 && (n_tiles == 0 || tiles), "sp_attention: missing tile list");
   hipStream_t s = (hipStream_t)stream;
   if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind)) {
     if (n_tiles == 0) return 0;

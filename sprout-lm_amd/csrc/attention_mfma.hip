@@ -493,7 +493,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   __shared__ float s_o[4][16][HD + 1];
   __shared__ float s_m[4][16], s_l[4][16];
   const int split = blockIdx.x, g = blockIdx.y, di = blockIdx.z;
-  const int seq = decode_seqs[di];
+  const int seq = decode_seqs ? decode_seqs[di] : di;   // no list: the batch is one-query sequences only, in order
   const int ctx = ctx_len[seq], pos = ctx - 1;
   const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int chunk0 = split * kDecodeChunk;
@@ -576,7 +576,7 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
   constexpr int HD = 16 * DT;
   __shared__ float s_f[64];
   const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int seq = decode_seqs[di];
+  const int seq = decode_seqs ? decode_seqs[di] : di;   // no list: the batch is one-query sequences only, in order
   const int pos = ctx_len[seq] - 1;
   const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int first = k_lo / kDecodeChunk, last = pos / kDecodeChunk;   // the chunks that wrote something

@@ -41,7 +41,7 @@ class _DecodeGraph:
         S, G = n_seqs, len(cache.groups)
         # layout of the int32 staging buffer
         names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots",
-                 "seq_of_token", "decode_seqs", "counter", "temperature", "feed_source"]
+                 "seq_of_token", "counter", "temperature", "feed_source"]
         self.offsets, total = {}, 0
         for name in names:
             self.offsets[name] = (total, S)
@@ -60,7 +60,7 @@ class _DecodeGraph:
         self.h = {name: self.host_np[o:o + n] for name, (o, n) in self.offsets.items()}
         # constant parts
         arange = np.arange(S, dtype=np.int32)
-        for name in ("q_start", "logit_rows", "seq_of_token", "decode_seqs"):
+        for name in ("q_start", "logit_rows", "seq_of_token"):
             self.h[name][:] = arange
         self.h["q_len"][:] = 1
         self.h["feed_source"][:] = -1
@@ -74,7 +74,7 @@ class _DecodeGraph:
         every = torch.from_numpy(np.stack([arange, np.zeros_like(arange)], axis=1)).to(runner.device)
         lists = {f"tiles_multi_{t}": empty for t in ops.kernels.TILE_SIZES}
         lists.update({f"tiles_all_{t}": (every, S) for t in ops.kernels.TILE_SIZES})
-        lists["decode_seqs"] = (view("decode_seqs"), S)
+        lists["decode_seqs"] = (None, S)        # every sequence brings one token, in order: no list needed
         ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, S, lists, ctx_bucket, ctx_bucket)
         ctx.group_tables = [view(f"tables{g}").view(S, self.max_blocks) for g in range(G)]
         ctx.group_slots = [view(f"slots{g}") for g in range(G)]

@@ -224,7 +224,10 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     _ints(tiles, 2 * n_tiles, "tiles")
     max_decode_ctx = batch.max_decode_ctx if n_decode else 0
     if n_decode:
-        _ints(decode, n_decode, "decode_seqs")
+        if decode is not None:         # None: sequences 0 .. n_decode - 1
+            _ints(decode, n_decode, "decode_seqs")
+        elif n_decode != n_seqs:
+            raise KernelError("attention: without a decode list every sequence must bring one query")
         if max_decode_ctx > block_tables.shape[1] * page_size:
             raise KernelError("attention: a decode context is longer than its block table")
     max_tile_ctx = min(batch.max_ctx, block_tables.shape[1] * page_size) if n_tiles else 0
