@@ -497,8 +497,17 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   const int ctx = ctx_len[seq], pos = ctx - 1;
   const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int chunk0 = split * kDecodeChunk;
-  if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) return;   // no visible key in this chunk
   const int G = nq / nkv;
+  if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) {
+    // no visible key in this chunk: the merge kernel reads every chunk's (maximum, sum) without looking at
+    // the context length, so an empty chunk says so itself
+    if (n_splits > 1 && threadIdx.x < G) {
+      const size_t slot = (size_t(di) * nq + g * G + threadIdx.x) * n_splits + split;
+      part_ml[2 * slot] = kNoKeyYet;
+      part_ml[2 * slot + 1] = 0.f;
+    }
+    return;
+  }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
 
   PagedKV kv;
@@ -563,54 +572,53 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 }
 
-// Merges the chunks of one (sequence, head): grid (decode sequences, heads), one wave each.
-// Lane i first takes chunk i's maximum (up to 64 chunks at a time), then lane d sums dimension d.
+// Merges the chunks of one (sequence, head): grid (decode sequences, heads), one wave each; lane d sums
+// dimension d.  Everything the wave reads depends on its indices alone (empty chunks are marked as such by
+// the decode kernel), so all of it is requested at once: one trip to memory.
 template <int DT>
 __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
                                                              const float* __restrict__ part_ml,
                                                              const int32_t* __restrict__ q_start,
-                                                             const int32_t* __restrict__ ctx_len,
                                                              const int32_t* __restrict__ decode_seqs,
-                                                             uint16_t* __restrict__ out, int n_splits, int nq,
-                                                             int window) {
-  constexpr int HD = 16 * DT;
-  __shared__ float s_f[64];
+                                                             uint16_t* __restrict__ out, int n_splits, int nq) {
+  constexpr int HD = 16 * DT, PER_LANE = (HD + 63) / 64, GROUP = 16;
   const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int seq = decode_seqs ? decode_seqs[di] : di;   // no list: the batch is one-query sequences only, in order
-  const int pos = ctx_len[seq] - 1;
-  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int first = k_lo / kDecodeChunk, last = pos / kDecodeChunk;   // the chunks that wrote something
+  const int seq = decode_seqs ? decode_seqs[di] : di;
   const size_t base = (size_t(di) * nq + head) * n_splits;
-  float mx = -INFINITY;
-  for (int s0 = first; s0 <= last; s0 += 64)
-    if (s0 + lane <= last) mx = fmaxf(mx, part_ml[2 * (base + s0 + lane)]);
-  mx = wave_max(mx);
-  float num[(HD + 63) / 64] = {}, den = 0.f;
-  for (int s0 = first; s0 <= last; s0 += 64) {
-    const int count = min(64, last - s0 + 1);
-    float f = 0.f, l = 0.f;
-    if (lane < count) {
-      const float ms = part_ml[2 * (base + s0 + lane)];
-      f = exp2f(ms - mx);
-      l = part_ml[2 * (base + s0 + lane) + 1];
-    }
-    den += wave_sum(f * l);
-    __syncthreads();
-    s_f[lane] = f;
-    __syncthreads();
+  float mx = kNoKeyYet, den = 0.f, num[PER_LANE] = {};
+  for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+    float ms[GROUP], ls[GROUP], os[GROUP][PER_LANE];
 #pragma unroll
-    for (int j = 0; j < (HD + 63) / 64; ++j) {
-      const int d = lane + 64 * j;
-      if (d < HD) {
-        float acc = 0.f;
-#pragma unroll 8
-        for (int i = 0; i < count; ++i) acc = fmaf(s_f[i], part_o[(base + s0 + i) * HD + d], acc);
-        num[j] += acc;
+    for (int i = 0; i < GROUP; ++i) {
+      const bool in = s0 + i < n_splits;
+      ms[i] = in ? part_ml[2 * (base + s0 + i)] : kNoKeyYet;      // the same address in every lane: one read
+      ls[i] = in ? part_ml[2 * (base + s0 + i) + 1] : 0.f;
+#pragma unroll
+      for (int j = 0; j < PER_LANE; ++j) {
+        const int d = lane + 64 * j;
+        os[i][j] = (in && d < HD) ? part_o[(base + s0 + i) * HD + d] : 0.f;
+      }
+    }
+    float group_max = mx;
+#pragma unroll
+    for (int i = 0; i < GROUP; ++i) group_max = fmaxf(group_max, ms[i]);
+    const float keep = exp2f(mx - group_max);
+    mx = group_max;
+    den *= keep;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) num[j] *= keep;
+#pragma unroll
+    for (int i = 0; i < GROUP; ++i) {
+      if (ls[i] > 0.f) {                      // an empty chunk left nothing to read in part_o
+        const float f = exp2f(ms[i] - mx);
+        den = fmaf(f, ls[i], den);
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) num[j] = fmaf(f, os[i][j], num[j]);
       }
     }
   }
 #pragma unroll
-  for (int j = 0; j < (HD + 63) / 64; ++j) {
+  for (int j = 0; j < PER_LANE; ++j) {
     const int d = lane + 64 * j;
     if (d < HD)
       out[size_t(q_start[seq]) * (size_t(nq) * HD) + head * HD + d] = f32_to_bf16_bits(den > 0.f ? num[j] / den : 0.f);
@@ -694,8 +702,8 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
         n_splits, nq, nkv, page_size, num_pages, window, scale2);
     if (check_launch("sp_attention (decode)")) return 1;
     if (n_splits > 1) {
-      attention_merge_kernel<DT><<<dim3(n_decode, nq), 64, 0, s>>>(part_o, part_ml, q_start, ctx_len, decode_seqs,
-                                                                    (uint16_t*)out, n_splits, nq, window);
+      attention_merge_kernel<DT><<<dim3(n_decode, nq), 64, 0, s>>>(part_o, part_ml, q_start, decode_seqs,
+                                                                    (uint16_t*)out, n_splits, nq);
       if (check_launch("sp_attention (merge)")) return 1;
     }
   }
