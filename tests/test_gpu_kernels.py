@@ -21,7 +21,8 @@ def bf16(x):
                                    (77, 300, 129), (200, 96, 224), (130, 257, 511), (129, 257, 200), (300, 331, 240),
                                    (513, 1152, 896), (2, 896, 4864), (40, 640, 1000), (64, 151, 72), (1000, 130, 136),
                                    (130, 257, 64), (200, 96, 192), (129, 300, 1024), (1000, 130, 128), (300, 331, 320),
-                                   (700, 896, 4864), (65, 2100, 448)])
+                                   (700, 896, 4864), (65, 2100, 448),
+                                   (300, 4608, 3584), (40, 3584, 18944), (24, 3584, 3584), (520, 9728, 896)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
