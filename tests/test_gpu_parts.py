@@ -345,3 +345,221 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
         s.release()
     assert runner.cache.free_pages() == [40, 40]
     print(f"toy {dtype}: worst error {worst:.3e}")
+
+
+# A second toy architecture: a feed-forward with routing and a position encoding of its own, both
+# registered here and nowhere in the engine.
+
+def register_routed_toy():
+    from dataclasses import dataclass
+    from typing import ClassVar
+
+    import sprout_lm_amd as S
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.config.base import ModelConfig
+    from sprout_lm_amd.models.plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+    from sprout_lm_amd.parts import FeedForward, PositionEncoding, register_part, registered_parts
+    from sprout_lm_amd.weights import TensorSpec
+
+    if "toy_top1_experts" in registered_parts("feed_forward"):
+        return
+
+    @register_part("position", "toy_stretched_rotary")
+    class StretchedRotary(PositionEncoding):
+        """Rotation of the first `rotary_dim` dims of a head only, with positions divided by `stretch`."""
+
+        graph_safe = True
+
+        def __init__(self, head_dim, theta, rotary_dim, stretch):
+            self.head_dim, self.theta, self.rotary_dim, self.stretch = head_dim, theta, rotary_dim, stretch
+            self.inv_freq = None
+
+        def prepare(self, device, dtype):
+            d = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
+            self.inv_freq = (float(self.theta) ** (-d / self.rotary_dim) / self.stretch).to(torch.float32).to(device)
+
+    @register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(FeedForward):
+        """Every token goes to the expert with the largest router logit; its SwiGLU output is weighted with
+        that expert's softmax probability.  Router logits and probabilities are float32."""
+
+        def __init__(self, hidden, inner, experts):
+            self.hidden, self.inner, self.experts = hidden, inner, experts
+
+        def tensors(self):
+            out = {"router.weight": TensorSpec((self.experts, self.hidden))}
+            for e in range(self.experts):
+                out[f"experts.{e}.gate_up.weight"] = TensorSpec((2 * self.inner, self.hidden))
+                out[f"experts.{e}.down.weight"] = TensorSpec((self.hidden, self.inner))
+            return out
+
+        def forward(self, ctx, h, residual):
+            T = h.shape[0]
+            logits = torch.empty(T, self.experts, dtype=torch.float32, device=h.device)
+            ops.gemm(h, self.w["router.weight"], logits)
+            prob, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            for e in range(self.experts):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                x = h[rows].contiguous()
+                gu = torch.empty(x.shape[0], 2 * self.inner, dtype=h.dtype, device=h.device)
+                ops.gemm(x, self.w[f"experts.{e}.gate_up.weight"], gu)
+                act = torch.empty(x.shape[0], self.inner, dtype=h.dtype, device=h.device)
+                ops.silu_mul(gu, act)
+                y = torch.empty(x.shape[0], self.hidden, dtype=torch.float32, device=h.device)
+                ops.gemm(act, self.w[f"experts.{e}.down.weight"], y)
+                residual.index_add_(0, rows, y * prob[rows, None])
+
+    @dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyRoutedForCausalLM"
+        model_types: ClassVar[tuple] = ("toy_routed",)
+        hidden: int = 0
+        inner: int = 0
+        vocab: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        experts: int = 0
+        rotary_dim: int = 0
+        stretch: float = 0.0
+        eps: float = 0.0
+        theta: float = 0.0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "experts", "rotary_dim",
+                                               "stretch", "eps", "theta")})
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "model_type": "toy_routed",
+                    **{k: getattr(self, k) for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "experts",
+                                                      "rotary_dim", "stretch", "eps", "theta")}}
+
+    def build(cfg):
+        hd = cfg.hidden // cfg.heads
+        norm = lambda prefix: PartPlan("norm", "rmsnorm", {"size": cfg.hidden, "eps": cfg.eps}, prefix)
+        attention = lambda prefix, position: PartPlan("mixer", "attention", {
+            "hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.kv_heads, "head_dim": hd, "position": position,
+            "qkv_bias": False}, prefix)
+        stretched = PartPlan("position", "toy_stretched_rotary", {"head_dim": hd, "theta": cfg.theta,
+                                                                   "rotary_dim": cfg.rotary_dim, "stretch": cfg.stretch})
+        layers = [
+            LayerPlan("pre_norm", {"mixer_norm": norm("l0.n1."), "mixer": attention("l0.attn.", stretched),
+                                   "ffn_norm": norm("l0.n2."),
+                                   "ffn": PartPlan("feed_forward", "toy_top1_experts",
+                                                   {"hidden": cfg.hidden, "inner": cfg.inner, "experts": cfg.experts},
+                                                   "l0.moe.")}),
+            LayerPlan("pre_norm", {"mixer_norm": norm("l1.n1."),
+                                   "mixer": attention("l1.attn.", PartPlan("position", "none", {"head_dim": hd})),
+                                   "ffn_norm": norm("l1.n2."),
+                                   "ffn": PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner},
+                                                   "l1.mlp.")}),
+        ]
+        return ModelPlan("ToyRoutedForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
+                         PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.hidden}, "embed."),
+                         layers, [LayerCall(0, 0), LayerCall(1, 1)], norm("final."),
+                         PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.hidden, "tied": False}, "head."))
+
+    S.register_architecture("ToyRoutedForCausalLM", RoutedConfig, build, model_types=("toy_routed",))
+
+
+ROUTED = dict(model_type="toy_routed", hidden=64, inner=48, vocab=101, heads=2, kv_heads=2, experts=3, rotary_dim=16,
+              stretch=4.0, eps=1e-6, theta=5e3)
+
+
+def plain_routed_logits(w, tokens, store):
+    """The routed toy, whole sequence.  Returns the logits and, per token, the gap between the two largest
+    router logits (a token on the edge between two experts may go either way in bfloat16)."""
+    c = ROUTED
+    hd = c["hidden"] // c["heads"]
+    pos = np.arange(len(tokens), dtype=np.float64)
+    x = P.f32(w["embed.weight"][np.asarray(tokens)])
+
+    def stretched_rope(t):
+        t = np.asarray(t, dtype=np.float64).reshape(len(tokens), c["heads"], hd).copy()
+        half = c["rotary_dim"] // 2
+        d = np.arange(half, dtype=np.float64)
+        angle = (pos / c["stretch"])[:, None] / c["theta"] ** (2.0 * d / c["rotary_dim"])
+        cos, sin = np.cos(angle)[:, None, :], np.sin(angle)[:, None, :]
+        a, b = t[..., :half].copy(), t[..., half:2 * half].copy()
+        t[..., :half] = a * cos - b * sin
+        t[..., half:2 * half] = b * cos + a * sin
+        return P.f32(t.reshape(len(tokens), -1))
+
+    def attn(x, i, rotate):
+        n = store(P.rms_norm(x, w[f"l{i}.n1.weight"], c["eps"]))
+        p = f"l{i}.attn."
+        q, k, v = (store(P.linear(n, w[p + f"{name}_proj.weight"])) for name in "qkv")
+        if rotate:
+            q, k = store(stretched_rope(q)), store(stretched_rope(k))
+        a = store(P.causal_gqa_attention(q, k, v, c["heads"], c["kv_heads"], hd))
+        return P.f32(x + P.linear(a, w[p + "o_proj.weight"]))
+
+    x = attn(x, 0, True)
+    n = store(P.rms_norm(x, w["l0.n2.weight"], c["eps"]))
+    logits = np.asarray(P.linear(n, w["l0.moe.router.weight"]), dtype=np.float64)
+    top = np.sort(logits, axis=-1)
+    gap = top[:, -1] - top[:, -2]
+    prob = np.exp(logits - logits.max(-1, keepdims=True))
+    prob /= prob.sum(-1, keepdims=True)
+    choice = logits.argmax(-1)
+    out = np.zeros_like(x, dtype=np.float64)
+    for e in range(c["experts"]):
+        rows = np.nonzero(choice == e)[0]
+        if len(rows) == 0:
+            continue
+        gu = store(P.linear(n[rows], w[f"l0.moe.experts.{e}.gate_up.weight"]))
+        act = store(P.swiglu(gu[:, :c["inner"]], gu[:, c["inner"]:]))
+        out[rows] = np.asarray(P.linear(act, w[f"l0.moe.experts.{e}.down.weight"]), dtype=np.float64) * prob[rows, e, None]
+    x = P.f32(x + out)
+    x = attn(x, 1, False)
+    n = store(P.rms_norm(x, w["l1.n2.weight"], c["eps"]))
+    gate, up = store(P.linear(n, w["l1.mlp.gate_proj.weight"])), store(P.linear(n, w["l1.mlp.up_proj.weight"]))
+    x = P.f32(x + P.linear(store(P.swiglu(gate, up)), w["l1.mlp.down_proj.weight"]))
+    return P.linear(store(P.rms_norm(x, w["final.weight"], c["eps"])), w["head.weight"]), gap
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path, dtype):
+    """A feed-forward with routing (router logits and probabilities in float32) and a position encoding that the
+    engine does not have, defined and registered in this file, built from a model folder and stepped in portions
+    beside another request."""
+    register_routed_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    folder = str(tmp_path / "routed")
+    write_model_folder(folder, S.config_from_dict(ROUTED), seed=5, dtype=torch.bfloat16, std=0.2)
+    runner = ModelRunner.from_folder(folder, dtype, block_size=8, num_blocks=24, max_sequences=2)
+    assert not runner.parts.graph_safe                        # the routed feed-forward decides on the host
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    store = P.bf16_round if dtype == "bfloat16" else P.f32
+    requests = {"a": H.random_tokens(101, 37, 7), "b": H.random_tokens(101, 20, 8)}
+    want = {k: plain_routed_logits(w, t, store) for k, t in requests.items()}
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    seqs = {k: runner.cache.create() for k in requests}
+    fed = {k: 0 for k in requests}
+    used = set()
+    checked = 0
+    for step in [{"a": 11, "b": 3}, {"a": 1, "b": 9}, {"a": 2, "b": 1}, {"a": 23, "b": 7}]:
+        entries, rows = [], []
+        for rid, n in step.items():
+            assert runner.cache.reserve(seqs[rid], fed[rid] + n)
+            entries.append(StepEntry(seqs[rid], requests[rid][fed[rid]:fed[rid] + n], list(range(n))))
+            rows += [(rid, fed[rid] + i) for i in range(n)]
+            fed[rid] += n
+        got = runner.step(entries).cpu().numpy()
+        for row, (rid, pos) in zip(got, rows):
+            logits, gap = want[rid]
+            # a token's own routing must be clear of ties, and so must that of every earlier token it attends to
+            if gap[:pos + 1].min() < 0.05:
+                continue
+            checked += 1
+            err = np.abs(row - logits[pos]).max()
+            assert err <= tol * (1 + np.abs(logits[pos]).max()), f"{rid} position {pos}: {err:.3e}"
+    assert fed == {k: len(v) for k, v in requests.items()} and checked >= 20
+    for s in seqs.values():
+        s.release()
+    assert runner.cache.free_pages() == [24]             # both layers have the same needs: one group of pages
