@@ -207,11 +207,14 @@ class DecodeGraphs:
         longest = max(e.seq.length for e in entries) + 1
         ctx_bucket = min(_bucket(longest, 256), -(-runner.max_positions // 256) * 256)
         key = (S, ctx_bucket)
-        state = self.graphs.get(key)
+        state = self.graphs.pop(key, None)
         if state is None:
             if len(self.graphs) >= self.max_graphs:
+                # the least recently used graph goes; a step launched ahead may still be running from it
+                torch.cuda.current_stream().synchronize()
                 self.graphs.pop(next(iter(self.graphs)))
-            state = self.graphs[key] = _DecodeGraph(runner, S, ctx_bucket)
+            state = _DecodeGraph(runner, S, ctx_bucket)
+        self.graphs[key] = state          # most recently used last
         previous, sources = (None, None) if feed is None else (feed[0].sampled, feed[1])
         state.fill(entries, params, counters, sources)
         state.launch(previous)

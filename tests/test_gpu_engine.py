@@ -187,9 +187,12 @@ def test_lookahead_equals_synchronous_steps(folders):
     vocab = H.CONFIGS[name]["vocab_size"]
     prompts = [H.random_tokens(vocab, n, 40 + i) for i, n in enumerate((6, 19, 33, 4))]
 
-    def run(lookahead):
+    def run(lookahead, max_graphs=None):
         engine = Engine.from_folder(folders[name], "bfloat16", block_size=16, num_blocks=48, max_sequences=4,
                                     max_batch_tokens=32, prefill_chunk_size=16, decode_lookahead=lookahead)
+        if max_graphs is not None:        # so few that recorded graphs are dropped and recorded again under way
+            from sprout_lm_amd.engine.graphs import DecodeGraphs
+            engine.model._graphs = DecodeGraphs(engine.model, max_graphs=max_graphs)
         engine.add("r0", prompts[0], 40, ignore_eos=True)
         engine.add("r1", prompts[1], 22, temperature=0.7, seed=11, ignore_eos=True)
         engine.add("r2", prompts[2], 9, ignore_eos=True)
@@ -206,6 +209,8 @@ def test_lookahead_equals_synchronous_steps(folders):
     overlapped, launched = run(True)
     assert none == 0 and launched > 20
     assert overlapped == sync
+    crowded, launched = run(True, max_graphs=1)
+    assert launched > 20 and crowded == sync
 
 
 def test_lookahead_steps_give_the_tokens_of_synchronous_steps(folders):
