@@ -6,6 +6,10 @@
 Default: Qwen2.5-0.5B layer sizes (BASELINE.json configs[2]) with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
+Beside the contract's fields the line holds the prefill of 2,048 tokens, the roofline of the decode
+step, decoding at batch 1 and 64, `mixed` (the batch decoding while another prompt is prefilled 256
+tokens a step) and, with --pressure SHARE, a run in a pool too small for its requests (preemptions,
+tokens computed again, net tokens a second).
 """
 from __future__ import annotations
 
@@ -43,12 +47,13 @@ def prefill_flops(cfg, T: int) -> float:
     return linear + attention + 2.0 * V * H  # logits of the last position only
 
 
-def make_engine(cfg, dtype, batch, context, prefill_tokens):
+def make_engine(cfg, dtype, batch, context, prefill_tokens, pages=None):
     from sprout_lm_amd.engine import Engine
     pages_per_request = -(-context // 16)
-    pages = max(batch * (pages_per_request + 1), -(-prefill_tokens // 16) + 1)
+    # one request more than the batch: the prompt that is prefilled in portions beside the decoding batch
+    pages = pages or max((batch + 1) * (pages_per_request + 1), -(-prefill_tokens // 16) + 1)
     return Engine.from_config(cfg, seed=0, dtype=dtype, block_size=16, num_blocks=pages,
-                              max_sequences=batch, max_batch_tokens=max(2048, batch), prefill_chunk_size=2048,
+                              max_sequences=batch + 1, max_batch_tokens=max(2048, batch), prefill_chunk_size=2048,
                               prefix_caching=False, record_trace=False)
 
 
@@ -79,6 +84,69 @@ def measure_decode(engine, cfg, batch, context, steps, warmup):
         engine.cancel(rid)
         engine.forget(rid)
     return elapsed / steps
+
+
+def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup):
+    """`batch` requests decode while one long prompt is prefilled beside them, `chunk` tokens a step."""
+    import random
+    from dataclasses import replace
+    import torch
+    from sprout_lm_amd.engine import Engine
+    rng = random.Random(batch + chunk)
+    steps = max(1, min(steps, context // chunk - warmup - 1))
+    mixed = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk))
+    # requests that finish their prompt early decode while the others still prefill: leave them room
+    slack = -(-batch * context // engine.options.max_batch_tokens) + 2
+    ahead = steps + warmup + slack
+    for i in range(batch):
+        prompt = [rng.randrange(cfg.vocab_size) for _ in range(context - ahead - 1)]
+        mixed.add(f"m{i}", prompt, ahead + 1, ignore_eos=True)
+    while any(not r.output for r in mixed.scheduler.requests.values()):
+        mixed.step()
+    mixed.add("long", [rng.randrange(cfg.vocab_size) for _ in range((steps + warmup + 1) * chunk)], 1, ignore_eos=True)
+    for _ in range(warmup):
+        mixed.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        report = mixed.step()
+        work = {w["id"]: w for w in report.work}
+        assert len(work) == batch + 1 and work["long"]["tokens"] == chunk, "timed steps must hold the batch and a portion"
+    torch.cuda.synchronize()
+    elapsed = (time.perf_counter() - t0) / steps
+    for rid in list(mixed.scheduler.requests):
+        mixed.cancel(rid)
+        mixed.forget(rid)
+    mixed.close()
+    return {"chunk": chunk, "batch": batch, "steps": steps, "ms_per_step": round(elapsed * 1000, 4),
+            "decode_value": round(batch / elapsed, 1), "chunk_value": round(chunk / elapsed, 1)}
+
+
+def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
+    """A pool that holds `share` of what the requests need at their end: requests are preempted and
+    their keys computed again.  Net tokens a second count every token once, however often it was computed."""
+    import random
+    import torch
+    rng = random.Random(7)
+    need = batch * -(-(prompt_len + new_tokens) // 16)
+    engine = make_engine(cfg, dtype, batch, prompt_len + new_tokens, prompt_len, pages=max(int(need * share), 2))
+    for i in range(batch):
+        engine.add(f"q{i}", [rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], new_tokens, ignore_eos=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ticks = 0
+    while engine.pending:
+        engine.step()
+        ticks += 1
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    stats = engine.stats()
+    made = sum(len(engine.result(f"q{i}")["output"]) for i in range(batch))
+    assert made == batch * new_tokens, "every request must finish at full length"
+    engine.close()
+    return {"batch": batch, "prompt": prompt_len, "new_tokens": new_tokens, "pages": engine.options.num_blocks,
+            "pages_needed": need, "preemptions": stats["preemptions"], "recomputed_tokens": stats["recomputed_tokens"],
+            "steps": ticks, "seconds": round(elapsed, 3), "net_value": round(made / elapsed, 1)}
 
 
 def measure_prefill(engine, cfg, tokens, repeats=3):
@@ -113,6 +181,10 @@ def main() -> int:
     parser.add_argument("--preset", default="qwen2.5-0.5b")
     parser.add_argument("--prefill-tokens", type=int, default=2048)
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    parser.add_argument("--mixed-chunk", type=int, default=256,
+                        help="also time the batch decoding beside a prompt prefilled this many tokens a step (0: skip)")
+    parser.add_argument("--pressure", type=float, default=0.0, metavar="SHARE",
+                        help="also run the batch from 512-token prompts in a pool of this share of the pages it needs")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs.")
@@ -138,7 +210,14 @@ def main() -> int:
         for b in (1, 64):
             s = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
             points[f"decode_b{b}"] = round(b / s, 1)
+    mixed = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2) \
+        if args.mixed_chunk else None
     prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
+    engine.close()
+    pressure = None
+    if args.pressure:
+        del engine
+        pressure = measure_pressure(cfg, dtype, args.batch, 512, 256, args.pressure)
 
     read = weight_bytes_per_step(cfg, element) + kv_bytes(cfg, args.batch, args.context, element)
     achieved = read / step_s / 1e9
@@ -162,6 +241,10 @@ def main() -> int:
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},
         "points": points,
     }
+    if mixed:
+        line["mixed"] = mixed
+    if pressure:
+        line["pressure"] = pressure
     print(json.dumps(line))
     return 0
 

@@ -357,6 +357,15 @@ extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rot
   return kind == kEpiStore || kind == kEpiAccumulate || kind == kEpiStoreF32;
 }
 
+// Whether the norm prologue is faster than a norm kernel of its own before the product.  Every block
+// normalises all the rows by itself and keeps them in LDS, which costs more the wider the rows are:
+// measured at 8 tokens, QKV product with prologue against norm kernel + product: 7.0 against 7.9 us at a
+// width of 896, 11.6 against 9.4 at 1536, 22.2 against 16.2 at 3584; the gated product alike.
+extern "C" int sp_fused_norm_pays(int T, int N, int K) {
+  (void)N;
+  return fused_shape_ok(T, K, true) && K <= 1024;
+}
+
 namespace sprout {
 int gemm_decode_plain(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, int mode, void* out,
                       int T, int N, int K) {

@@ -26,6 +26,8 @@ int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w
 // [T, K] bfloat16, or, with residual != null, rmsnorm(residual [T, K] float32) * norm_w computed inside.
 // sp_fused_supported(kind, ...): kind 0..2 = plain modes of sp_gemm, 3 = sp_qkv_rope_cache, 4 = sp_gate_up_silu.
 int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm);
+// Whether folding the norm into the product (norm = 1 above) is faster than a norm kernel before it.
+int sp_fused_norm_pays(int T, int N, int K);
 int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
                    const void* w, int bias_dtype, const void* bias, int mode, void* out, int T, int N, int K);
 // q, k, v projection (+ bias), rotation of q and k, q to q_out [T, nq * hd], k and v into the paged pools.

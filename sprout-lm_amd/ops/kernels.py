@@ -262,6 +262,11 @@ def fused_supported(kind: int, T: int, N: int, K: int, hd: int = 0, rotary_dim: 
     return bool(library().sp_fused_supported(kind, T, N, K, hd, rotary_dim, int(norm)))
 
 
+def fused_norm_pays(T: int, N: int, K: int) -> bool:
+    """Whether the norm folded into the product beats a norm kernel of its own followed by the product."""
+    return bool(library().sp_fused_norm_pays(T, N, K))
+
+
 def _activations(x, residual, norm_weight, K: int, what: str):
     """Checks the two ways activations reach a fused kernel; returns (x ptr, residual ptr, norm dtype, norm ptr, T)."""
     if residual is not None:

@@ -70,7 +70,8 @@ class Attention(Mixer):
                                         self.position.rotary_dim, norm))
 
     # Folding the norm into the projection kernel (up to 16 tokens) saves a launch; the kernel asks for the
-    # residual rows before its weights, so the norm is computed while the weights are on their way.
+    # residual rows before its weights, so the norm is computed while the weights are on their way.  Every
+    # block of the kernel normalises the rows by itself, so this pays for narrow models only (the library says).
     fuse_input_norm = True
 
     def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
@@ -78,6 +79,8 @@ class Attention(Mixer):
         if not self.fuse_input_norm:
             return False
         if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, cache, True):
+            return False
+        if not ops.fused_norm_pays(T, self.w_qkv.shape[0], self.hidden):
             return False
         q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
         ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq, self.position.rotary_dim,

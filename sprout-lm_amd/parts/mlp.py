@@ -42,6 +42,8 @@ class GatedMLP(FeedForward):
             return False
         if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
             return False
+        if not ops.fused_norm_pays(T, 2 * self.inner, self.hidden):
+            return False
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
         ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=norm.w["weight"], eps=norm.eps)
         ops.gemm(act, self.w_down, residual, accumulate=True)
