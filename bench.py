@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Default: Qwen2.5-0.5B layer sizes (BASELINE.json configs[2]) with random weights, bfloat16, a batch
+Default: Qwen2.5-0.5B layer sizes with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
 Beside the contract's fields the line holds the prefill of 2,048 tokens, the roofline of the decode

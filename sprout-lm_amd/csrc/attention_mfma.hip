@@ -572,21 +572,22 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 }
 
-// Merges the chunks of one (sequence, head): grid (decode sequences, heads), one wave each; lane d sums
-// dimension d.  Everything the wave reads depends on its indices alone (empty chunks are marked as such by
-// the decode kernel), so all of it is requested at once: one trip to memory.
-template <int DT>
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ part_o,
-                                                             const float* __restrict__ part_ml,
-                                                             const int32_t* __restrict__ q_start,
-                                                             const int32_t* __restrict__ decode_seqs,
-                                                             uint16_t* __restrict__ out, int n_splits, int nq) {
+// Merges the chunks of one (sequence, head): grid (decode sequences, heads); lane d of a wave sums
+// dimension d.  Everything a wave reads depends on its indices alone (empty chunks are marked as such by
+// the decode kernel), so a wave requests 16 chunks at once: one trip to memory.  With WAVES > 1 (long
+// contexts) the waves take turns of 16 chunks each and wave 0 joins their sums through LDS.
+template <int DT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void attention_merge_kernel(const float* __restrict__ part_o,
+                                                                     const float* __restrict__ part_ml,
+                                                                     const int32_t* __restrict__ q_start,
+                                                                     const int32_t* __restrict__ decode_seqs,
+                                                                     uint16_t* __restrict__ out, int n_splits, int nq) {
   constexpr int HD = 16 * DT, PER_LANE = (HD + 63) / 64, GROUP = 16;
-  const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int di = blockIdx.x, head = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int seq = decode_seqs ? decode_seqs[di] : di;
   const size_t base = (size_t(di) * nq + head) * n_splits;
   float mx = kNoKeyYet, den = 0.f, num[PER_LANE] = {};
-  for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+  for (int s0 = wave * GROUP; s0 < n_splits; s0 += GROUP * WAVES) {
     float ms[GROUP], ls[GROUP], os[GROUP][PER_LANE];
 #pragma unroll
     for (int i = 0; i < GROUP; ++i) {
@@ -615,6 +616,28 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __rest
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) num[j] = fmaf(f, os[i][j], num[j]);
       }
+    }
+  }
+  if constexpr (WAVES > 1) {
+    __shared__ float s_mx[WAVES], s_den[WAVES], s_num[WAVES][64 * PER_LANE];
+    if (lane == 0) { s_mx[wave] = mx; s_den[wave] = den; }
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) s_num[wave][lane + 64 * j] = num[j];
+    __syncthreads();
+    if (wave > 0) return;
+    float all_max = mx;
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) all_max = fmaxf(all_max, s_mx[w]);
+    const float keep = exp2f(mx - all_max);
+    den *= keep;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) num[j] *= keep;
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      const float f = exp2f(s_mx[w] - all_max);   // a wave without keys holds zeros: its factor does not matter
+      den = fmaf(f, s_den[w], den);
+#pragma unroll
+      for (int j = 0; j < PER_LANE; ++j) num[j] = fmaf(f, s_num[w][lane + 64 * j], num[j]);
     }
   }
 #pragma unroll
@@ -702,8 +725,12 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
         n_splits, nq, nkv, page_size, num_pages, window, scale2);
     if (check_launch("sp_attention (decode)")) return 1;
     if (n_splits > 1) {
-      attention_merge_kernel<DT><<<dim3(n_decode, nq), 64, 0, s>>>(part_o, part_ml, q_start, decode_seqs,
-                                                                    (uint16_t*)out, n_splits, nq);
+      if (n_splits <= 16)
+        attention_merge_kernel<DT, 1><<<dim3(n_decode, nq), 64, 0, s>>>(part_o, part_ml, q_start, decode_seqs,
+                                                                         (uint16_t*)out, n_splits, nq);
+      else
+        attention_merge_kernel<DT, 4><<<dim3(n_decode, nq), 256, 0, s>>>(part_o, part_ml, q_start, decode_seqs,
+                                                                          (uint16_t*)out, n_splits, nq);
       if (check_launch("sp_attention (merge)")) return 1;
     }
   }

@@ -272,6 +272,23 @@ def test_attention_split_walk_finds_one_far_key(far):
     assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("nq,nkv,hd,page", [(14, 2, 64, 16), (8, 2, 128, 16), (3, 1, 32, 8)])
+@pytest.mark.parametrize("window", [None, 5000])
+def test_attention_decodes_over_long_contexts(nq, nkv, hd, page, window):
+    """One query each over thousands of keys: more chunks than one wave of the merge kernel takes in a trip
+    (several waves share them, unevenly), beside a short sequence whose chunks are nearly all empty."""
+    seqs = [(9000, 1), (100, 1), (20000, 1), (4097, 1)]
+    got, want = run_attention(torch.bfloat16, nq, nkv, hd, page, seqs, window=window, kind=0, seed=hd)
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("far", [0, 4095, 4096, 12345, 19999])
+def test_attention_decode_finds_one_far_key_among_thousands(far):
+    got, want = run_attention(torch.bfloat16, 4, 2, 64, 16, [(300, 1), (20000, 1)], kind=0, spike=(1, far), seed=far)
+    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+
+
 def test_attention_refuses_what_it_cannot_take():
     from sprout_lm_amd import ops
     q = torch.zeros(1, 4 * 16, device=DEV)
