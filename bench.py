@@ -7,7 +7,8 @@ Default: Qwen2.5-0.5B layer sizes with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
 Beside the contract's fields the line holds the prefill of 2,048 tokens, the roofline of the decode
-step, decoding at batch 1 and 64, `mixed` (the batch decoding while another prompt is prefilled 256
+step, decoding at batch 1 and 64, `step_ms` (median, 95th percentile and maximum of the timed steps as the
+host sees them), `prefill_in_portions` (the same prompt prefilled 256 and 512 tokens a step), `mixed` (the batch decoding while another prompt is prefilled 256
 tokens a step) and, with --pressure SHARE, a run in a pool too small for its requests (preemptions,
 tokens computed again, net tokens a second).
 """
@@ -75,15 +76,20 @@ def measure_decode(engine, cfg, batch, context, steps, warmup):
         engine.step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    returned = [t0]
     for _ in range(steps):
         report = engine.step()
+        returned.append(time.perf_counter())      # the step's tokens are on the host
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert len(report.work) == batch and all(w["phase"] == "decode" for w in report.work), "timed steps must decode"
     for rid in list(engine.scheduler.requests):
         engine.cancel(rid)
         engine.forget(rid)
-    return elapsed / steps
+    gaps = sorted(b - a for a, b in zip(returned, returned[1:]))
+    spread = {"median": round(gaps[len(gaps) // 2] * 1000, 4), "p95": round(gaps[min(len(gaps) - 1, int(len(gaps) * 0.95))] * 1000, 4),
+              "max": round(gaps[-1] * 1000, 4)}
+    return elapsed / steps, spread
 
 
 def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup):
@@ -149,9 +155,14 @@ def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
             "steps": ticks, "seconds": round(elapsed, 3), "net_value": round(made / elapsed, 1)}
 
 
-def measure_prefill(engine, cfg, tokens, repeats=3):
+def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
+    """Seconds from a prompt's arrival to its first token; `chunk`: the prompt goes in portions of that size."""
     import random
+    from dataclasses import replace
     import torch
+    from sprout_lm_amd.engine import Engine
+    if chunk:
+        engine = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk))
     rng = random.Random(1)
     best = None
     for r in range(repeats + 1):
@@ -204,15 +215,17 @@ def main() -> int:
     engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
     warmup = max(args.warmup, 1)
 
-    step_s = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
+    step_s, spread = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            s = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
+            s, _ = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
             points[f"decode_b{b}"] = round(b / s, 1)
     mixed = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2) \
         if args.mixed_chunk else None
     prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
+    portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 2, c), 1)
+                for c in (256, 512) if c < args.prefill_tokens and not args.no_points}
     engine.close()
     pressure = None
     if args.pressure:
@@ -239,8 +252,10 @@ def main() -> int:
                     "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / MFMA_PEAK[args.dtype], 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},
-        "points": points,
+        "points": points, "step_ms": spread,
     }
+    if portions:
+        line["prefill_in_portions"] = portions
     if mixed:
         line["mixed"] = mixed
     if pressure:
