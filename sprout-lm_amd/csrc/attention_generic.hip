@@ -11,6 +11,66 @@ namespace sprout {
 constexpr int AQ = 16;  // queries per block
 constexpr int AK = 32;  // keys per iteration
 
+// One 32-key tile of keys or values of a sequence, from the pages into registers (element i of the tile is
+// thread i % 256's i / 256-th).  All loads of a thread are requested before any is used.  Keys lie
+// [slot][head size] inside a page, values [head size][slot]: neighbouring threads take neighbouring addresses.
+// Quotient and remainder by a divisor known only at run time, for 0 <= x < 2^24, without the long
+// instruction sequence of an integer division: a float product, then one step of correction either way.
+struct Divider {
+  int d;
+  float inv;
+  __device__ __forceinline__ void set(int divisor) { d = divisor; inv = 1.0f / float(divisor); }
+  __device__ __forceinline__ void divmod(int x, int& q, int& r) const {
+    q = int(float(x) * inv);
+    r = x - q * d;
+    if (r < 0) { r += d; --q; }
+    if (r >= d) { r -= d; ++q; }
+  }
+};
+
+struct TileSource {
+  const int32_t* bt;
+  int nkv, g, hd, page_size, num_pages, k_lo, k_end;
+  Divider by_hd, by_page;
+};
+
+template <typename T, int MAXD, bool VALUES>
+__device__ __forceinline__ void load_tile(const TileSource& src, const T* __restrict__ pool, int kb, float (&tmp)[2 * MAXD]) {
+#pragma unroll
+  for (int u = 0; u < 2 * MAXD; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    float v = 0.f;
+    if (i < AK * src.hd) {
+      int jj = i % AK, d = i / AK;
+      if (!VALUES) src.by_hd.divmod(i, jj, d);
+      const int j = kb + jj;
+      if (j >= src.k_lo && j < src.k_end) {
+        int logical, slot;
+        src.by_page.divmod(j, logical, slot);
+        const int page = src.bt[logical];
+        if (page >= 0 && page < src.num_pages) {
+          const size_t base = (size_t(page) * src.nkv + src.g) * src.page_size * src.hd;
+          v = to_float(pool[base + (VALUES ? size_t(d) * src.page_size + slot : size_t(slot) * src.hd + d)]);
+        }
+      }
+    }
+    tmp[u] = v;
+  }
+}
+
+template <int MAXD, bool VALUES>
+__device__ __forceinline__ void store_tile(float* KVs, int hd, const Divider& by_hd, const float (&tmp)[2 * MAXD]) {
+#pragma unroll
+  for (int u = 0; u < 2 * MAXD; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    if (i < AK * hd) {
+      int jj = i % AK, d = i / AK;
+      if (!VALUES) by_hd.divmod(i, jj, d);
+      KVs[jj * (hd + 1) + d] = tmp[u];
+    }
+  }
+}
+
 template <typename T, int MAXD>  // MAXD = ceil(hd / 16) upper bound
 __global__ __launch_bounds__(256) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
@@ -18,10 +78,13 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
     T* __restrict__ out, int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale) {
   extern __shared__ float lds[];
-  float* Qs = lds;                         // [AQ][hd]
-  float* KVs = Qs + AQ * hd;               // [AK][hd + 1]
-  float* Ps = KVs + AK * (hd + 1);         // [AQ][AK]
+  // rows one float longer than their content: the four query rows that a wave reads at the same column
+  // then lie in different LDS banks
+  float* Qs = lds;                         // [AQ][hd + 1]
+  float* KVs = Qs + AQ * (hd + 1);         // [AK][hd + 1]
+  float* Ps = KVs + AK * (hd + 1);         // [AQ][AK + 1]
   const int kv_stride = hd + 1;
+  constexpr int PS = AK + 1;
 
   const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
   const int h = blockIdx.y;
@@ -29,35 +92,38 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   const int nvalid = min(AQ, qlen - q_off);
   if (nvalid <= 0) return;
   const int pos0 = ctx - qlen + q_off;
-  const int g = h / (nq / nkv);
-  const int32_t* bt = block_tables + size_t(seq) * max_blocks;
 
   for (int i = threadIdx.x; i < AQ * hd; i += 256) {
     const int r = i / hd, d = i % hd;
-    Qs[i] = r < nvalid ? to_float(q[size_t(qs + q_off + r) * q_stride + h * hd + d]) : 0.f;
+    Qs[r * kv_stride + d] = r < nvalid ? to_float(q[size_t(qs + q_off + r) * q_stride + h * hd + d]) : 0.f;
   }
 
   const int r = threadIdx.x / 16, c16 = threadIdx.x % 16;
   const int my_pos = pos0 + r;
-  const int k_end = pos0 + nvalid;  // one past the last visible key of the tile
-  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  TileSource src;
+  src.bt = block_tables + size_t(seq) * max_blocks;
+  src.nkv = nkv; src.g = h / (nq / nkv); src.hd = hd; src.page_size = page_size; src.num_pages = num_pages;
+  src.k_end = pos0 + nvalid;  // one past the last visible key of the tile
+  src.k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  src.by_hd.set(hd);
+  src.by_page.set(page_size);
+  const int k_lo = src.k_lo, k_end = src.k_end;
   float m = -INFINITY, l = 0.f;
   float acc[MAXD];
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) acc[i] = 0.f;
 
-  for (int kb = (k_lo / AK) * AK; kb < k_end; kb += AK) {
+  // The keys and values of a tile are requested while the tile before it is still being summed: the walk
+  // waits for memory once per tile, not once per element.
+  float ktile[2 * MAXD], vtile[2 * MAXD];
+  const int kb0 = (k_lo / AK) * AK;
+  if (kb0 < k_end) {
+    load_tile<T, MAXD, false>(src, k_pool, kb0, ktile);
+    load_tile<T, MAXD, true>(src, v_pool, kb0, vtile);
+  }
+  for (int kb = kb0; kb < k_end; kb += AK) {
     __syncthreads();  // Qs written / previous V tile consumed
-    for (int i = threadIdx.x; i < AK * hd; i += 256) {
-      const int jj = i / hd, d = i % hd, j = kb + jj;
-      float v = 0.f;
-      if (j >= k_lo && j < k_end) {
-        const int page = bt[j / page_size];
-        if (page >= 0 && page < num_pages)
-          v = to_float(k_pool[((size_t(page) * nkv + g) * page_size + j % page_size) * hd + d]);
-      }
-      KVs[jj * kv_stride + d] = v;
-    }
+    store_tile<MAXD, false>(KVs, hd, src.by_hd, ktile);
     __syncthreads();
     float s[2];
     float row_max = -INFINITY;
@@ -65,7 +131,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     for (int u = 0; u < 2; ++u) {
       const int c = c16 + 16 * u, j = kb + c;
       float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot = fmaf(Qs[r * hd + d], KVs[c * kv_stride + d], dot);
+#pragma unroll 8   // several LDS reads on their way at a time; the order of the sum stays
+      for (int d = 0; d < hd; ++d) dot = fmaf(Qs[r * kv_stride + d], KVs[c * kv_stride + d], dot);
       const bool visible = r < nvalid && j >= k_lo && j <= my_pos && (window <= 0 || my_pos - j < window);
       s[u] = visible ? dot * scale : -INFINITY;
       row_max = fmaxf(row_max, s[u]);
@@ -87,18 +154,13 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     for (int o = 8; o > 0; o >>= 1) row_sum += __shfl_xor(row_sum, o, 64);
     l = l * alpha + row_sum;
     m = m_new;
-    Ps[r * AK + c16] = p[0];
-    Ps[r * AK + c16 + 16] = p[1];
+    Ps[r * PS + c16] = p[0];
+    Ps[r * PS + c16 + 16] = p[1];
     __syncthreads();  // scores done with the K tile; Ps complete
-    for (int i = threadIdx.x; i < AK * hd; i += 256) {
-      const int jj = i / hd, d = i % hd, j = kb + jj;
-      float v = 0.f;
-      if (j >= k_lo && j < k_end) {
-        const int page = bt[j / page_size];
-        if (page >= 0 && page < num_pages)
-          v = to_float(v_pool[((size_t(page) * nkv + g) * hd + d) * page_size + j % page_size]);
-      }
-      KVs[jj * kv_stride + d] = v;
+    store_tile<MAXD, true>(KVs, hd, src.by_hd, vtile);
+    if (kb + AK < k_end) {
+      load_tile<T, MAXD, false>(src, k_pool, kb + AK, ktile);
+      load_tile<T, MAXD, true>(src, v_pool, kb + AK, vtile);
     }
     __syncthreads();
 #pragma unroll
@@ -106,7 +168,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       const int d = c16 + 16 * i;
       if (d < hd) {
         float sum = acc[i] * alpha;
-        for (int c = 0; c < AK; ++c) sum = fmaf(Ps[r * AK + c], KVs[c * kv_stride + d], sum);
+#pragma unroll
+        for (int c = 0; c < AK; ++c) sum = fmaf(Ps[r * PS + c], KVs[c * kv_stride + d], sum);
         acc[i] = sum;
       }
     }
@@ -128,7 +191,7 @@ int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const v
                              const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
                              void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
                              float scale) {
-  const size_t lds = sizeof(float) * (size_t(AQ) * hd + size_t(AK) * (hd + 1) + AQ * AK);
+  const size_t lds = sizeof(float) * (size_t(AQ + AK) * (hd + 1) + AQ * (AK + 1));
   dim3 grid(n_tiles, nq);
 #define SP_ATT(MAXD)                                                                                        \
   attention_generic_kernel<T, MAXD><<<grid, 256, lds, s>>>(                                                 \
@@ -145,6 +208,9 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale) {
+  SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
+             "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
+             max_blocks, page_size);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,

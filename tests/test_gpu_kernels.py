@@ -45,6 +45,27 @@ def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     assert np.abs(acc.cpu().numpy() - (base + want)).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("T,N,K", [(8, 151, 96), (16, 64, 1024), (7, 2050, 132), (13, 33, 4), (1, 896, 4864), (16, 1, 260)])
+@pytest.mark.parametrize("a_dtype,w_dtype", [(torch.float32, torch.float32), (torch.float32, torch.bfloat16),
+                                             (torch.bfloat16, torch.float32)])
+def test_gemm_float32_sums_for_few_tokens(T, N, K, a_dtype, w_dtype):
+    """Up to 16 tokens with K in fours: the kernel whose waves own rows of the weights (odd N, one row, all modes)."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T + N + K)
+    a, w, b = rng.standard_normal((T, K)), rng.standard_normal((N, K)) / math.sqrt(K), rng.standard_normal(N)
+    a = bf16(a) if a_dtype == torch.bfloat16 else a.astype(np.float32)
+    w = bf16(w) if w_dtype == torch.bfloat16 else w.astype(np.float32)
+    want = a.astype(np.float64) @ w.astype(np.float64).T
+    tol = 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
+    out = torch.full((T, N), float("nan"), dtype=torch.float32, device=DEV)
+    ops.gemm(t(a, a_dtype), t(w, w_dtype), out, bias=t(b.astype(np.float32)))
+    assert np.abs(out.cpu().numpy() - (want + b)).max() <= tol
+    base = rng.standard_normal((T, N)).astype(np.float32)
+    acc = t(base)
+    ops.gemm(t(a, a_dtype), t(w, w_dtype), acc, accumulate=True)
+    assert np.abs(acc.cpu().numpy() - (base + want)).max() <= tol
+
+
 def test_gemm_mixed_operand_dtypes_and_refusals():
     from sprout_lm_amd import ops
     rng = np.random.default_rng(0)
