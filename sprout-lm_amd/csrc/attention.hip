@@ -11,7 +11,7 @@ bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
 size_t attention_decode_workspace_floats(int n_decode, int nq, int hd, int max_ctx);
-size_t attention_prefill_workspace_floats(int n_tiles, int nq, int hd, int page_size, int max_tile_ctx);
+size_t attention_prefill_workspace_floats(int n_tiles, int nq, int nkv, int hd, int page_size, int max_tile_ctx);
 int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
@@ -45,7 +45,7 @@ static int64_t workspace_floats_of(int hd, int page_size, int nq, int nkv, int n
                                    int n_tiles, int max_tile_ctx) {
   const size_t decode = attention_mfma_decode_supports(nq, nkv)
                             ? attention_decode_workspace_floats(n_decode, nq, hd, max_decode_ctx) : 0;
-  return (int64_t)(decode + attention_prefill_workspace_floats(n_tiles, nq, hd, page_size, max_tile_ctx));
+  return (int64_t)(decode + attention_prefill_workspace_floats(n_tiles, nq, nkv, hd, page_size, max_tile_ctx));
 }
 
 extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,

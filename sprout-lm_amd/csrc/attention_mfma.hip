@@ -7,7 +7,8 @@
 // layout of P^T once the 32 keys of a step are numbered (group of 4, tile) instead of in order, and
 // V^T is loaded with the same numbering, so probabilities never leave registers.
 //
-// Prefill: one wave per (tile of 16 * NQT queries of one sequence, head).
+// Prefill: one wave per (tile of 16 * NQT queries of one sequence, head); with pages of a power of two,
+// the staged kernel below (keys and values through LDS, shared by several heads and split between waves).
 // Decode (one query per sequence): one block per (256 keys, key/value head, sequence); the rows of
 // the MFMA are the query heads of the group, so keys and values are read once per group.  The four
 // waves take 64 keys each and are merged in LDS; blocks are merged by a second small kernel.  (Letting
@@ -261,17 +262,18 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ prefill, staged
-// One block of four waves per (tile of 16 * NQT queries, head).  The keys are walked in stages of 128
-// that the block copies into LDS; wave w takes keys 32 w .. 32 w + 31 of every stage with a running
-// softmax of its own, and the four waves are merged in LDS at the end.  Against one wave walking all
-// keys this cuts the chain of dependent steps by four, and several blocks per CU hide the copy.
+// One block per (tile of 16 * NQT queries, HPB heads of one key/value head): a team of four waves per head.
+// The keys are walked in stages of 128 that the block copies into LDS once for all its teams; wave w of
+// a team takes keys 32 w .. 32 w + 31 of every stage with a running softmax of its own, and the four waves
+// are merged in LDS at the end.  Against one wave walking all keys this cuts the chain of dependent steps
+// by four; sharing a stage between heads cuts the traffic from L2, which bounds the kernel.
 // The sequence's page numbers are copied to LDS first, so that a fetch is one trip to memory.
 // Needs pages of 8, 16, 32, ... tokens (a power of two).
 constexpr int kStageKeys = 128;
 constexpr int kMaxTableLds = 2048;    // page numbers held in LDS; longer tables are read from memory
 
-template <int DT, int NQT>
-__global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
+template <int DT, int NQT, int HPB, bool AHEAD>
+__global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
@@ -279,12 +281,13 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     float* __restrict__ part_ml, int n_splits, int stages_per_split, int nq, int nkv, int page_shift, int num_pages,
     int window, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
+  constexpr int THREADS = 256 * HPB;
   constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
   constexpr int VP = kStageKeys + 8;          // value row pitch: the stage's keys + 16 bytes of padding
   constexpr int KCHUNKS = kStageKeys * (HD / 8);      // 16-byte pieces of the stage's keys ...
   const int page_size = 1 << page_shift, page_mask = page_size - 1;   // pages are a power of two of tokens
   constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
-  constexpr int PER_THREAD = CHUNKS / 256;
+  constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
   constexpr int STAGE_BYTES = (kStageKeys * KP + HD * VP) * 2;
   constexpr int MERGE_BYTES = 4 * 16 * NQT * (HD + 2) * 4;
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
@@ -295,8 +298,12 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
   // tiles are listed in order of position; the last ones walk the most keys, so they start first
   const int tile = gridDim.x - 1 - blockIdx.x;
   const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
-  const int h = blockIdx.y, g = h / (nq / nkv);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  // the block's HPB heads belong to one key/value head: its four-wave teams share the staged keys and values
+  const int G = nq / nkv, teams_per_group = (G + HPB - 1) / HPB;
+  const int g = blockIdx.y / teams_per_group, first_head = (blockIdx.y % teams_per_group) * HPB;
+  const int team = threadIdx.x >> 8, wave = (threadIdx.x >> 6) & 3, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const bool has_head = first_head + team < G;          // the last block of a group may have teams to spare
+  const int h = g * G + min(first_head + team, G - 1);
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
   const int nvalid = min(16 * NQT, qlen - q_off);
   if (nvalid <= 0) return;
@@ -308,10 +315,10 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
   const int first_page = k_lo >> page_shift, n_pages = (k_hi >> page_shift) - first_page + 1;
   const bool table_in_lds = n_pages <= kMaxTableLds;
   if (table_in_lds)
-    for (int i = threadIdx.x; i < n_pages; i += 256) s_table[i] = table[first_page + i];
+    for (int i = threadIdx.x; i < n_pages; i += THREADS) s_table[i] = table[first_page + i];
   // where the page numbers are read from is a compile-time choice of the caller (a run-time choice
   // between LDS and memory would turn every read into a flat load)
-  auto page_at = [&](int key, auto in_lds) {
+  auto page_at = [&](int key, auto in_lds) __attribute__((always_inline)) {
     int page;
     if constexpr (decltype(in_lds)::value) page = s_table[(key >> page_shift) - first_page];
     else page = table[key >> page_shift];
@@ -345,43 +352,52 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     range_lo = max(range_lo, split * stages_per_split * kStageKeys);
     if (split + 1 < n_splits) range_hi = min(range_hi, (split + 1) * stages_per_split * kStageKeys - 1);
   }
-  for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
-    __syncthreads();   // the page numbers are in LDS; the last stage has been used
+  // A stage travels memory -> registers -> LDS.  With AHEAD the registers are asked for the next stage as soon
+  // as this one lies in LDS, so its trip to memory runs while this one is being used (the registers stay
+  // occupied meanwhile: worth it where there are few per thread).
+  uint4 stage[PER_THREAD];
+  auto fetch_from = [&](int key0, auto in_lds) __attribute__((always_inline)) {
     const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
-    uint4 stage[PER_THREAD];
-    auto fetch = [&](auto in_lds) {
-#pragma unroll
-      for (int u = 0; u < PER_THREAD; ++u) {
-        const int i = threadIdx.x + 256 * u;
-        if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
-          const int r = i / (HD / 8), c = i % (HD / 8);
-          int key = key0 + r;
-          if (!interior) key = min(max(key, k_lo), k_hi);
-          stage[u] = ldg128(kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
-        } else {                                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
-          const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
-          int kb = key0 + 8 * c;
-          if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
-          stage[u] = ldg128(vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
-        }
-      }
-    };
-    if (table_in_lds) fetch(std::true_type{});
-    else fetch(std::false_type{});
 #pragma unroll
     for (int u = 0; u < PER_THREAD; ++u) {
-      const int i = threadIdx.x + 256 * u;
+      const int i = threadIdx.x + THREADS * u;
+      if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
+        const int r = i / (HD / 8), c = i % (HD / 8);
+        int key = key0 + r;
+        if (!interior) key = min(max(key, k_lo), k_hi);
+        stage[u] = ldg128(kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
+      } else if (i < CHUNKS) {                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
+        const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
+        int kb = key0 + 8 * c;
+        if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+        stage[u] = ldg128(vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
+      }
+    }
+  };
+  auto fetch = [&](int key0) __attribute__((always_inline)) {
+    if (table_in_lds) fetch_from(key0, std::true_type{});
+    else fetch_from(key0, std::false_type{});
+  };
+  __syncthreads();   // the page numbers are in LDS
+  if (AHEAD && range_lo <= range_hi) fetch(range_lo);
+  for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
+    if (!AHEAD) fetch(key0);
+    __syncthreads();   // the last stage has been used
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) {
+      const int i = threadIdx.x + THREADS * u;
       if (i < KCHUNKS) {
         const int r = i / (HD / 8), c = i % (HD / 8);
         *reinterpret_cast<uint4*>(&ks[r * KP + 8 * c]) = stage[u];
-      } else {
+      } else if (i < CHUNKS) {
         const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
         *reinterpret_cast<uint4*>(&vs[d * VP + 8 * c]) = stage[u];
       }
     }
     __syncthreads();
+    if (AHEAD && key0 + kStageKeys <= range_hi) fetch(key0 + kStageKeys);
     const int wkey = key0 + 32 * wave;         // this wave's 32 keys of the stage
-    if (wkey <= k_hi && wkey + 32 > k_lo) {
+    if (has_head && wkey <= k_hi && wkey + 32 > k_lo) {
       KVStep<DT> r;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -400,47 +416,54 @@ __global__ __launch_bounds__(256) void attention_prefill_staged_kernel(
     }
   }
 
-  // merge the four waves: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
-  __syncthreads();
+  // merge the four waves of each team in turn: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
   float* mg = reinterpret_cast<float*>(smem);
   constexpr int MP = HD + 2;
+#pragma unroll 1
+  for (int turn = 0; turn < HPB; ++turn) {
+    if (first_head + turn >= G) break;
+    __syncthreads();   // the last stage, or the team before, has been read
+    if (team == turn) {
 #pragma unroll
-  for (int qt = 0; qt < NQT; ++qt) {
-    float l = lsum[qt];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    float* row = mg + (size_t(wave) * 16 * NQT + 16 * qt + lr) * MP;
+      for (int qt = 0; qt < NQT; ++qt) {
+        float l = lsum[qt];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        float* row = mg + (size_t(wave) * 16 * NQT + 16 * qt + lr) * MP;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) row[16 * dt + 4 * lj + r4] = o[qt][dt][r4];
-    if (lj == 0) { row[HD] = m[qt]; row[HD + 1] = l; }
-  }
-  __syncthreads();
-  for (int i = threadIdx.x; i < nvalid * (HD / 4); i += 256) {
-    const int row = i / (HD / 4), d = 4 * (i % (HD / 4));
-    float mx = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) mx = fmaxf(mx, mg[(size_t(w) * 16 * NQT + row) * MP + HD]);
-    float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float* src = mg + (size_t(w) * 16 * NQT + row) * MP;
-      const float f = exp2f(src[HD] - mx);
-      den += f * src[HD + 1];
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) num[r4] += f * src[d + r4];
+          for (int r4 = 0; r4 < 4; ++r4) row[16 * dt + 4 * lj + r4] = o[qt][dt][r4];
+        if (lj == 0) { row[HD] = m[qt]; row[HD + 1] = l; }
+      }
     }
-    if (n_splits > 1) {
-      // partial result of this block's keys: sums against the maximum mx, for the merge kernel
-      const size_t slot = ((size_t(tile) * (16 * NQT) + row) * nq + h) * n_splits + split;
-      *reinterpret_cast<float4*>(part_o + slot * HD + d) = make_float4(num[0], num[1], num[2], num[3]);
-      if (d == 0) *reinterpret_cast<float2*>(part_ml + 2 * slot) = make_float2(mx, den);
-      continue;
+    __syncthreads();
+    const int head = g * G + first_head + turn;
+    for (int i = threadIdx.x; i < nvalid * (HD / 4); i += THREADS) {
+      const int row = i / (HD / 4), d = 4 * (i % (HD / 4));
+      float mx = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) mx = fmaxf(mx, mg[(size_t(w) * 16 * NQT + row) * MP + HD]);
+      float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const float* src = mg + (size_t(w) * 16 * NQT + row) * MP;
+        const float f = exp2f(src[HD] - mx);
+        den += f * src[HD + 1];
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) num[r4] += f * src[d + r4];
+      }
+      if (n_splits > 1) {
+        // partial result of this block's keys: sums against the maximum mx, for the merge kernel
+        const size_t slot = ((size_t(tile) * (16 * NQT) + row) * nq + head) * n_splits + split;
+        *reinterpret_cast<float4*>(part_o + slot * HD + d) = make_float4(num[0], num[1], num[2], num[3]);
+        if (d == 0) *reinterpret_cast<float2*>(part_ml + 2 * slot) = make_float2(mx, den);
+        continue;
+      }
+      const float inv = den > 0.f ? 1.0f / den : 0.f;
+      uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + head * HD + d;
+      *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
     }
-    const float inv = den > 0.f ? 1.0f / den : 0.f;
-    uint16_t* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + h * HD + d;
-    *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
   }
 }
 
@@ -663,15 +686,28 @@ static bool staged_prefill(int page_size) { return page_size >= 8 && (page_size 
 
 // Blocks per tile and head along the keys.  A step with few queries over a long context (a portion of a long
 // prompt) has few tiles, each with a long walk: the walk is cut until the grid fills the chip about three times.
-int attention_prefill_splits(int n_tiles, int nq, int page_size, int max_tile_ctx) {
-  if (!staged_prefill(page_size)) return 1;
-  const int blocks = n_tiles * nq, stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
-  if (blocks <= 0 || blocks >= 512 || stages <= 4) return 1;
-  return max(1, min(min((768 + blocks - 1) / blocks, stages / 2), kMaxPrefillSplits));
+// Heads of one key/value head that a block of the staged kernel works on (a team of four waves each): they
+// share every stage of keys and values, which the kernel otherwise fetches from L2 once per head -- and that
+// traffic, not the matrix cores, is what bounds it (measured ~8.5 TB/s at every size).  Four teams where the
+// registers of 16 waves suffice (head sizes up to 64), two above that; three teams were slower than two.
+// A portion of 2,048 tokens at a context of 32,768: 835 -> 472 us (14 heads of 64), 2,350 -> 1,910 us (28 of 128).
+static int heads_per_block(int nq, int nkv, int hd) {
+  const int G = nq / nkv;
+  if (hd > 64) return min(G, 2);
+  return G >= 3 ? 4 : G;
 }
 
-size_t attention_prefill_workspace_floats(int n_tiles, int nq, int hd, int page_size, int max_tile_ctx) {
-  const size_t splits = attention_prefill_splits(n_tiles, nq, page_size, max_tile_ctx);
+int attention_prefill_splits(int n_tiles, int nq, int nkv, int hd, int page_size, int max_tile_ctx) {
+  if (!staged_prefill(page_size)) return 1;
+  const int hpb = heads_per_block(nq, nkv, hd), G = nq / nkv;
+  const int blocks = n_tiles * nkv * ((G + hpb - 1) / hpb), stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
+  const int enough = 2048 / (4 * hpb);          // blocks that hold 2,048 waves: two rounds of the chip's CUs
+  if (blocks <= 0 || blocks >= enough || stages <= 4) return 1;
+  return max(1, min(min((enough * 3 / 2 + blocks - 1) / blocks, stages / 2), kMaxPrefillSplits));
+}
+
+size_t attention_prefill_workspace_floats(int n_tiles, int nq, int nkv, int hd, int page_size, int max_tile_ctx) {
+  const size_t splits = attention_prefill_splits(n_tiles, nq, nkv, hd, page_size, max_tile_ctx);
   return splits <= 1 ? 0 : size_t(n_tiles) * 32 * nq * splits * (hd + 2);
 }
 
@@ -696,14 +732,27 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
     if (staged_prefill(page_size)) {
       int page_shift = 0;
       while ((1 << page_shift) < page_size) ++page_shift;
-      const int splits = attention_prefill_splits(n_tiles, nq, page_size, max_tile_ctx);
+      const int splits = attention_prefill_splits(n_tiles, nq, nkv, HD, page_size, max_tile_ctx);
       const int stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
       const int per_split = (stages + splits - 1) / splits;
       float* part_o = splits > 1 ? prefill_ws : nullptr;
       float* part_ml = splits > 1 ? prefill_ws + size_t(n_tiles) * 16 * NQT * nq * splits * HD : nullptr;
-      attention_prefill_staged_kernel<DT, NQT><<<dim3(n_tiles, nq, splits), 256, 0, s>>>(
-          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, part_o,
-          part_ml, splits, per_split, nq, nkv, page_shift, num_pages, window, scale2);
+      const int hpb = heads_per_block(nq, nkv, HD);
+      const dim3 grid(n_tiles, nkv * ((nq / nkv + hpb - 1) / hpb), splits);
+#define SP_STAGED(HPB, AHEAD)                                                                                   \
+  attention_prefill_staged_kernel<DT, NQT, HPB, AHEAD><<<grid, 256 * HPB, 0, s>>>(                              \
+      qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, part_o,   \
+      part_ml, splits, per_split, nq, nkv, page_shift, num_pages, window, scale2)
+      // the next stage is requested ahead where a thread holds few pieces of it, or has registers to spare
+      if constexpr (DT <= 4) {
+        if (hpb == 4) SP_STAGED(4, true);
+        else if (hpb == 2) SP_STAGED(2, false);
+        else SP_STAGED(1, false);
+      } else {
+        if (hpb == 2) SP_STAGED(2, true);
+        else SP_STAGED(1, false);
+      }
+#undef SP_STAGED
       if (splits > 1) {
         if (check_launch("sp_attention (prefill)")) return 1;
         attention_prefill_merge_kernel<DT, NQT><<<dim3(n_tiles * (16 * NQT / 4), nq), 256, 0, s>>>(
