@@ -262,9 +262,9 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
 }
 
 // ------------------------------------------------------------------------------------------ prefill, staged
-// One block per (tile of 16 * NQT queries, HPB heads of one key/value head): a team of four waves per head.
+// One block per (tile of 16 * NQT queries, HPB heads of one key/value head): a team of WPT waves per head.
 // The keys are walked in stages of 128 that the block copies into LDS once for all its teams; wave w of
-// a team takes keys 32 w .. 32 w + 31 of every stage with a running softmax of its own, and the four waves
+// a team takes its share of every stage (128 / WPT keys, 32 at a time) with a running softmax of its own, and the waves
 // are merged in LDS at the end.  Against one wave walking all keys this cuts the chain of dependent steps
 // by four; sharing a stage between heads cuts the traffic from L2, which bounds the kernel.
 // The sequence's page numbers are copied to LDS first, so that a fetch is one trip to memory.
@@ -272,8 +272,8 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
 constexpr int kStageKeys = 128;
 constexpr int kMaxTableLds = 2048;    // page numbers held in LDS; longer tables are read from memory
 
-template <int DT, int NQT, int HPB, bool AHEAD>
-__global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
+template <int DT, int NQT, int HPB, int WPT, bool AHEAD>
+__global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
@@ -281,7 +281,8 @@ __global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
     float* __restrict__ part_ml, int n_splits, int stages_per_split, int nq, int nkv, int page_shift, int num_pages,
     int window, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
-  constexpr int THREADS = 256 * HPB;
+  constexpr int THREADS = 64 * WPT * HPB;
+  constexpr int WAVE_KEYS = kStageKeys / WPT;          // keys of a stage that one wave of a team takes
   constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
   constexpr int VP = kStageKeys + 8;          // value row pitch: the stage's keys + 16 bytes of padding
   constexpr int KCHUNKS = kStageKeys * (HD / 8);      // 16-byte pieces of the stage's keys ...
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
   constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
   constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
   constexpr int STAGE_BYTES = (kStageKeys * KP + HD * VP) * 2;
-  constexpr int MERGE_BYTES = 4 * 16 * NQT * (HD + 2) * 4;
+  constexpr int MERGE_BYTES = WPT * 16 * NQT * (HD + 2) * 4;
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
   __shared__ int32_t s_table[kMaxTableLds];
   uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
@@ -301,7 +302,7 @@ __global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
   // the block's HPB heads belong to one key/value head: its four-wave teams share the staged keys and values
   const int G = nq / nkv, teams_per_group = (G + HPB - 1) / HPB;
   const int g = blockIdx.y / teams_per_group, first_head = (blockIdx.y % teams_per_group) * HPB;
-  const int team = threadIdx.x >> 8, wave = (threadIdx.x >> 6) & 3, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int team = threadIdx.x / (64 * WPT), wave = (threadIdx.x >> 6) % WPT, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const bool has_head = first_head + team < G;          // the last block of a group may have teams to spare
   const int h = g * G + min(first_head + team, G - 1);
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
@@ -396,27 +397,31 @@ __global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
     }
     __syncthreads();
     if (AHEAD && key0 + kStageKeys <= range_hi) fetch(key0 + kStageKeys);
-    const int wkey = key0 + 32 * wave;         // this wave's 32 keys of the stage
-    if (has_head && wkey <= k_hi && wkey + 32 > k_lo) {
-      KVStep<DT> r;
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int c = 0; c < HC; ++c) {
-          const int d0 = 32 * c + 8 * lj;
-          r.ka[kt][c] = d0 < HD ? as_bf16x8(*reinterpret_cast<const uint4*>(&ks[(32 * wave + 16 * kt + lr) * KP + d0]))
-                                : as_bf16x8(make_uint4(0, 0, 0, 0));
-        }
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
+    for (int sub = 0; sub < WAVE_KEYS / 32; ++sub) {
+      const int skey = WAVE_KEYS * wave + 32 * sub;     // this wave's keys of the stage, 32 at a time
+      const int wkey = key0 + skey;
+      if (has_head && wkey <= k_hi && wkey + 32 > k_lo) {
+        KVStep<DT> r;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
-          r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[(16 * dt + lr) * VP + 32 * wave + 16 * kt + 4 * lj]);
-      attend_step<DT, NQT>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+#pragma unroll
+          for (int c = 0; c < HC; ++c) {
+            const int d0 = 32 * c + 8 * lj;
+            r.ka[kt][c] = d0 < HD ? as_bf16x8(*reinterpret_cast<const uint4*>(&ks[(skey + 16 * kt + lr) * KP + d0]))
+                                  : as_bf16x8(make_uint4(0, 0, 0, 0));
+          }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)
+            r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[(16 * dt + lr) * VP + skey + 16 * kt + 4 * lj]);
+        attend_step<DT, NQT>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+      }
     }
   }
 
-  // merge the four waves of each team in turn: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
+  // merge the waves of each team in turn: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
   float* mg = reinterpret_cast<float*>(smem);
   constexpr int MP = HD + 2;
 #pragma unroll 1
@@ -443,10 +448,10 @@ __global__ __launch_bounds__(256 * HPB) void attention_prefill_staged_kernel(
       const int row = i / (HD / 4), d = 4 * (i % (HD / 4));
       float mx = -INFINITY;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) mx = fmaxf(mx, mg[(size_t(w) * 16 * NQT + row) * MP + HD]);
+      for (int w = 0; w < WPT; ++w) mx = fmaxf(mx, mg[(size_t(w) * 16 * NQT + row) * MP + HD]);
       float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
+      for (int w = 0; w < WPT; ++w) {
         const float* src = mg + (size_t(w) * 16 * NQT + row) * MP;
         const float f = exp2f(src[HD] - mx);
         den += f * src[HD + 1];
@@ -686,22 +691,26 @@ static bool staged_prefill(int page_size) { return page_size >= 8 && (page_size 
 
 // Blocks per tile and head along the keys.  A step with few queries over a long context (a portion of a long
 // prompt) has few tiles, each with a long walk: the walk is cut until the grid fills the chip about three times.
-// Heads of one key/value head that a block of the staged kernel works on (a team of four waves each): they
-// share every stage of keys and values, which the kernel otherwise fetches from L2 once per head -- and that
-// traffic, not the matrix cores, is what bounds it (measured ~8.5 TB/s at every size).  Four teams where the
-// registers of 16 waves suffice (head sizes up to 64), two above that; three teams were slower than two.
-// A portion of 2,048 tokens at a context of 32,768: 835 -> 472 us (14 heads of 64), 2,350 -> 1,910 us (28 of 128).
-static int heads_per_block(int nq, int nkv, int hd) {
+// Teams of a block of the staged kernel: HPB heads of one key/value head, WPT waves each.  The heads share
+// every stage of keys and values, which the kernel otherwise fetches from L2 once per head -- and that
+// traffic, not the matrix cores, is what bounds it (measured ~8.5 TB/s at every size).  Head sizes up to 64:
+// four teams of four waves.  Above that the registers of 16 waves do not suffice: four teams of two waves
+// (each wave then takes 64 keys of a stage).  Three teams were slower than two or four at every size.
+// A portion of 2,048 tokens at a context of 32,768: 835 -> 472 us (14 heads of 64), 2,350 -> 1,470 us (28 of 128).
+struct StagedShape { int hpb, wpt; bool ahead; };
+static StagedShape staged_shape(int nq, int nkv, int hd) {
   const int G = nq / nkv;
-  if (hd > 64) return min(G, 2);
-  return G >= 3 ? 4 : G;
+  if (G <= 1) return {1, 4, false};
+  if (G == 2) return {2, 4, hd > 64};
+  return hd > 64 ? StagedShape{4, 2, false} : StagedShape{4, 4, true};
 }
 
 int attention_prefill_splits(int n_tiles, int nq, int nkv, int hd, int page_size, int max_tile_ctx) {
   if (!staged_prefill(page_size)) return 1;
-  const int hpb = heads_per_block(nq, nkv, hd), G = nq / nkv;
-  const int blocks = n_tiles * nkv * ((G + hpb - 1) / hpb), stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
-  const int enough = 2048 / (4 * hpb);          // blocks that hold 2,048 waves: two rounds of the chip's CUs
+  const StagedShape shape = staged_shape(nq, nkv, hd);
+  const int G = nq / nkv;
+  const int blocks = n_tiles * nkv * ((G + shape.hpb - 1) / shape.hpb), stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
+  const int enough = 2048 / (shape.wpt * shape.hpb);   // blocks that hold 2,048 waves: two rounds of the chip's CUs
   if (blocks <= 0 || blocks >= enough || stages <= 4) return 1;
   return max(1, min(min((enough * 3 / 2 + blocks - 1) / blocks, stages / 2), kMaxPrefillSplits));
 }
@@ -737,21 +746,16 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
       const int per_split = (stages + splits - 1) / splits;
       float* part_o = splits > 1 ? prefill_ws : nullptr;
       float* part_ml = splits > 1 ? prefill_ws + size_t(n_tiles) * 16 * NQT * nq * splits * HD : nullptr;
-      const int hpb = heads_per_block(nq, nkv, HD);
-      const dim3 grid(n_tiles, nkv * ((nq / nkv + hpb - 1) / hpb), splits);
-#define SP_STAGED(HPB, AHEAD)                                                                                   \
-  attention_prefill_staged_kernel<DT, NQT, HPB, AHEAD><<<grid, 256 * HPB, 0, s>>>(                              \
+      const StagedShape shape = staged_shape(nq, nkv, HD);
+      const dim3 grid(n_tiles, nkv * ((nq / nkv + shape.hpb - 1) / shape.hpb), splits);
+#define SP_STAGED(HPB, WPT, AHEAD)                                                                              \
+  attention_prefill_staged_kernel<DT, NQT, HPB, WPT, AHEAD><<<grid, 64 * WPT * HPB, 0, s>>>(                    \
       qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, part_o,   \
       part_ml, splits, per_split, nq, nkv, page_shift, num_pages, window, scale2)
-      // the next stage is requested ahead where a thread holds few pieces of it, or has registers to spare
-      if constexpr (DT <= 4) {
-        if (hpb == 4) SP_STAGED(4, true);
-        else if (hpb == 2) SP_STAGED(2, false);
-        else SP_STAGED(1, false);
-      } else {
-        if (hpb == 2) SP_STAGED(2, true);
-        else SP_STAGED(1, false);
-      }
+      // the same cases as staged_shape()
+      if (shape.hpb == 1) SP_STAGED(1, 4, false);
+      else if (shape.hpb == 2) { if constexpr (DT > 4) SP_STAGED(2, 4, true); else SP_STAGED(2, 4, false); }
+      else { if constexpr (DT > 4) SP_STAGED(4, 2, false); else SP_STAGED(4, 4, true); }
 #undef SP_STAGED
       if (splits > 1) {
         if (check_launch("sp_attention (prefill)")) return 1;
