@@ -25,12 +25,13 @@ def requests_for(name, lengths, seed=100):
     return {f"r{i}": H.random_tokens(vocab, n, seed + i) for i, n in enumerate(lengths)}
 
 
-def replay_in_process(folder, name, dtype, trace, max_tokens):
+def replay_in_process(folder, name, dtype, trace, max_tokens, page=None, num_blocks=None):
     """Drive the engine's TraceSession directly; returns per step the logits rows (or None)."""
     from sprout_lm_amd.engine import ModelRunner
     from sprout_lm_amd.engine.trace import TraceSession
-    page = H.PAGE_SIZE[name]
-    runner = ModelRunner.from_folder(folder, dtype, block_size=page, num_blocks=-(-max_tokens // page), max_sequences=8)
+    page = page or H.PAGE_SIZE[name]
+    runner = ModelRunner.from_folder(folder, dtype, block_size=page, num_blocks=num_blocks or -(-max_tokens // page),
+                                     max_sequences=8)
     session = TraceSession(runner)
     out = []
     for record in trace.steps:
@@ -78,6 +79,18 @@ def test_replay_family(folders, name, dtype, family):
     results = replay_in_process(folders[name], name, dtype, trace, pool)
     worst = check(folders[name], dtype, requests, trace, results)
     print(f"{family} {name} {dtype}: {len(trace.steps)} steps, worst error {worst:.3e}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("A", 12), ("B", 20), ("C", 6)])
+def test_replay_with_pages_of_odd_sizes(folders, name, dtype, page):
+    """Pages whose size is no power of two (and, at 6, no multiple of 4): other attention kernels take over.
+    The pool holds the four longest requests and no page more, so pages are used again."""
+    requests = requests_for(name, LENGTHS[name], seed=300)
+    trace = traces.mixed(requests, seed=11)
+    pages = sum(sorted(-(-len(t) // page) for t in requests.values())[-4:])
+    results = replay_in_process(folders[name], name, dtype, trace, None, page=page, num_blocks=pages)
+    check(folders[name], dtype, requests, trace, results)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
