@@ -8,7 +8,8 @@ of 8 requests at a context of 4,096 tokens.  A step is one decode step of the wh
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
 Beside the contract's fields the line holds the prefill of 2,048 tokens, the roofline of the decode
 step, decoding at batch 1 and 64, `step_ms` (median, 95th percentile and maximum of the timed steps as the
-host sees them), `prefill_in_portions` (the same prompt prefilled 256 and 512 tokens a step), `mixed` (the batch decoding while another prompt is prefilled 256
+host sees them, and `host`: the part of a step that the host spends planning and launching, which the
+look-ahead hides behind the GPU's work), `prefill_in_portions` (the same prompt prefilled 256 and 512 tokens a step), `mixed` (the batch decoding while another prompt is prefilled 256
 tokens a step) and, with --pressure SHARE, a run in a pool too small for its requests (preemptions,
 tokens computed again, net tokens a second).
 """
@@ -74,6 +75,17 @@ def measure_decode(engine, cfg, batch, context, steps, warmup):
         engine.step()
     for _ in range(warmup - 1):
         engine.step()
+    # the host's own share of a step: what is not spent waiting for the step's tokens
+    waited = [0.0]
+    finish = engine.model.finish_decode
+
+    def timed_finish(pending):
+        t = time.perf_counter()
+        tokens = finish(pending)
+        waited[0] += time.perf_counter() - t
+        return tokens
+
+    engine.model.finish_decode = timed_finish
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     returned = [t0]
@@ -82,13 +94,14 @@ def measure_decode(engine, cfg, batch, context, steps, warmup):
         returned.append(time.perf_counter())      # the step's tokens are on the host
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    del engine.model.finish_decode
     assert len(report.work) == batch and all(w["phase"] == "decode" for w in report.work), "timed steps must decode"
     for rid in list(engine.scheduler.requests):
         engine.cancel(rid)
         engine.forget(rid)
     gaps = sorted(b - a for a, b in zip(returned, returned[1:]))
     spread = {"median": round(gaps[len(gaps) // 2] * 1000, 4), "p95": round(gaps[min(len(gaps) - 1, int(len(gaps) * 0.95))] * 1000, 4),
-              "max": round(gaps[-1] * 1000, 4)}
+              "max": round(gaps[-1] * 1000, 4), "host": round((elapsed - waited[0]) / steps * 1000, 4)}
     return elapsed / steps, spread
 
 
