@@ -373,7 +373,9 @@ def _normed(res, w, eps):
 
 
 @pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64])
-@pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4)])
+# the last two: few rows with a long K, which eight waves of a block share instead of four
+@pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4),
+                                              (4, 2, 128, 3584, 16), (3, 1, 64, 2120, 8)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     from sprout_lm_amd import ops
@@ -419,7 +421,7 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
 
 
 @pytest.mark.parametrize("T", [1, 8, 16, 33, 64, 65, 200, 513])
-@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72)])
+@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
