@@ -289,3 +289,65 @@ def test_real_layer_sizes_both_dtypes(tmp_path):
             else:
                 assert err.max() <= H.tolerance(dtype, want[pos]), f"position {pos}: {err.max():.3e}"
         seq.release()
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_scheduling_never_changes_generation(folders, block):
+    """Random page sizes, pools down to one request's need, budgets, portions, arrivals, cancellations,
+    prefix sharing, look-ahead on and off and as few as one recorded graph: every request generates what it
+    generates alone (float32, where no near tie can fall the other way), and no page is lost."""
+    import random
+    from sprout_lm_amd.engine import Engine
+    from sprout_lm_amd.engine.graphs import DecodeGraphs
+
+    def alone(name, r):
+        engine = Engine.from_folder(folders[name], "float32", block_size=16, num_blocks=16, max_sequences=1,
+                                    max_batch_tokens=256, prefill_chunk_size=256, prefix_caching=False,
+                                    decode_lookahead=False)
+        engine.add("s", r["prompt"], r["max_new"], temperature=r["temperature"], seed=r["seed"], stop_token_ids=r["stops"])
+        while engine.pending:
+            engine.step()
+        output = engine.result("s")["output"]
+        engine.close()
+        return output
+
+    for case in range(8 * block, 8 * block + 8):
+        rng = random.Random(4000 + case)
+        name = rng.choice("AB")
+        vocab = H.CONFIGS[name]["vocab_size"]
+        page = rng.choice([4, 8, 12, 16, 32])
+        shared = H.random_tokens(vocab, rng.randint(0, 40), case)
+        requests = []
+        for i in range(rng.randint(2, 6)):
+            prompt = (shared[:rng.randint(0, len(shared))] + H.random_tokens(vocab, rng.randint(1, 60), 7 * case + i))[:90]
+            requests.append(dict(id=f"r{i}", prompt=prompt, max_new=rng.randint(1, 20), temperature=rng.choice([0.0, 0.0, 0.8]),
+                                 seed=rng.randrange(1 << 30), arrive=rng.randint(0, 10),
+                                 stops=rng.choice([None, None, [rng.randrange(vocab), rng.randrange(vocab)]]),
+                                 cancel=rng.choice([None, None, None, rng.randint(1, 25)])))
+        need = max(-(-(len(r["prompt"]) + r["max_new"]) // page) for r in requests)
+        num_blocks = rng.randint(need, need * rng.randint(1, 4))
+        engine = Engine.from_folder(folders[name], "float32", block_size=page, num_blocks=num_blocks,
+                                    max_sequences=rng.randint(1, 6), max_batch_tokens=rng.choice([8, 16, 48, 256]),
+                                    prefill_chunk_size=rng.choice([2, 5, 16, 64]), prefix_caching=rng.random() < 0.6,
+                                    decode_lookahead=rng.random() < 0.7)
+        engine.model._graphs = DecodeGraphs(engine.model, max_graphs=rng.choice([1, 2, 32]))
+        tick, cancelled, waiting = 0, set(), sorted(requests, key=lambda r: r["arrive"])
+        while waiting or engine.pending:
+            while waiting and waiting[0]["arrive"] <= tick:
+                r = waiting.pop(0)
+                engine.add(r["id"], r["prompt"], r["max_new"], temperature=r["temperature"], seed=r["seed"],
+                           stop_token_ids=r["stops"])
+            for r in requests:
+                known = engine.scheduler.requests.get(r["id"])
+                if r["cancel"] == tick and known is not None and known.status in ("waiting", "running"):
+                    engine.cancel(r["id"])
+                    cancelled.add(r["id"])
+            engine.step()
+            tick += 1
+            assert tick < 2000, f"case {case}: no progress"
+        for r in requests:
+            got, want = engine.result(r["id"])["output"], alone(name, r)
+            assert got == (want[:len(got)] if r["id"] in cancelled else want), f"case {case}, request {r['id']}"
+        engine.cache.clear_prefixes()
+        assert engine.cache.free_pages() == [num_blocks], f"case {case}: pages were lost"
+        engine.close()
