@@ -61,9 +61,12 @@ __global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, in
 // One block per token.  Pair (d, d + rotary_dim/2) of each q and k head turns by
 // positions[t] * inv_freq[d]; k (rotated) and v go to the pools.  Keys lie [page][group][slot][dim]; values lie
 // [page][group][dim][slot], so that the keys of one dimension are contiguous for the P.V matrix product.
+// inv_freq_tail (float32 storage only, may be null): what the float32 table lost of the float64 one.  With it
+// the angle and its sine and cosine are computed in float64: a float32 angle is off by up to position * 6e-8,
+// which at positions in the thousands is more than all other roundings of the float32 path together.
 template <typename T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
-                                  const float* __restrict__ inv_freq, int rotary_dim,
+                                  const float* __restrict__ inv_freq, const float* __restrict__ inv_freq_tail, int rotary_dim,
                                   const int32_t* __restrict__ slot_mapping, T* __restrict__ k_pool,
                                   T* __restrict__ v_pool, int nq, int nkv, int hd, int page_size) {
   const int t = blockIdx.x;
@@ -79,7 +82,14 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict
   for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
     const int head = i / half, d = i % half;
     float sn, cs;
-    sincosf(pos * inv_freq[d], &sn, &cs);
+    if (inv_freq_tail) {
+      double sn64, cs64;
+      sincos(double(positions[t]) * (double(inv_freq[d]) + double(inv_freq_tail[d])), &sn64, &cs64);
+      sn = float(sn64);
+      cs = float(cs64);
+    } else {
+      sincosf(pos * inv_freq[d], &sn, &cs);
+    }
     T* h = row + size_t(head) * hd;
     const float a = to_float(h[d]), b = to_float(h[d + half]);
     const T ra = from_float<T>(a * cs - b * sn), rb = from_float<T>(b * cs + a * sn);
@@ -190,7 +200,8 @@ extern "C" int sp_cast(void* stream, int src_dtype, const void* src, int dst_dty
 }
 
 extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions,
-                             const float* inv_freq, int rotary_dim, const int32_t* slot_mapping, void* k_pool,
+                             const float* inv_freq, const float* inv_freq_tail, int rotary_dim,
+                             const int32_t* slot_mapping, void* k_pool,
                              void* v_pool, int T, int nq, int nkv, int hd, int page_size, int num_pages) {
   SP_REQUIRE(T >= 0 && nq > 0 && nkv >= 0 && hd > 0, "sp_rope_cache: bad sizes");
   SP_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
@@ -200,10 +211,10 @@ extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* 
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == kF32)
-    rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, positions, inv_freq, rotary_dim, slot_mapping,
+    rope_cache_kernel<float><<<T, 256, 0, s>>>((float*)qkv, positions, inv_freq, inv_freq_tail, rotary_dim, slot_mapping,
                                                (float*)k_pool, (float*)v_pool, nq, nkv, hd, page_size);
   else if (dtype == kBF16)
-    rope_cache_kernel<bf16_t><<<T, 256, 0, s>>>((bf16_t*)qkv, positions, inv_freq, rotary_dim, slot_mapping,
+    rope_cache_kernel<bf16_t><<<T, 256, 0, s>>>((bf16_t*)qkv, positions, inv_freq, nullptr, rotary_dim, slot_mapping,
                                                 (bf16_t*)k_pool, (bf16_t*)v_pool, nq, nkv, hd, page_size);
   else
     SP_REQUIRE(false, "sp_rope_cache: unsupported dtype %d", dtype);

@@ -44,7 +44,7 @@ int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm
 // (= page * page_size + offset; negative: not written).  nkv == 0: only q is rotated.
 // The key pool is [pages][nkv][page_size][hd], the value pool [pages][nkv][hd][page_size], of `dtype`.
 int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, const float* inv_freq,
-                  int rotary_dim, const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int nq,
+                  const float* inv_freq_tail, int rotary_dim, const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int nq,
                   int nkv, int hd, int page_size, int num_pages);
 
 // Causal attention of a mixed batch over the paged pools.

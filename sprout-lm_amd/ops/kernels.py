@@ -124,9 +124,10 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: torch.Tensor
 
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int, nq: int, nkv: int,
                hd: int, slot_mapping: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
-               v_pool: torch.Tensor | None = None) -> None:
+               v_pool: torch.Tensor | None = None, inv_freq_tail: torch.Tensor | None = None) -> None:
     """Rotate q and k heads of qkv in place and write k, v into the pools (keys [pages, nkv, page, hd], values
-    [pages, nkv, hd, page])."""
+    [pages, nkv, hd, page]).  `inv_freq_tail` (float32 qkv only): the float64 table minus `inv_freq`; with it
+    angles, sines and cosines are computed in float64."""
     _gpu(qkv, "qkv")
     T = qkv.shape[0]
     if qkv.shape[1] != (nq + 2 * nkv) * hd:
@@ -135,12 +136,16 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tenso
     _gpu(inv_freq, "inv_freq")
     if inv_freq.dtype != torch.float32 or inv_freq.numel() < max(rotary_dim // 2, 0):
         raise KernelError("rope_cache: inv_freq must hold rotary_dim / 2 float32 values")
+    if inv_freq_tail is not None:
+        _gpu(inv_freq_tail, "inv_freq_tail")
+        if inv_freq_tail.dtype != torch.float32 or inv_freq_tail.numel() != inv_freq.numel():
+            raise KernelError("rope_cache: inv_freq_tail must be float32 and as long as inv_freq")
     page_size = num_pages = 0
     if nkv:
         _ints(slot_mapping, T, "slot_mapping")
         num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, qkv.dtype, "rope_cache")
     check(library().sp_rope_cache(_stream(), _code(qkv, "qkv"), qkv.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(),
-                                  rotary_dim, _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), T, nq, nkv, hd, page_size,
+                                  _ptr(inv_freq_tail), rotary_dim, _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), T, nq, nkv, hd, page_size,
                                   num_pages))
 
 

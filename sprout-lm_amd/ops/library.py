@@ -20,8 +20,8 @@ def _declare(lib):
         "sp_embed": [c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int],
         "sp_rmsnorm": [c_void, c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int],
         "sp_gemm": [c_void, c_int, c_void, c_int, c_void, c_int, c_void, c_int, c_int, c_void, c_int, c_int, c_int],
-        "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int,
-                          c_int, c_int, c_int],
+        "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int,
+                          c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
                          c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_float, c_int],

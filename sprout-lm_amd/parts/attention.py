@@ -117,5 +117,6 @@ class Attention(Mixer):
         ops.gemm(h, w, qkv, bias=b)
         ops.rope_cache(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim, self.heads, nkv,
                        self.head_dim, cache.slot_mapping if nkv else None, cache.k if nkv else None,
-                       cache.v if nkv else None)
+                       cache.v if nkv else None,
+                       inv_freq_tail=getattr(self.position, "inv_freq_tail", None) if qkv.dtype == torch.float32 else None)
         self._attend(ctx, qkv, width, residual, cache)

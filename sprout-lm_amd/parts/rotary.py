@@ -11,7 +11,10 @@ class NeoxRotary(PositionEncoding):
     """Pair (d, d + rotary_dim/2) of a head turns by position * theta^(-2d / rotary_dim).
 
     The table of inverse frequencies is computed in float64 and kept in float32; angles, sines
-    and cosines are float32 in the kernel.
+    and cosines are float32 in the kernel.  For float32 models the part also keeps what the float32
+    table lost (`inv_freq_tail`), and the kernel computes angle, sine and cosine in float64: a float32
+    angle is off by up to position * 6e-8, more than every other rounding of that path together once
+    positions reach the thousands.
     """
 
     graph_safe = True
@@ -22,10 +25,14 @@ class NeoxRotary(PositionEncoding):
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {head_dim}.")
         self.inv_freq = None
+        self.inv_freq_tail = None
 
     def prepare(self, device, dtype):
         d = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
-        self.inv_freq = (float(self.theta) ** (-d / self.rotary_dim)).to(torch.float32).to(device)
+        exact = float(self.theta) ** (-d / self.rotary_dim)
+        self.inv_freq = exact.to(torch.float32).to(device)
+        if dtype == torch.float32:
+            self.inv_freq_tail = (exact - exact.to(torch.float32).to(torch.float64)).to(torch.float32).to(device)
 
 
 @register_part("position", "none")

@@ -365,6 +365,27 @@ def test_sampling_greedy_ties_nonfinite_and_temperature():
     assert (out == 0).float().mean().item() > 0.99
 
 
+@pytest.mark.parametrize("hd,rotary,theta", [(48, 48, 50000.0), (64, 64, 1e6), (32, 16, 10000.0)])
+def test_rope_with_float64_angles_at_far_positions(hd, rotary, theta):
+    """Float32 storage with the tail of the frequency table: angles are exact to float64 rounding, so positions
+    in the tens of thousands turn as exactly as position 1 (a float32 angle would be off by 1e-3 there)."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(hd)
+    T, nq = 9, 3
+    x = rng.standard_normal((T, nq * hd)).astype(np.float32)
+    pos = np.array([0, 1, 999, 4097, 12345, 20000, 31999, 32767, 100000])
+    exact = theta ** (-2.0 * np.arange(rotary // 2) / rotary)
+    head = torch.tensor(exact, dtype=torch.float32)
+    tail = torch.tensor(exact - head.double().numpy(), dtype=torch.float32)
+    with_tail, without = t(x), t(x)
+    ops.rope_cache(with_tail, torch.tensor(pos, dtype=torch.int32, device=DEV), head.to(DEV), rotary, nq, 0, hd,
+                   inv_freq_tail=tail.to(DEV))
+    ops.rope_cache(without, torch.tensor(pos, dtype=torch.int32, device=DEV), head.to(DEV), rotary, nq, 0, hd)
+    want = plain_rope(x, pos, hd, rotary, theta)
+    assert np.abs(with_tail.cpu().numpy() - want).max() <= 1e-6
+    assert np.abs(without.cpu().numpy() - want).max() > 1e-5    # what the tail is for
+
+
 # ---- decode-sized fused kernels --------------------------------------------------------------------
 
 def _normed(res, w, eps):

@@ -39,6 +39,35 @@ def test_whole_prompts_match_plain(folders, name, dtype):
     assert runner.cache.free_pages() == [64]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_far_positions_match_plain(folders, dtype):
+    """Configuration C up to position 1,000, in portions and then token by token.  The error must not grow with
+    the position: rotation angles of the float32 path are computed in float64 (a float32 angle is off by
+    position * 6e-8, which at these positions is more than the whole bound)."""
+    from sprout_lm_amd.engine import StepEntry
+    name, n = "C", 1000
+    runner = make_runner(folders[name], name, dtype, num_blocks=64)
+    tokens = H.random_tokens(H.CONFIGS[name]["vocab_size"], n, 61)
+    want = H.plain_logits(folders[name], dtype, tokens)
+    seq = runner.cache.create()
+    fed, worst_near, worst_far = 0, 0.0, 0.0
+    for size in [300, 257, 300, 127] + [1] * 16:
+        assert runner.cache.reserve(seq, fed + size)
+        got = runner.step([StepEntry(seq, tokens[fed:fed + size], list(range(size)))]).cpu().numpy()
+        for i in range(size):
+            share = float(np.abs(got[i] - want[fed + i]).max()) / H.tolerance(dtype, want[fed + i])
+            assert share <= 1.0, f"position {fed + i}: {share:.2f} of the bound"
+            if fed + i < 200:
+                worst_near = max(worst_near, share)
+            elif fed + i >= 800:
+                worst_far = max(worst_far, share)
+        fed += size
+    assert fed == n
+    seq.release()
+    print(f"{dtype}: worst share of the bound below position 200: {worst_near:.2f}, from 800 on: {worst_far:.2f}")
+    assert worst_far <= max(2 * worst_near, 0.5)
+
+
 def test_reference_fixture_logits_fp32(reference_fixture):
     """The reference's own fixture: logits computed by an independent library (test/qwen.test.ts:15-46).
 
