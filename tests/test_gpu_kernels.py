@@ -290,6 +290,17 @@ def test_attention_few_queries_over_a_long_context(dtype, kind, nq, nkv, hd, pag
     assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("nq,nkv,hd,page", [(8, 8, 32, 8), (16, 8, 32, 16), (14, 2, 64, 16), (24, 8, 80, 32)])
+@pytest.mark.parametrize("seqs,window", [([(2080, 2080)], None), ([(1500, 1000), (1100, 1100), (40, 40)], None),
+                                         ([(1500, 1000), (1100, 1100), (40, 40)], 300)])
+def test_attention_long_prompts_whose_tiles_are_taken_in_pairs(nq, nkv, hd, page, seqs, window):
+    """Enough tiles that the bfloat16 prefill kernel gives each block a long walk and a short one (an odd
+    number of tiles: the middle one is taken once), with one, two, four and three query heads per group."""
+    got, want = run_attention(torch.bfloat16, nq, nkv, hd, page, seqs, window=window, kind=0, seed=nq)
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+
+
 @pytest.mark.parametrize("far", [0, 127, 128, 1000, 2047, 2999])
 def test_attention_split_walk_finds_one_far_key(far):
     got, want = run_attention(torch.bfloat16, 4, 2, 64, 16, [(3000, 1), (3000, 9)], kind=0, spike=(1, far), seed=far)
