@@ -17,6 +17,12 @@ int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_poo
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
                    int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq, int nkv, int hd,
                    int page_size, int num_pages, int window, float scale);
+bool attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx, int hidden);
+int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                  const int32_t* block_tables, int max_blocks, const int32_t* q_start,
+                                  const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
+                                  float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
+                                  int hd, int page_size, int num_pages, int window, float scale);
 }  // namespace sprout
 
 using namespace sprout;
@@ -87,4 +93,37 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   return attention_mfma(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
                         n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, workspace, out, nq, nkv, hd,
                         page_size, num_pages, window, scale);
+}
+
+// Whether sp_attention_decode_project takes a step of n_decode one-query sequences (bfloat16 only).
+extern "C" int sp_attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode,
+                                                 int max_decode_ctx, int hidden) {
+  return nq > 0 && nkv > 0 && nq % nkv == 0 &&
+         attention_decode_project_takes(hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden);
+}
+
+// A step of one-query sequences only, bfloat16: attention and the output projection w_o [hidden, nq * hd]
+// (bfloat16, no bias) in one: residual[q_start[seq], :] += attention(seq) . w_o^T, residual float32
+// [rows, hidden].  The workspace is the one of sp_attention for the same step.
+extern "C" int sp_attention_decode_project(void* stream, const void* q, int q_stride, const void* k_pool,
+                                           const void* v_pool, const int32_t* block_tables, int max_blocks,
+                                           const int32_t* q_start, const int32_t* ctx_len, const int32_t* decode_seqs,
+                                           int n_decode, int max_decode_ctx, float* workspace, int64_t workspace_floats,
+                                           const void* w_o, float* residual, int hidden, int nq, int nkv, int hd,
+                                           int page_size, int num_pages, int window, float scale) {
+  SP_REQUIRE(sp_attention_decode_project_takes(hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden),
+             "sp_attention_decode_project: hd=%d page=%d heads=%d/%d sequences=%d context=%d hidden=%d is not taken",
+             hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden);
+  SP_REQUIRE(q && k_pool && v_pool && block_tables && q_start && ctx_len && w_o && residual,
+             "sp_attention_decode_project: null operand");
+  SP_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0 && max_decode_ctx <= max_blocks * page_size,
+             "sp_attention_decode_project: decode context %d exceeds the block tables", max_decode_ctx);
+  SP_REQUIRE(q_stride >= nq * hd, "sp_attention_decode_project: q row stride %d is smaller than %d", q_stride, nq * hd);
+  const int64_t need = workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, 0, 0);
+  SP_REQUIRE(workspace && workspace_floats >= need,
+             "sp_attention_decode_project: workspace of %lld floats is smaller than the %lld needed",
+             (long long)workspace_floats, (long long)need);
+  return attention_mfma_decode_project((hipStream_t)stream, q, q_stride, k_pool, v_pool, block_tables, max_blocks,
+                                       q_start, ctx_len, decode_seqs, n_decode, max_decode_ctx, workspace, w_o, residual,
+                                       hidden, nq, nkv, hd, page_size, num_pages, window, scale);
 }

@@ -684,6 +684,106 @@ __global__ __launch_bounds__(64 * WAVES) void attention_merge_kernel(const float
   }
 }
 
+// Merge of the chunks of one head, folded into that head's share of the output projection (decode steps):
+//   residual[row(di), n] += sum_d merged[di, head, d] * w_o[n, head * HD + d]
+// grid (heads, blocks of 64 TPW rows of w_o).  A block merges its head's chunks for every decode sequence
+// (as attention_merge_kernel does, rounded to bfloat16 as the attention output is) into LDS, while its rows
+// of w_o, requested first, are on their way; each wave then multiplies TPW tiles of 16 rows and adds them
+// into the float32 residual.  Against merge kernel + projection kernel this saves a launch and the trip of
+// the attention output through memory.
+template <int DT, int TN, int TPW>
+__global__ __launch_bounds__(256) void attention_merge_project_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ decode_seqs, const uint16_t* __restrict__ w_o, float* __restrict__ residual,
+    int n_decode, int n_splits, int nq, int hidden) {
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2, XP = HD + 8, GROUP = 8;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[16 * TN][XP];
+  __shared__ int32_t s_row[16 * TN];
+  const int head = blockIdx.x, n_begin = blockIdx.y * (64 * TPW);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+
+  uint4 wa[TPW][HC];
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) {
+    const int n = min(n_begin + 16 * (wave + 4 * i) + lr, hidden - 1);
+    const uint16_t* wrow = w_o + size_t(n) * (size_t(nq) * HD) + head * HD;
+#pragma unroll
+    for (int c = 0; c < HC; ++c) {
+      const int d0 = 32 * c + 8 * lj;
+      wa[i][c] = d0 < HD ? ldg128(wrow + d0) : make_uint4(0, 0, 0, 0);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // merge: HD / 4 threads per decode sequence, four dimensions each
+  constexpr int TPR = HD / 4, ROWS = 256 / TPR;
+  for (int r0 = 0; r0 < 16 * TN; r0 += ROWS) {
+    const int di = r0 + int(threadIdx.x) / TPR, d = 4 * (int(threadIdx.x) % TPR);
+    if (int(threadIdx.x) >= ROWS * TPR || di >= 16 * TN) continue;
+    float mx = kNoKeyYet, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
+    if (di < n_decode) {
+      const size_t base = (size_t(di) * nq + head) * n_splits;
+      for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+        float2 ml[GROUP];
+        float4 os[GROUP];
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) {
+          const bool in = s0 + i < n_splits;
+          ml[i] = in ? *reinterpret_cast<const float2*>(part_ml + 2 * (base + s0 + i)) : make_float2(kNoKeyYet, 0.f);
+          // an empty chunk left nothing in part_o: its sum is zero, and what is read here is not used
+          os[i] = in ? *reinterpret_cast<const float4*>(part_o + (base + s0 + i) * HD + d) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float group_max = mx;
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) group_max = fmaxf(group_max, ml[i].x);
+        const float keep = exp2f(mx - group_max);
+        mx = group_max;
+        den *= keep;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) num[r] *= keep;
+#pragma unroll
+        for (int i = 0; i < GROUP; ++i) {
+          if (ml[i].y > 0.f) {
+            const float f = exp2f(ml[i].x - mx);
+            den = fmaf(f, ml[i].y, den);
+            num[0] = fmaf(f, os[i].x, num[0]);
+            num[1] = fmaf(f, os[i].y, num[1]);
+            num[2] = fmaf(f, os[i].z, num[2]);
+            num[3] = fmaf(f, os[i].w, num[3]);
+          }
+        }
+      }
+      if (d == 0) s_row[di] = q_start[decode_seqs ? decode_seqs[di] : di];
+    }
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    *reinterpret_cast<uint2*>(&xs[di][d]) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) {
+    const int n0 = n_begin + 16 * (wave + 4 * i);
+    if (n0 >= hidden) continue;
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+      if (16 * tn >= n_decode) continue;
+      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < HC; ++c) {
+        const int d0 = 32 * c + 8 * lj;
+        const uint4 b = d0 < HD ? *reinterpret_cast<const uint4*>(&xs[16 * tn + lr][d0]) : make_uint4(0, 0, 0, 0);
+        acc = mfma16(as_bf16x8(wa[i][c]), as_bf16x8(b), acc);
+      }
+      const int t = 16 * tn + lr;                 // lane holds rows n0 + 4 lj + 0..3 of w_o for token t
+      if (t >= n_decode) continue;
+      float* dst = residual + size_t(s_row[t]) * hidden + n0 + 4 * lj;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + 4 * lj + r < hidden) unsafeAtomicAdd(dst + r, acc[r]);
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------ host side
 bool attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
   const int dt = hd / 16;
@@ -836,6 +936,60 @@ int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_poo
   }
 #undef SP_MFMA
   set_error("sp_attention: no matrix-core kernel for head size %d", hd);
+  return 1;
+}
+
+// Decode steps whose chunks' merge is folded into the output projection.  Worth it where the merged partial
+// results, which every block of a head reads again, stay small beside the rows of w_o.
+bool attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx, int hidden) {
+  if (!attention_mfma_supports(hd, page_size, nq, nkv) || !attention_mfma_decode_supports(nq, nkv)) return false;
+  const int n_splits = (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk;
+  // (measured at 14 heads of 64, a width of 896, contexts of 4,096: 8 sequences 7,930 -> 8,250 tokens/s, 64
+  // sequences 31,700 -> 27,800: every block of a head reads all its sequences' chunks)
+  return n_decode >= 1 && n_decode <= 64 && n_splits > 1 && n_decode * n_splits <= 256 && hidden >= 16 && hidden <= 2048;
+}
+
+template <int DT>
+static int launch_decode_project(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                 const int32_t* block_tables, int max_blocks, const int32_t* q_start,
+                                 const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
+                                 float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
+                                 int page_size, int num_pages, int window, float scale) {
+  constexpr int HD = 16 * DT;
+  const int n_splits = (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk;
+  float* part_o = workspace;
+  float* part_ml = workspace + size_t(n_decode) * nq * n_splits * HD;
+  attention_decode_kernel<DT><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+      (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
+      ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
+  if (check_launch("sp_attention_decode_project (decode)")) return 1;
+  const dim3 grid(nq, (hidden + 63) / 64);
+#define SP_PROJECT(TN)                                                                                          \
+  attention_merge_project_kernel<DT, TN, 1><<<grid, 256, 0, s>>>(part_o, part_ml, q_start, decode_seqs,         \
+                                                                  (const uint16_t*)w_o, residual, n_decode,       \
+                                                                  n_splits, nq, hidden)
+  if (n_decode <= 16) SP_PROJECT(1);
+  else if (n_decode <= 32) SP_PROJECT(2);
+  else SP_PROJECT(4);
+#undef SP_PROJECT
+  return check_launch("sp_attention_decode_project (merge and projection)");
+}
+
+int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                  const int32_t* block_tables, int max_blocks, const int32_t* q_start,
+                                  const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
+                                  float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
+                                  int hd, int page_size, int num_pages, int window, float scale) {
+#define SP_MFMA(DT)                                                                                              \
+  case DT:                                                                                                       \
+    return launch_decode_project<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, \
+                                     decode_seqs, n_decode, max_decode_ctx, workspace, w_o, residual, hidden,    \
+                                     nq, nkv, page_size, num_pages, window, scale)
+  switch (hd / 16) {
+    SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
+  }
+#undef SP_MFMA
+  set_error("sp_attention_decode_project: no matrix-core kernel for head size %d", hd);
   return 1;
 }
 

@@ -69,6 +69,19 @@ int sp_attention(void* stream, int dtype, const void* q, int q_stride, const voi
                  int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size, int num_pages,
                  int window, float scale, int kernel_kind);
 
+// A step of one-query sequences only (bfloat16): attention with the output projection folded into the merge
+// of the key chunks: residual[q_start[seq], :] += attention(seq) . w_o^T with w_o [hidden, nq * hd] bfloat16
+// and residual float32 [rows, hidden].  sp_attention_decode_project_takes says whether a step is taken
+// (several chunks of keys, at most 64 sequences, a narrow model); the workspace is sp_attention's for the step.
+int sp_attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx,
+                                      int hidden);
+int sp_attention_decode_project(void* stream, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                                const int32_t* block_tables, int max_blocks, const int32_t* q_start,
+                                const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
+                                float* workspace, int64_t workspace_floats, const void* w_o, float* residual,
+                                int hidden, int nq, int nkv, int hd, int page_size, int num_pages, int window,
+                                float scale);
+
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i]
 int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I);
 

@@ -200,10 +200,14 @@ def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: in
 
 def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
               batch: AttentionBatch, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
-              workspace=None, kind: int = 0) -> None:
+              workspace=None, kind: int = 0, project=None) -> bool:
     """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h).
 
     `workspace(n)` must return a float32 device tensor of at least n elements (default: a new one).
+    `project`: (w_o [hidden, nq * hd], residual float32 [T, hidden]) of an output projection without bias
+    that may be folded in: where the kernels take the step that way (one-query sequences only, bfloat16),
+    residual += attention . w_o^T, `out` is left untouched and True is returned; otherwise False, and the
+    projection is the caller's.
     """
     for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
@@ -243,6 +247,21 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         ws = workspace(need) if workspace is not None else torch.empty(need, dtype=torch.float32, device=q.device)
         if ws.dtype != torch.float32 or ws.numel() < need:
             raise KernelError("attention: workspace too small")
+    if project is not None and kind == 0 and n_tiles == 0 and n_decode and need and q.dtype == torch.bfloat16:
+        w_o, residual = project
+        hidden = w_o.shape[0]
+        if (w_o.dtype == torch.bfloat16 and w_o.is_contiguous() and tuple(w_o.shape) == (hidden, nq * hd)
+                and residual.dtype == torch.float32 and residual.is_contiguous() and residual.dim() == 2
+                and residual.shape[1] == hidden and residual.shape[0] >= T
+                and library().sp_attention_decode_project_takes(hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden)):
+            _gpu(w_o, "w_o"); _gpu(residual, "residual")
+            check(library().sp_attention_decode_project(
+                _stream(), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
+                block_tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
+                _ptr(decode) if decode is not None else None, n_decode, max_decode_ctx, _ptr(ws), need, w_o.data_ptr(),
+                residual.data_ptr(), hidden, nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
+                float(scale)))
+            return True
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
                                  batch.q_len.data_ptr(), batch.ctx_len.data_ptr(), _ptr(tiles) if n_tiles else None,
@@ -250,6 +269,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
                                  float(scale), kind))
+    return False
 
 
 def feed_tokens(tokens: torch.Tensor, previous: torch.Tensor, source: torch.Tensor, vocab: int) -> None:

@@ -92,10 +92,13 @@ class Attention(Mixer):
     def _attend(self, ctx, q, q_stride, residual, cache):
         T = q.shape[0]
         attn = ctx.buffer("attn", (T, self.heads * self.head_dim), ctx.act_dtype)
-        ops.attention(q, q_stride, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads, self.kv_heads,
-                      self.head_dim, self.window, self.scale,
-                      workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
-                      kind=ctx.attention_kind)
+        # a step of decoded tokens only: the kernels may fold the projection into the merge of the key chunks
+        project = (self.w_o, residual) if self.b_o is None else None
+        if ops.attention(q, q_stride, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads,
+                         self.kv_heads, self.head_dim, self.window, self.scale,
+                         workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
+                         kind=ctx.attention_kind, project=project):
+            return
         ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)
 
     def forward(self, ctx, h, residual, cache):

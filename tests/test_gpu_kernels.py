@@ -194,8 +194,11 @@ def plain_attention(q, keys, values, nq, nkv, hd, first_pos, window, scale):
     return out
 
 
-def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=None, seed=0):
-    """seqs: list of (ctx_len, q_len).  Pages are scattered over the pool in random order."""
+def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=None, seed=0, hidden=None):
+    """seqs: list of (ctx_len, q_len).  Pages are scattered over the pool in random order.
+
+    hidden: an output projection [hidden, nq * hd] is given along, which the kernels must fold in; what is
+    compared is then what was added to a float32 residual."""
     from sprout_lm_amd import ops
     rng = np.random.default_rng(seed)
     n_pages = sum(-(-c // page) for c, _ in seqs) + 3
@@ -234,12 +237,22 @@ def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=Non
     out = torch.full((T, nq * hd), float("nan"), dtype=dtype, device=DEV)
     scale = 1 / math.sqrt(hd)
     batch = ops.AttentionBatch.build([ql for _, ql in seqs], [c for c, _ in seqs], DEV)
-    ops.attention(t(q, dtype), nq * hd, t(kp, dtype), t(vp.transpose(0, 1, 3, 2), dtype), t(tables, torch.int32), batch,
-                  out, nq, nkv, hd, window, scale, kind=kind)
-    got = out.float().cpu().numpy()
+    project = None
+    if hidden:
+        w_o = bf16(rng.standard_normal((hidden, nq * hd)).astype(np.float32) / math.sqrt(nq * hd))
+        before = rng.standard_normal((T, hidden)).astype(np.float32)
+        project = (t(w_o, dtype), t(before, torch.float32))
+    folded = ops.attention(t(q, dtype), nq * hd, t(kp, dtype), t(vp.transpose(0, 1, 3, 2), dtype), t(tables, torch.int32),
+                           batch, out, nq, nkv, hd, window, scale, kind=kind, project=project)
     want = np.concatenate([plain_attention(q[starts[s]:starts[s] + ql].astype(np.float64), keys[s].astype(np.float64),
                                            values[s].astype(np.float64), nq, nkv, hd, c - ql, window, scale)
                            for s, (c, ql) in enumerate(seqs)])
+    if hidden:
+        assert folded, "the projection was not folded in"
+        got = project[1].cpu().numpy().astype(np.float64) - before
+        return got, bf16(want.astype(np.float32)).astype(np.float64) @ w_o.astype(np.float64).T
+    assert not folded
+    got = out.float().cpu().numpy()
     return got, want
 
 
@@ -314,6 +327,21 @@ def test_attention_decodes_over_long_contexts(nq, nkv, hd, page, window):
     (several waves share them, unevenly), beside a short sequence whose chunks are nearly all empty."""
     seqs = [(9000, 1), (100, 1), (20000, 1), (4097, 1)]
     got, want = run_attention(torch.bfloat16, nq, nkv, hd, page, seqs, window=window, kind=0, seed=hd)
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("nq,nkv,hd,page,hidden", [(14, 2, 64, 16, 896), (3, 1, 32, 8, 100), (4, 4, 128, 16, 264),
+                                                   (5, 1, 96, 4, 17), (6, 2, 48, 16, 1000), (2, 1, 16, 32, 64)])
+@pytest.mark.parametrize("contexts", [[300], [257, 4096, 1000, 513, 300, 2049, 777, 4000], list(range(258, 258 + 40 * 37, 37)),
+                                      [1, 5000, 256, 255]])
+@pytest.mark.parametrize("window", [None, 700])
+def test_attention_decode_with_the_projection_folded_in(nq, nkv, hd, page, hidden, contexts, window):
+    """Decoded tokens only, contexts of several chunks of keys: the merge of the chunks multiplies by the
+    output projection and adds into the residual.  1, 8, 40 and 4 sequences (one, three and one tiles of 16
+    tokens), among them contexts of a single chunk and of one key, whose other chunks are empty."""
+    got, want = run_attention(torch.bfloat16, nq, nkv, hd, page, [(c, 1) for c in contexts], window=window, kind=0,
+                              seed=hidden, hidden=hidden)
     assert not np.isnan(got).any()
     assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
 
