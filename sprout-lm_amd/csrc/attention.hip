@@ -15,8 +15,8 @@ size_t attention_prefill_workspace_floats(int n_tiles, int nq, int nkv, int hd, 
 int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
-                   int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq, int nkv, int hd,
-                   int page_size, int num_pages, int window, float scale);
+                   int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace, void* out, int nq, int nkv,
+                   int hd, int page_size, int num_pages, int window, float scale);
 bool attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx, int hidden);
 int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                   const int32_t* block_tables, int max_blocks, const int32_t* q_start,
@@ -63,7 +63,7 @@ extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_siz
 extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                             const void* v_pool, const int32_t* block_tables, int max_blocks,
                             const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
-                            const int32_t* tiles, int n_tiles, int tile_q, int max_tile_ctx,
+                            const int32_t* tiles, int n_tiles, int tile_q, int max_tile_ctx, int mean_tile_walk,
                             const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
                             int64_t workspace_floats, void* out, int nq,
                             int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind) {
@@ -91,8 +91,9 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
              "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
              (long long)need);
   return attention_mfma(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
-                        n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, workspace, out, nq, nkv, hd,
-                        page_size, num_pages, window, scale);
+                        n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx,
+                        mean_tile_walk > 0 ? mean_tile_walk : max_tile_ctx, workspace, out,
+                        nq, nkv, hd, page_size, num_pages, window, scale);
 }
 
 // Whether sp_attention_decode_project takes a step of n_decode one-query sequences (bfloat16 only).

@@ -813,17 +813,21 @@ static StagedShape staged_shape(int nq, int nkv, int hd) {
   return hd > 64 ? StagedShape{4, 2, false} : StagedShape{4, 4, true};
 }
 // Whether the tiles are taken in pairs (a long walk and a short one per block), and with which teams.
-static bool staged_paired(int n_tiles, int nq, int nkv, int hd, int splits, StagedShape* shape) {
-  // Measured (one causal prompt, kernel time in us, unpaired -> paired): 14 heads of 64 in 2 groups, 2,048 tokens
-  // 39.6 -> 33.4, 4,096 tokens 104 -> 86; 28 heads of 128 in 4 groups, 2,048 tokens 112 -> 73, 16,384 tokens
-  // 3,240 -> 3,140; 16 heads of 64 in 8 groups, 2,048 tokens 57 -> 34.  With fewer pairs than CUs, halving the
-  // number of blocks costs more than the even walks gain.
+static bool staged_paired(int n_tiles, int nq, int nkv, int hd, int splits, int max_tile_ctx, int mean_tile_walk,
+                          StagedShape* shape) {
+  // Measured (one causal prompt, kernel time in us, unpaired -> paired): 28 heads of 128 in 4 groups, 2,048 tokens
+  // 112 -> 73, 16,384 tokens 3,240 -> 3,140, a portion of 2,048 after 8,192 earlier tokens 519 -> 503; 16 heads of
+  // 64 in 8 groups, 2,048 tokens 57 -> 34.  With fewer pairs than CUs, halving the number of blocks costs more
+  // than the even walks gain.
   const int G = nq / nkv;
   if (splits > 1 || n_tiles < 2) return false;
   const int pairs = (n_tiles + 1) / 2;
   if (pairs * nkv * ((G + shape->hpb - 1) / shape->hpb) >= 256) return true;
-  // teams of 16 waves: two heads a block instead of four make twice the blocks
-  if (hd <= 64 && shape->hpb == 4 && pairs * nkv * ((G + 1) / 2) >= 256) {
+  // Teams of 16 waves: two heads a block instead of four make twice the blocks, but fetch every stage twice
+  // as often.  That pays only while the walks differ much: the longest at least 1.5 times the mean, as in a prompt's
+  // first portion (14 heads of 64 in 2 groups, 2,048 tokens: 39.5 -> 33.5 after no earlier tokens, 55.7 -> 55.7
+  // after 1,024, 72 -> 79 after 2,048).
+  if (hd <= 64 && shape->hpb == 4 && pairs * nkv * ((G + 1) / 2) >= 256 && 3 * mean_tile_walk <= 2 * max_tile_ctx) {
     *shape = StagedShape{2, 4, true};
     return true;
   }
@@ -854,8 +858,8 @@ template <int DT>
 static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                        const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                        const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs,
-                       int n_decode, int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq,
-                       int nkv, int page_size, int num_pages, int window, float scale) {
+                       int n_decode, int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace,
+                       void* out, int nq, int nkv, int page_size, int num_pages, int window, float scale) {
   constexpr int HD = 16 * DT;
   constexpr int NQT = 2;
   const float scale2 = scale * kLog2e;
@@ -872,7 +876,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
       float* part_o = splits > 1 ? prefill_ws : nullptr;
       float* part_ml = splits > 1 ? prefill_ws + size_t(n_tiles) * 16 * NQT * nq * splits * HD : nullptr;
       StagedShape shape = staged_shape(nq, nkv, HD);
-      const bool paired = staged_paired(n_tiles, nq, nkv, HD, splits, &shape);
+      const bool paired = staged_paired(n_tiles, nq, nkv, HD, splits, max_tile_ctx, mean_tile_walk, &shape);
       const dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, nkv * ((nq / nkv + shape.hpb - 1) / shape.hpb), splits);
 #define SP_STAGED(HPB, WPT, AHEAD, PAIRED)                                                                      \
   attention_prefill_staged_kernel<DT, NQT, HPB, WPT, AHEAD, PAIRED><<<grid, 64 * WPT * HPB, 0, s>>>(            \
@@ -924,13 +928,13 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
 int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
-                   int max_decode_ctx, int max_tile_ctx, float* workspace, void* out, int nq, int nkv, int hd,
-                   int page_size, int num_pages, int window, float scale) {
+                   int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace, void* out, int nq, int nkv,
+                   int hd, int page_size, int num_pages, int window, float scale) {
 #define SP_MFMA(DT)                                                                                              \
   case DT:                                                                                                       \
     return launch_mfma<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len,    \
-                           tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, workspace, out,  \
-                           nq, nkv, page_size, num_pages, window, scale)
+                           tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, mean_tile_walk,  \
+                           workspace, out, nq, nkv, page_size, num_pages, window, scale)
   switch (hd / 16) {
     SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
   }

@@ -56,7 +56,9 @@ int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, 
 // decode_seqs (plan[1] == 0; a null decode_seqs stands for sequences 0 .. n_decode - 1, which saves the kernels
 // one dependent read).  max_decode_ctx: largest ctx_len among decode_seqs; max_tile_ctx: largest
 // ctx_len among the sequences of the tile list (it only guides how a long walk over the keys is shared out
-// between blocks: a smaller value than the truth costs time, not correctness).
+// between blocks: a smaller value than the truth costs time, not correctness); mean_tile_walk: the mean over
+// the tiles of the keys a tile walks (likewise a hint, 0 if unknown: where the longest walk is much longer than
+// the mean, as in a prompt's first portion, a block takes a long and a short tile).
 // window <= 0: all keys; else keys with position - key < window.
 // workspace: sp_attention_workspace_floats(...) floats of scratch for partial results.
 int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind, int* plan);
@@ -65,9 +67,9 @@ int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, 
 int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                  const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                  const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, int tile_q,
-                 int max_tile_ctx, const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
-                 int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size, int num_pages,
-                 int window, float scale, int kernel_kind);
+                 int max_tile_ctx, int mean_tile_walk, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
+                 float* workspace, int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size,
+                 int num_pages, int window, float scale, int kernel_kind);
 
 // A step of one-query sequences only (bfloat16): attention with the output projection folded into the merge
 // of the key chunks: residual[q_start[seq], :] += attention(seq) . w_o^T with w_o [hidden, nq * hd] bfloat16

@@ -157,7 +157,8 @@ def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, wor
     on_device = {name: (d, len(lists[name])) for name, d in zip(list_names, dev[8:8 + len(list_names)])}
     decode_ctx = [int(c) for c, q in zip(ctx_len, q_lens) if q == 1]
     ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, len(entries), on_device,
-                                       max(decode_ctx, default=0), max((int(c) for c in ctx_len), default=0))
+                                       max(decode_ctx, default=0), max((int(c) for c in ctx_len), default=0),
+                                       ops.mean_tile_walk(q_lens, ctx_len))
     rest = dev[8 + len(list_names):]
     ctx.group_tables = rest[0::2]
     ctx.group_slots = rest[1::2]

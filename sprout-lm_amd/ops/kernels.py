@@ -169,14 +169,30 @@ def attention_lists(q_lens) -> dict:
     return out
 
 
+def mean_tile_walk(q_lens, ctx_lens, tile: int = 32) -> int:
+    """Mean over the tiles of `tile` queries (of sequences with more than one query) of the keys a tile walks."""
+    tiles = walked = 0
+    for q, c in zip(q_lens, ctx_lens):
+        q, c = int(q), int(c)
+        if q > 1:
+            n = -(-q // tile)
+            tiles += n
+            walked += n * (c - q) + tile * n * (n + 1) // 2     # the last tile counted as a whole one
+    return walked // tiles if tiles else 0
+
+
 class AttentionBatch:
     """The device-side description of a step's sequences that `attention` reads."""
 
-    def __init__(self, q_start, q_len, ctx_len, n_seqs: int, lists: dict, max_decode_ctx: int, max_ctx: int):
+    def __init__(self, q_start, q_len, ctx_len, n_seqs: int, lists: dict, max_decode_ctx: int, max_ctx: int,
+                 mean_walk: int = 0):
         """`lists`: name -> (device int32 tensor, number of entries), names as in `attention_lists`;
-        `max_decode_ctx`, `max_ctx`: the longest context among one-query sequences, and among all."""
+        `max_decode_ctx`, `max_ctx`: the longest context among one-query sequences, and among all;
+        `mean_walk`: the mean number of keys that a tile of queries walks, see `mean_tile_walk` (a hint for
+        how the kernels share out the work; unknown: 0)."""
         self.q_start, self.q_len, self.ctx_len, self.n_seqs = q_start, q_len, ctx_len, n_seqs
         self.lists, self.max_decode_ctx, self.max_ctx = lists, max_decode_ctx, max_ctx
+        self.mean_walk = mean_walk
 
     @classmethod
     def build(cls, q_lens, ctx_lens, device) -> "AttentionBatch":
@@ -187,7 +203,8 @@ class AttentionBatch:
         lists = {k: (to(v), len(v)) for k, v in attention_lists(q_lens).items()}
         decode_ctx = [c for c, q in zip(ctx_lens, q_lens) if q == 1]
         return cls(to(starts), to(q_lens), to(ctx_lens), len(q_lens), lists, max(decode_ctx, default=0),
-                   max((int(c) for c in ctx_lens), default=0))
+                   max((int(c) for c in ctx_lens), default=0),
+                   mean_tile_walk(q_lens, ctx_lens))
 
 
 def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: int, kind: int = 0) -> tuple[int, bool]:
@@ -265,7 +282,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
                                  batch.q_len.data_ptr(), batch.ctx_len.data_ptr(), _ptr(tiles) if n_tiles else None,
-                                 n_tiles, tile_q, max_tile_ctx, _ptr(decode) if n_decode else None, n_decode,
+                                 n_tiles, tile_q, max_tile_ctx, int(batch.mean_walk), _ptr(decode) if n_decode else None, n_decode,
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
                                  float(scale), kind))

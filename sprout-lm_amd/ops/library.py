@@ -23,7 +23,7 @@ def _declare(lib):
         "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int,
                           c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
-                         c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
+                         c_int, c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_float, c_int],
         "sp_attention_decode_project_takes": [c_int] * 7,
         "sp_attention_decode_project": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void,
