@@ -212,6 +212,7 @@ static const PipeShape kPipeShapes[] = {
     {64, 64, 2, 0.41f},     // 4 waves, 4 stages
     {64, 256, 1, 0.75f},    // 8 waves, 3 stages (few tokens)
     {64, 128, 2, 0.7f},     // 4 waves, 3 stages (few tokens)
+    {384, 256, 1, 3.3f},    // 8 waves, 2 stages (all of the LDS): where it saves a round of blocks
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -239,7 +240,7 @@ static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* sp
     }
     return;
   }
-  for (int c = 0; c < 4; ++c) {
+  for (int c : {0, 1, 2, 3, 6}) {
     const PipeShape& p = kPipeShapes[c];
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
@@ -265,6 +266,7 @@ static int pipe_shape(hipStream_t s, const void* x, const void* w, const void* b
     case 2: return launch_pipe<2, 2, 2, 2, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 4: return launch_pipe<1, 2, 2, 4, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 5: return launch_pipe<1, 2, 2, 2, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
+    case 6: return launch_pipe<6, 2, 2, 4, 2, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     default: return launch_pipe<1, 1, 2, 2, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
   }
 }
@@ -284,6 +286,7 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
   if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   return launch_pipe_mode<2, 2, 2, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
 }
 

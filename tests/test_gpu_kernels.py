@@ -22,7 +22,8 @@ def bf16(x):
                                    (513, 1152, 896), (2, 896, 4864), (40, 640, 1000), (64, 151, 72), (1000, 130, 136),
                                    (130, 257, 64), (200, 96, 192), (129, 300, 1024), (1000, 130, 128), (300, 331, 320),
                                    (700, 896, 4864), (65, 2100, 448),
-                                   (300, 4608, 3584), (40, 3584, 18944), (24, 3584, 3584), (520, 9728, 896)])
+                                   (300, 4608, 3584), (40, 3584, 18944), (24, 3584, 3584), (520, 9728, 896),
+                                   (1100, 13400, 192)])   # the last: blocks of 384 tokens save a round of blocks
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
@@ -480,8 +481,9 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     assert np.all((kp == 0) | written[:, None, :, None]) and np.all((vp == 0) | written[:, None, :, None])
 
 
-@pytest.mark.parametrize("T", [1, 8, 16, 33, 64, 65, 200, 513])
-@pytest.mark.parametrize("I,K", [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)])
+@pytest.mark.parametrize("T,I,K", [(t_, i_, k_) for t_ in [1, 8, 16, 33, 64, 65, 200, 513]
+                                   for i_, k_ in [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)]]
+                         + [(1100, 6700, 128), (2048, 4864, 896)])   # the last two: blocks of 384 tokens
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
