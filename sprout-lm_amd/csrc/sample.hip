@@ -9,7 +9,7 @@
 
 namespace sprout {
 
-constexpr int SAMPLE_CHUNK = 8192;  // logits per first-stage block
+constexpr int SAMPLE_CHUNK = 2048;  // logits per first-stage block: two groups of four per thread
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {  // splitmix64 finaliser
   z += 0x9e3779b97f4a7c15ull;
@@ -34,9 +34,9 @@ __global__ __launch_bounds__(256) void sample_stage1(const float* __restrict__ l
                                                      const int32_t* __restrict__ counter,
                                                      float* __restrict__ part_value, int* __restrict__ part_index,
                                                      int V, int chunks) {
-  __shared__ float sv[256];
-  __shared__ int si[256];
-  __shared__ int sbad[256];
+  __shared__ float sv[4];
+  __shared__ int si[4];
+  __shared__ int sbad[4];
   const int r = blockIdx.y, chunk = blockIdx.x;
   const float* row = logits + size_t(r) * V;
   const float temp = temperature ? temperature[r] : 0.f;
@@ -45,21 +45,44 @@ __global__ __launch_bounds__(256) void sample_stage1(const float* __restrict__ l
   const uint32_t ctr = counter ? uint32_t(counter[r]) : 0;
   float bv = -INFINITY;
   int bi = 0x7fffffff, bad = 0;
-  const int end = min(V, (chunk + 1) * SAMPLE_CHUNK);
-  for (int i = chunk * SAMPLE_CHUNK + threadIdx.x; i < end; i += 256) {
-    float v = row[i];
+  const int begin = chunk * SAMPLE_CHUNK, end = min(V, begin + SAMPLE_CHUNK);
+  auto take = [&](float v, int i) {
     if (!isfinite(v)) bad = 1;
     if (temp > 0.f) v = v * inv_temp + gumbel(sd, ctr, uint32_t(i));
     take_better(bv, bi, v, i);
-  }
-  sv[threadIdx.x] = bv; si[threadIdx.x] = bi; sbad[threadIdx.x] = bad;
-  __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (threadIdx.x < s) {
-      sbad[threadIdx.x] |= sbad[threadIdx.x + s];
-      take_better(sv[threadIdx.x], si[threadIdx.x], sv[threadIdx.x + s], si[threadIdx.x + s]);
+  };
+  if ((V & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    // the row starts at a multiple of 16 bytes: both groups of four are requested before either is looked at
+    float4 v[SAMPLE_CHUNK / 1024];
+#pragma unroll
+    for (int j = 0; j < SAMPLE_CHUNK / 1024; ++j) {
+      const int i = begin + 4 * (int(threadIdx.x) + 256 * j);
+      v[j] = i < end ? *reinterpret_cast<const float4*>(row + i) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     }
-    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < SAMPLE_CHUNK / 1024; ++j) {
+      const int i = begin + 4 * (int(threadIdx.x) + 256 * j);
+      if (i < end) { take(v[j].x, i); take(v[j].y, i + 1); take(v[j].z, i + 2); take(v[j].w, i + 3); }
+    }
+  } else {
+    for (int i = begin + threadIdx.x; i < end; i += 256) take(row[i], i);
+  }
+  // within the wave by lane exchange, between the four waves through LDS
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    bad |= __shfl_xor(bad, o, 64);
+    take_better(bv, bi, ov, oi);
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { sv[wave] = bv; si[wave] = bi; sbad[wave] = bad; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) {
+      sbad[0] |= sbad[w];
+      take_better(sv[0], si[0], sv[w], si[w]);
+    }
   }
   if (threadIdx.x == 0) {
     part_value[size_t(r) * chunks + chunk] = sv[0];
