@@ -5,8 +5,9 @@
 //   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from
 //                    the float32 residual and kept in LDS (no separate norm kernel, no round trip)
 //   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
-//             kEpiRope   the two tiles are rotation partners (dims d and d + head/2 of one head): adds
-//                        the bias, rotates q and k heads, writes q and scatters k, v into the paged cache
+//             kEpiRope   one tile a block (NT = 1): 8 dimensions of a head and their 8 rotation partners (dims
+//                        d and d + head/2), so that the few rows of q, k and v are spread over many blocks;
+//                        adds the bias, rotates q and k heads, writes q and scatters k, v into the paged cache
 //             kEpiSilu   the two tiles are gate rows and the matching up rows: writes silu(gate) * up
 // Accumulating products may also be split along K over several blocks (hardware float atomics).
 #include "mfma.h"
@@ -46,20 +47,21 @@ __device__ __forceinline__ float load_param(const void* p, int is_bf16, int i) {
 template <int EPI>
 __device__ __forceinline__ int tile_row0(const FusedArgs& a, int b, int which) {
   if (EPI == kEpiRope) {
-    const int per_head = a.hd / 32;                       // pairs of tiles per head
+    const int per_head = a.hd / 16;                       // tiles per head: 8 dims and their 8 partners each
     const int head = b / per_head, j = b % per_head;
-    return head * a.hd + 16 * j + which * a.partner;
+    return head * a.hd + 8 * j + which * a.partner;
   }
   if (EPI == kEpiSilu) return 16 * b + which * a.partner;
   return 16 * (2 * b + which);
 }
 
-template <int TN, int EPI, bool NORM>
+template <int TN, int EPI, bool NORM, int NT = 2>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
+  static_assert((NT == 1) == (EPI == kEpiRope), "one gathered tile a block for the rotation, two tiles otherwise");
   extern __shared__ uint4 lds[];
-  // reduction buffer [4 waves][2 tiles][TN][64 lanes] float4, then (NORM) activations [TN * 16][K / 8 + 1] uint4
+  // reduction buffer [4 waves][NT tiles][TN][64 lanes] float4, then (NORM) activations [TN * 16][K / 8 + 1] uint4
   float4* red = reinterpret_cast<float4*>(lds);
-  uint4* xs = lds + 4 * 2 * TN * 64;
+  uint4* xs = lds + 4 * NT * TN * 64;
   const int LD = a.K / 8 + 1;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const int k_begin = blockIdx.y * a.k_per_split;
@@ -68,22 +70,26 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   int row0[2];
   row0[0] = tile_row0<EPI>(a, blockIdx.x, 0);
   row0[1] = tile_row0<EPI>(a, blockIdx.x, 1);
-  const uint16_t* wrow[2];
+  const uint16_t* wrow[NT];
+  if (NT == 1) {   // rows 0..7 of the tile: dims row0[0] .. + 7 of the head; rows 8..15: their partners, half a head on
+    wrow[0] = a.w + size_t(min(a.N - 1, row0[0] + (lr < 8 ? lr : a.partner + lr - 8))) * a.K;
+  } else {
 #pragma unroll
-  for (int i = 0; i < 2; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
+    for (int i = 0; i < NT; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
+  }
 
   // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
   // of this wave together.
   constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
   const int steps = (k_end - k_begin + 63) / 64;
-  uint4 wa[UN][2][2];
+  uint4 wa[UN][NT][2];
   auto load_weights = [&](int s0) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
       const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
       const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < NT; ++i) {
         wa[u][i][0] = in0 ? ldg128(wrow[i] + k) : make_uint4(0, 0, 0, 0);
         wa[u][i][1] = in1 ? ldg128(wrow[i] + k + 8) : make_uint4(0, 0, 0, 0);
       }
@@ -137,13 +143,16 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   float bias_of[2] = {0.f, 0.f};
   if (a.bias && blockIdx.y == 0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      if (row0[i] + ei < a.N) bias_of[i] = load_param(a.bias, a.bias_bf16, row0[i] + ei);
+    for (int i = 0; i < 2; ++i) {
+      // one gathered tile: threads ei < 8 own dimension row0[0] + ei (i = 0) and its partner (i = 1)
+      const int n = NT == 1 ? row0[0] + (ei & 7) + i * a.partner : row0[i] + ei;
+      if (n < a.N) bias_of[i] = load_param(a.bias, a.bias_bf16, n);
+    }
   }
   int position_of[TN], slot_of[TN];
   float frequency = 0.f;
   if (EPI == kEpiRope) {
-    const int d = row0[0] % a.hd + ei;
+    const int d = row0[0] % a.hd + (ei & 7);
     if (d < a.rotary_dim / 2) frequency = a.inv_freq[d];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -181,9 +190,9 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     __syncthreads();
   }
 
-  floatx4 acc[2][TN];
+  floatx4 acc[NT][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NT; ++i)
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -213,17 +222,17 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
       for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < NT; ++i) {
           acc[i][tn] = mfma16(as_bf16x8(wa[u][i][0]), as_bf16x8(xb[u][tn][0]), acc[i][tn]);
           acc[i][tn] = mfma16(as_bf16x8(wa[u][i][1]), as_bf16x8(xb[u][tn][1]), acc[i][tn]);
         }
   }
 
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NT; ++i)
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
-      red[((wave * 2 + i) * TN + tn) * 64 + lane] = make_float4(acc[i][tn][0], acc[i][tn][1], acc[i][tn][2], acc[i][tn][3]);
+      red[((wave * NT + i) * TN + tn) * 64 + lane] = make_float4(acc[i][tn][0], acc[i][tn][1], acc[i][tn][2], acc[i][tn][3]);
   __syncthreads();
 
   // thread -> (token t of the tile, row i of the tile); the MFMA lane that holds it is (i / 4) * 16 + t, element i % 4
@@ -235,11 +244,17 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       float sum = 0.f;
+      if (NT == 1) {   // row ei & 7 of the one tile (i = 0) and its partner, row 8 + (ei & 7) (i = 1)
+        const int row = (ei & 7) + 8 * i, lane_of = (row >> 2) * 16 + et;
 #pragma unroll
-      for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * 2 + i) * TN + tn) * 64 + src_lane])[src_r];
+        for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[(w * TN + tn) * 64 + lane_of])[row & 3];
+      } else {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * NT + i) * TN + tn) * 64 + src_lane])[src_r];
+      }
       v[i] = sum + bias_of[i];
     }
-    if (t >= a.T) continue;
+    if (t >= a.T || (NT == 1 && ei >= 8)) continue;
     if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
@@ -259,7 +274,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
       }
     } else {  // kEpiRope
-      const int head = row0[0] / a.hd, d = row0[0] % a.hd + ei;      // d < hd / 2; partner dim d + hd / 2
+      const int head = row0[0] / a.hd, d = row0[0] % a.hd + (ei & 7);  // d < hd / 2; partner dim d + hd / 2
       // projections are kept as bfloat16 before the rotation, as in the unfused path
       float lo = to_float(bf16_t{f32_to_bf16_bits(v[0])}), hi = to_float(bf16_t{f32_to_bf16_bits(v[1])});
       const int half = a.hd / 2;
@@ -294,16 +309,17 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   }
 }
 
-static size_t fused_lds_bytes(int TN, bool norm, int K) {
-  return sizeof(float4) * 4 * 2 * TN * 64 + (norm ? sizeof(uint4) * size_t(TN) * 16 * (K / 8 + 1) : 0);
+static size_t fused_lds_bytes(int TN, bool norm, int K, int NT = 2) {
+  return sizeof(float4) * 4 * NT * TN * 64 + (norm ? sizeof(uint4) * size_t(TN) * 16 * (K / 8 + 1) : 0);
 }
 
 template <int TN, int EPI, bool NORM>
 static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
-  const size_t lds = fused_lds_bytes(TN, NORM, a.K);
+  constexpr int NT = EPI == kEpiRope ? 1 : 2;
+  const size_t lds = fused_lds_bytes(TN, NORM, a.K, NT);
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fused_kernel<TN, EPI, NORM>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fused_kernel<TN, EPI, NORM, NT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (e != hipSuccess) {
       set_error("sp_gemm_fused: cannot raise the LDS limit: %s", hipGetErrorString(e));
@@ -311,7 +327,7 @@ static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int split
     }
     raised = true;
   }
-  gemm_fused_kernel<TN, EPI, NORM><<<dim3(blocks, splits), 256, lds, s>>>(a);
+  gemm_fused_kernel<TN, EPI, NORM, NT><<<dim3(blocks, splits), 256, lds, s>>>(a);
   return check_launch("sp_gemm_fused");
 }
 
@@ -352,7 +368,7 @@ bool gemm_pipe_takes(int T, int N, int K);
 extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
   if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0;   // the tiled kernel's gated epilogue
   if (!fused_shape_ok(T, K, norm != 0)) return 0;
-  if (kind == kEpiRope) return hd % 32 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
+  if (kind == kEpiRope) return hd % 16 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
   if (kind == kEpiSilu) return N % 32 == 0;
   return kind == kEpiStore || kind == kEpiAccumulate || kind == kEpiStoreF32;
 }
@@ -418,7 +434,7 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.positions = positions; a.inv_freq = inv_freq; a.slot_mapping = slot_mapping;
   a.k_pool = (uint16_t*)k_pool; a.v_pool = (uint16_t*)v_pool;
   a.nq = nq; a.nkv = nkv; a.hd = hd; a.page_size = page_size; a.rotary_dim = rotary_dim;
-  const int blocks = (nq + 2 * nkv) * (hd / 32);
+  const int blocks = (nq + 2 * nkv) * (hd / 16);
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
 

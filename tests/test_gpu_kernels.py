@@ -436,7 +436,8 @@ def _normed(res, w, eps):
 @pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64])
 # the last two: few rows with a long K, which eight waves of a block share instead of four
 @pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4),
-                                              (4, 2, 128, 3584, 16), (3, 1, 64, 2120, 8)])
+                                              (4, 2, 128, 3584, 16), (3, 1, 64, 2120, 8), (4, 2, 16, 64, 16), (5, 5, 48, 240, 16),
+                                              (2, 1, 80, 160, 4)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     from sprout_lm_amd import ops
