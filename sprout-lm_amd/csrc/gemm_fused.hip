@@ -5,9 +5,10 @@
 //   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from
 //                    the float32 residual and kept in LDS (no separate norm kernel, no round trip)
 //   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
-//             kEpiRope   one tile a block (NT = 1): 8 dimensions of a head and their 8 rotation partners (dims
-//                        d and d + head/2), so that the few rows of q, k and v are spread over many blocks;
-//                        adds the bias, rotates q and k heads, writes q and scatters k, v into the paged cache
+//             kEpiRope   the block's rows are rotation partners (dims d and d + head/2 of one head): two tiles
+//                        of 16, or (NT = 1, up to 16 tokens) one tile of 8 dimensions and their 8 partners, so
+//                        that the few rows of q, k and v are spread over twice the blocks; adds the bias,
+//                        rotates q and k heads, writes q and scatters k, v into the paged cache
 //             kEpiSilu   the two tiles are gate rows and the matching up rows: writes silu(gate) * up
 // Accumulating products may also be split along K over several blocks (hardware float atomics).
 #include "mfma.h"
@@ -44,12 +45,13 @@ __device__ __forceinline__ float load_param(const void* p, int is_bf16, int i) {
 }
 
 // First row of tile `which` (0 or 1) of block `b`.
-template <int EPI>
+template <int EPI, int NT>
 __device__ __forceinline__ int tile_row0(const FusedArgs& a, int b, int which) {
   if (EPI == kEpiRope) {
-    const int per_head = a.hd / 16;                       // tiles per head: 8 dims and their 8 partners each
+    const int dims = NT == 1 ? 8 : 16;                    // dimensions of a head's first half that a block takes
+    const int per_head = a.hd / (2 * dims);
     const int head = b / per_head, j = b % per_head;
-    return head * a.hd + 8 * j + which * a.partner;
+    return head * a.hd + dims * j + which * a.partner;
   }
   if (EPI == kEpiSilu) return 16 * b + which * a.partner;
   return 16 * (2 * b + which);
@@ -57,7 +59,7 @@ __device__ __forceinline__ int tile_row0(const FusedArgs& a, int b, int which) {
 
 template <int TN, int EPI, bool NORM, int NT = 2>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
-  static_assert((NT == 1) == (EPI == kEpiRope), "one gathered tile a block for the rotation, two tiles otherwise");
+  static_assert(NT == 2 || EPI == kEpiRope, "one gathered tile a block only for the rotation");
   extern __shared__ uint4 lds[];
   // reduction buffer [4 waves][NT tiles][TN][64 lanes] float4, then (NORM) activations [TN * 16][K / 8 + 1] uint4
   float4* red = reinterpret_cast<float4*>(lds);
@@ -68,8 +70,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   const int k_end = min(a.K, k_begin + a.k_per_split);
 
   int row0[2];
-  row0[0] = tile_row0<EPI>(a, blockIdx.x, 0);
-  row0[1] = tile_row0<EPI>(a, blockIdx.x, 1);
+  row0[0] = tile_row0<EPI, NT>(a, blockIdx.x, 0);
+  row0[1] = tile_row0<EPI, NT>(a, blockIdx.x, 1);
   const uint16_t* wrow[NT];
   if (NT == 1) {   // rows 0..7 of the tile: dims row0[0] .. + 7 of the head; rows 8..15: their partners, half a head on
     wrow[0] = a.w + size_t(min(a.N - 1, row0[0] + (lr < 8 ? lr : a.partner + lr - 8))) * a.K;
@@ -140,19 +142,19 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
   // thread -> (token et of a tile, row ei of the tile), as in the epilogue below
   const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
+  const int er = NT == 1 ? (ei & 7) : ei;   // one gathered tile: threads ei < 8 own dimension er and its partner
   float bias_of[2] = {0.f, 0.f};
   if (a.bias && blockIdx.y == 0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      // one gathered tile: threads ei < 8 own dimension row0[0] + ei (i = 0) and its partner (i = 1)
-      const int n = NT == 1 ? row0[0] + (ei & 7) + i * a.partner : row0[i] + ei;
+      const int n = NT == 1 ? row0[0] + er + i * a.partner : row0[i] + ei;
       if (n < a.N) bias_of[i] = load_param(a.bias, a.bias_bf16, n);
     }
   }
   int position_of[TN], slot_of[TN];
   float frequency = 0.f;
   if (EPI == kEpiRope) {
-    const int d = row0[0] % a.hd + (ei & 7);
+    const int d = row0[0] % a.hd + er;
     if (d < a.rotary_dim / 2) frequency = a.inv_freq[d];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -244,8 +246,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       float sum = 0.f;
-      if (NT == 1) {   // row ei & 7 of the one tile (i = 0) and its partner, row 8 + (ei & 7) (i = 1)
-        const int row = (ei & 7) + 8 * i, lane_of = (row >> 2) * 16 + et;
+      if (NT == 1) {   // row er of the one tile (i = 0) and its partner, row 8 + er (i = 1)
+        const int row = er + 8 * i, lane_of = (row >> 2) * 16 + et;
 #pragma unroll
         for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[(w * TN + tn) * 64 + lane_of])[row & 3];
       } else {
@@ -274,7 +276,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
       }
     } else {  // kEpiRope
-      const int head = row0[0] / a.hd, d = row0[0] % a.hd + (ei & 7);  // d < hd / 2; partner dim d + hd / 2
+      const int head = row0[0] / a.hd, d = row0[0] % a.hd + er;      // d < hd / 2; partner dim d + hd / 2
       // projections are kept as bfloat16 before the rotation, as in the unfused path
       float lo = to_float(bf16_t{f32_to_bf16_bits(v[0])}), hi = to_float(bf16_t{f32_to_bf16_bits(v[1])});
       const int half = a.hd / 2;
@@ -313,9 +315,8 @@ static size_t fused_lds_bytes(int TN, bool norm, int K, int NT = 2) {
   return sizeof(float4) * 4 * NT * TN * 64 + (norm ? sizeof(uint4) * size_t(TN) * 16 * (K / 8 + 1) : 0);
 }
 
-template <int TN, int EPI, bool NORM>
+template <int TN, int EPI, bool NORM, int NT = 2>
 static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
-  constexpr int NT = EPI == kEpiRope ? 1 : 2;
   const size_t lds = fused_lds_bytes(TN, NORM, a.K, NT);
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
@@ -331,8 +332,21 @@ static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int split
   return check_launch("sp_gemm_fused");
 }
 
+// Whether the q/k/v product takes one gathered tile a block: with up to 16 tokens, where twice the blocks pull
+// the rows twice as fast; with more, every block reads all the activations again, which then costs more
+// (28 heads of 128 at a width of 3,584, 64 tokens: 36 us against about 20).  Head sizes that 32 does not divide
+// have no other way.
+static bool rope_one_tile(int T, int hd) { return T <= 16 || hd % 32 != 0; }
+
 template <int EPI, bool NORM>
 static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+  if (EPI == kEpiRope && rope_one_tile(a.T, a.hd)) {
+    if constexpr (EPI == kEpiRope) {
+      if (a.T <= 16) return launch_fused<1, EPI, NORM, 1>(s, a, blocks, splits);
+      if (a.T <= 32) return launch_fused<2, EPI, NORM, 1>(s, a, blocks, splits);
+      return launch_fused<4, EPI, NORM, 1>(s, a, blocks, splits);
+    }
+  }
   if (a.T <= 16) return launch_fused<1, EPI, NORM>(s, a, blocks, splits);
   if (a.T <= 32) return launch_fused<2, EPI, NORM>(s, a, blocks, splits);
   return launch_fused<4, EPI, NORM>(s, a, blocks, splits);
@@ -442,7 +456,7 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.positions = positions; a.inv_freq = inv_freq; a.slot_mapping = slot_mapping;
   a.k_pool = (uint16_t*)k_pool; a.v_pool = (uint16_t*)v_pool;
   a.nq = nq; a.nkv = nkv; a.hd = hd; a.page_size = page_size; a.rotary_dim = rotary_dim;
-  const int blocks = (nq + 2 * nkv) * (hd / 16);
+  const int blocks = (nq + 2 * nkv) * (hd / (rope_one_tile(T, hd) ? 16 : 32));
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
 
