@@ -160,6 +160,16 @@ __global__ void rope_cache_bf16_kernel(bf16_t* __restrict__ qkv, const int32_t* 
   }
 }
 
+// (cosine, sine) of positions[t] * inv_freq[d] for every token and pair: computed once per step for all layers.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq, int half,
+                                  float2* __restrict__ out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float sn, cs;
+  sincosf(float(positions[i / half]) * inv_freq[i % half], &sn, &cs);
+  out[i] = make_float2(cs, sn);
+}
+
 template <typename T>
 __global__ void rope_cache_kernel(T* __restrict__ qkv, const int32_t* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const float* __restrict__ inv_freq_tail, int rotary_dim,
@@ -300,6 +310,15 @@ extern "C" int sp_cast(void* stream, int src_dtype, const void* src, int dst_dty
   else
     SP_REQUIRE(false, "sp_cast: unsupported dtypes %d -> %d", src_dtype, dst_dtype);
   return check_launch("sp_cast");
+}
+
+extern "C" int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T) {
+  SP_REQUIRE(T >= 0 && half > 0 && positions && inv_freq && out, "sp_rope_table: bad arguments");
+  SP_REQUIRE(int64_t(T) * half < (int64_t(1) << 31), "sp_rope_table: too many entries");
+  if (T == 0) return 0;
+  const int n = T * half;
+  rope_table_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(positions, inv_freq, half, reinterpret_cast<float2*>(out), n);
+  return check_launch("sp_rope_table");
 }
 
 extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions,

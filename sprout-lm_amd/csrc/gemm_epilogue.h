@@ -6,7 +6,18 @@
 
 namespace sprout {
 
-enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2, kSilu = 3 };   // kSilu: gate rows and up rows, see below
+enum { kStore = 0, kAccumulate = 1, kStoreF32 = 2, kSilu = 3, kRope = 4 };   // kSilu, kRope: see below
+
+// What the rotating epilogue (kRope) needs beside the product: the rows of w are q, k and v heads of size hd.
+struct RopeArgs {
+  const int32_t* positions;      // [T]
+  const float* inv_freq;         // [hd / 2]
+  const int32_t* slot_mapping;   // [T]: page * page_size + slot of the token's key and value, or -1
+  uint16_t* k_pool;              // [page][kv head][slot][dim]
+  uint16_t* v_pool;              // [page][kv head][dim][slot]
+  int nq, nkv, hd, page_size;
+  const float2* table;           // [T][hd / 2] (cosine, sine) of positions[t] * inv_freq[d], or null: computed here
+};
 
 // Orders a wave's LDS writes before its own later reads of what other lanes wrote (and the reverse).
 __device__ __forceinline__ void wave_lds_fence() {
@@ -19,10 +30,81 @@ __device__ __forceinline__ void wave_lds_fence() {
 // it is used only when K is split over blocks (gridDim.z > 1).
 template <int WM, int WN, int MODE, typename TB, int WAVES_N = 2>
 __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[WM][WN], float* turn_all, const TB* __restrict__ bias,
-                                              void* __restrict__ out, int T, int N, int t0, int n0) {
+                                              void* __restrict__ out, int T, int N, int t0, int n0,
+                                              const RopeArgs& rope = RopeArgs{}) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int li = lane & 31, lk = lane >> 5;
+  if (MODE == kRope) {
+    // Tile columns come in groups of 64: 32 dimensions of a head's first half (tile column 2 m of a wave) and
+    // their rotation partners, half a head further on (tile column 2 m + 1), so that a lane holds both of a pair.
+    // Bias, rounding to bfloat16 (as where the projections pass through memory), rotation of q and k heads;
+    // q goes to out [T, nq * hd], k and v into the paged pools.
+    static_assert(MODE != kRope || WN % 2 == 0, "the rotating epilogue pairs tile columns");
+    const int hd = rope.hd, half = hd / 2, groups_per_head = half / 32, heads = rope.nq + 2 * rope.nkv;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int t = t0 + (wm * WM + i) * 32 + li;
+      if (t >= T) continue;
+      const float pos = float(rope.positions[t]);
+      const int slot = rope.slot_mapping[t];
+      const int page = slot >= 0 ? slot / rope.page_size : 0, off = slot >= 0 ? slot % rope.page_size : 0;
+#pragma unroll
+      for (int m = 0; m < WN / 2; ++m) {
+        const int group = n0 / 64 + wn * (WN / 2) + m, head = group / groups_per_head, u = group % groups_per_head;
+        if (head >= heads) continue;
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const int d0 = 32 * u + 8 * rg + 4 * lk;          // four consecutive dimensions of the first half
+          float lo[4], hi[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n = head * hd + d0 + r;
+            float a = acc[i][2 * m][4 * rg + r], b = acc[i][(2 * m + 1) % WN][4 * rg + r];
+            if (bias) { a += to_float(bias[n]); b += to_float(bias[n + half]); }
+            a = to_float(bf16_t{f32_to_bf16_bits(a)});
+            b = to_float(bf16_t{f32_to_bf16_bits(b)});
+            if (head < rope.nq + rope.nkv) {
+              float sn, cs;
+              if (rope.table) {
+                const float2 e = rope.table[size_t(t) * half + d0 + r];
+                cs = e.x;
+                sn = e.y;
+              } else {
+                sincosf(pos * rope.inv_freq[d0 + r], &sn, &cs);
+              }
+              lo[r] = a * cs - b * sn;
+              hi[r] = b * cs + a * sn;
+            } else {
+              lo[r] = a;
+              hi[r] = b;
+            }
+          }
+          const uint2 blo = make_uint2(pack_bf16x2(lo[0], lo[1]), pack_bf16x2(lo[2], lo[3]));
+          const uint2 bhi = make_uint2(pack_bf16x2(hi[0], hi[1]), pack_bf16x2(hi[2], hi[3]));
+          if (head < rope.nq) {
+            uint16_t* q = reinterpret_cast<uint16_t*>(out) + size_t(t) * (size_t(rope.nq) * hd) + head * hd + d0;
+            *reinterpret_cast<uint2*>(q) = blo;
+            *reinterpret_cast<uint2*>(q + half) = bhi;
+          } else if (slot >= 0) {
+            if (head < rope.nq + rope.nkv) {
+              uint16_t* k = rope.k_pool + ((size_t(page) * rope.nkv + (head - rope.nq)) * rope.page_size + off) * hd + d0;
+              *reinterpret_cast<uint2*>(k) = blo;
+              *reinterpret_cast<uint2*>(k + half) = bhi;
+            } else {
+              uint16_t* v = rope.v_pool + (size_t(page) * rope.nkv + (head - rope.nq - rope.nkv)) * hd * rope.page_size + off;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                v[size_t(d0 + r) * rope.page_size] = f32_to_bf16_bits(lo[r]);
+                v[size_t(d0 + half + r) * rope.page_size] = f32_to_bf16_bits(hi[r]);
+              }
+            }
+          }
+        }
+      }
+    }
+    return;
+  }
   if (MODE == kSilu) {
     // tile columns 2 m of a wave hold gate rows, columns 2 m + 1 the matching up rows:
     // out[t, n] = silu(gate) * up, both rounded to bfloat16 first, as where they are stored before the gated product

@@ -377,10 +377,15 @@ extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual
 namespace sprout {
 int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K);
 bool gemm_pipe_takes(int T, int N, int K);
+bool gemm_pipe_rope_takes(int T, int N, int K, int hd);
+int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
+                        const int32_t* positions, const float* inv_freq, const int32_t* slot_mapping, void* k_pool,
+                        void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, const float* table);
 }
 
 extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
   if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0;   // the tiled kernel's gated epilogue
+  if (kind == kEpiRope && T > 64) return !norm && rotary_dim == hd && gemm_pipe_rope_takes(T, N, K, hd);   // and its rotating one
   if (!fused_shape_ok(T, K, norm != 0)) return 0;
   if (kind == kEpiRope) return hd % 16 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
   if (kind == kEpiSilu) return N % 32 == 0;
@@ -443,12 +448,15 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
                                  const void* norm_w, float eps, const void* w, int bias_dtype, const void* bias,
                                  void* q_out, const int32_t* positions, const float* inv_freq, int rotary_dim,
                                  const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int K, int nq,
-                                 int nkv, int hd, int page_size) {
+                                 int nkv, int hd, int page_size, const float* cos_sin) {
   const int N = (nq + 2 * nkv) * hd;
   SP_REQUIRE(sp_fused_supported(kEpiRope, T, N, K, hd, rotary_dim, residual != nullptr),
              "sp_qkv_rope_cache: shape T=%d K=%d hd=%d rotary=%d is not taken", T, K, hd, rotary_dim);
   SP_REQUIRE((x || residual) && w && q_out && positions && inv_freq && slot_mapping && k_pool && v_pool,
              "sp_qkv_rope_cache: null operand");
+  if (T > 64)   // many tokens: the pipelined tiled product with the rotation as its epilogue
+    return gemm_bf16_pipe_rope((hipStream_t)stream, x, w, bias_dtype, bias, q_out, positions, inv_freq, slot_mapping, k_pool,
+                               v_pool, T, K, nq, nkv, hd, page_size, cos_sin);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.bias = bias; a.bias_bf16 = bias_dtype == kBF16; a.out = q_out;

@@ -43,7 +43,7 @@ __device__ __forceinline__ void wait_loads_then_barrier() {
 template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_pipe_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                         const TB* __restrict__ bias, void* __restrict__ out, int T,
-                                                        int N, int K, int k_per_split) {
+                                                        int N, int K, int k_per_split, RopeArgs rope) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   constexpr int ROW = 128;                              // bytes of a tile row
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_pipe_kernel(const
 
   // ---- what this lane fetches: row 8 (NW j + wave) + lane / 8 of each operand tile, for j < LX (LW)
   const unsigned char* xbase = reinterpret_cast<const unsigned char*>(x + size_t(t0) * K + k_begin);
-  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(w + (MODE == kSilu ? size_t(0) : size_t(n0) * K) + k_begin);
+  const unsigned char* wbase = reinterpret_cast<const unsigned char*>(w + (MODE == kSilu || MODE == kRope ? size_t(0) : size_t(n0) * K) + k_begin);
   uint32_t xoff[LX], woff[LW];
 #pragma unroll
   for (int j = 0; j < LX; ++j) {
@@ -91,6 +91,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_pipe_kernel(const
       // gate rows and the matching up rows, so that a lane ends with both of one index.
       const int gate = min(N - 1, tile_n * (BN / 2) + (r / 64) * 32 + (r & 31));
       row = ((r >> 5) & 1) ? N + gate : gate;
+    } else if (MODE == kRope) {
+      // Tile rows in runs of 32: 32 dimensions of a head's first half, then their rotation partners half a
+      // head further on, so that a lane ends with both of a pair.
+      const int half = rope.hd / 2, groups_per_head = half / 32;
+      const int group = tile_n * (BN / 64) + r / 64, head = group / groups_per_head, u = group % groups_per_head;
+      row = min(N - 1, head * rope.hd + 32 * u + (r & 31) + ((r >> 5) & 1) * half);
     } else {
       row = min(r, N - 1 - n0);
     }
@@ -159,12 +165,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_pipe_kernel(const
   }
   if (MODE == kAccumulate && gridDim.z > 1) __syncthreads();   // the epilogue turns tiles round in this LDS
   static_assert(NW * 32 * (32 * WN + 4) * sizeof(float) <= size_t(STAGES) * STAGE, "the turning buffer must fit");
-  tile_epilogue<WM, WN, MODE, TB, WAVES_N>(acc, reinterpret_cast<float*>(pipe_lds), bias, out, T, N, t0, n0);
+  tile_epilogue<WM, WN, MODE, TB, WAVES_N>(acc, reinterpret_cast<float*>(pipe_lds), bias, out, T, N, t0, n0, rope);
 }
 
 template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB>
 static int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const uint16_t* w, const TB* bias, void* out,
-                            int T, int N, int K, int k_per_split) {
+                            int T, int N, int K, int k_per_split, const RopeArgs& rope = RopeArgs{}) {
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   constexpr size_t lds = size_t(STAGES) * (BM + BN) * 128;
   static bool raised = false;
@@ -181,7 +187,7 @@ static int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const 
   const int tiles_t = (T + BM - 1) / BM, tiles_n = ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN;
   const int per_xcd = (tiles_n + 7) / 8, group = min(tiles_t, 8), groups = (tiles_t + group - 1) / group;
   dim3 grid(8 * per_xcd * group * groups, 1, splits);
-  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split);
+  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope);
   return check_launch("sp_gemm (pipelined)");
 }
 
@@ -218,7 +224,7 @@ static const PipeShape kPipeShapes[] = {
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
 // kernels, so large tiles win whenever they still fill the chip; products with few tiles (narrow outputs)
 // take small tiles or, when accumulating, a split of K, whose float atomics are charged per element.
-static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits) {
+static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, bool paired_columns = false) {
   const int steps = K / 64;
   float best = 1e30f;
   *shape = 2;
@@ -241,6 +247,7 @@ static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* sp
     return;
   }
   for (int c : {0, 1, 2, 3, 6}) {
+    if (paired_columns && c == 3) continue;     // one tile column per wave: nothing to pair
     const PipeShape& p = kPipeShapes[c];
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
@@ -288,6 +295,40 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   return launch_pipe_mode<2, 2, 2, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+}
+
+// q, k, v = x . w^T + bias with w [(nq + 2 nkv) * hd, K]; q and k heads rotated; q to q_out [T, nq * hd], k and v
+// into the paged pools.  Head sizes that are multiples of 64, more than 64 tokens.
+template <typename TB>
+static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const TB* bias, void* q_out, int T, int N, int K,
+                     const RopeArgs& rope) {
+  int shape, splits;
+  pipe_choice(T, N, K, false, &shape, &splits, true);
+  if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+}
+
+// Taken where the plain product would not run on blocks of 64 x 64 (one tile column per wave: no lane holds both
+// of a pair): with few tokens those fill the chip better than anything larger, and a rotation kernel of its own
+// after them costs less than that (256 tokens at 14 + 2 + 2 heads of 64: 7.6 + 5 us against 17).
+bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
+  if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
+  int shape, splits;
+  pipe_choice(T, N, K, false, &shape, &splits);
+  return shape != 3;
+}
+
+int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
+                        const int32_t* positions, const float* inv_freq, const int32_t* slot_mapping, void* k_pool,
+                        void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, const float* table) {
+  RopeArgs rope = {positions, inv_freq, slot_mapping, (uint16_t*)k_pool, (uint16_t*)v_pool, nq, nkv, hd, page_size,
+                   reinterpret_cast<const float2*>(table)};
+  const int N = (nq + 2 * nkv) * hd;
+  if (bias && bias_dtype == kBF16)
+    return pipe_rope<bf16_t>(s, (const uint16_t*)x, (const uint16_t*)w, (const bf16_t*)bias, q_out, T, N, K, rope);
+  return pipe_rope<float>(s, (const uint16_t*)x, (const uint16_t*)w, (const float*)bias, q_out, T, N, K, rope);
 }
 
 }  // namespace sprout

@@ -31,10 +31,15 @@ int sp_fused_norm_pays(int T, int N, int K);
 int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
                    const void* w, int bias_dtype, const void* bias, int mode, void* out, int T, int N, int K);
 // q, k, v projection (+ bias), rotation of q and k, q to q_out [T, nq * hd], k and v into the paged pools.
+// With more than 64 tokens (head sizes that are multiples of 64) the tiled product does it in its epilogue;
+// cos_sin (may be null): the table of sp_rope_table for these positions, which saves it the sines and cosines.
 int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w,
                       float eps, const void* w, int bias_dtype, const void* bias, void* q_out,
                       const int32_t* positions, const float* inv_freq, int rotary_dim, const int32_t* slot_mapping,
-                      void* k_pool, void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size);
+                      void* k_pool, void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size,
+                      const float* cos_sin);
+// out [T][half][2] = (cosine, sine) of positions[t] * inv_freq[d]: the same for every layer of a step.
+int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T);
 // out [T, I] = silu(x . w[:I]^T) * (x . w[I:]^T)
 int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
                     const void* w, void* out, int T, int I, int K);

@@ -71,6 +71,7 @@ class StepContext:
         self.group_tables: list[torch.Tensor] = []
         self.group_slots: list[torch.Tensor] = []
         self.host = {}   # the same arrays on the host (numpy), for parts that plan on the CPU
+        self.shared = {}   # what a part computes once per step for all layers (key chosen by the part)
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)

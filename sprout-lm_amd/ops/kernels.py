@@ -324,10 +324,12 @@ def _activations(x, residual, norm_weight, K: int, what: str):
 
 def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_freq, rotary_dim: int, slot_mapping,
                    k_pool, v_pool, nq: int, nkv: int, hd: int, x=None, residual=None, norm_weight=None,
-                   eps: float = 0.0) -> None:
+                   eps: float = 0.0, table=None) -> None:
     """q, k, v = activations . w^T + bias; rotate q and k; q to q_out, k and v into the paged pools.
 
-    Activations are x (bfloat16) or rmsnorm(residual) * norm_weight computed inside the kernel."""
+    Activations are x (bfloat16) or rmsnorm(residual) * norm_weight computed inside the kernel.
+    `table`: `rope_table` of these positions (float32 [T, hd / 2, 2]), which the many-token kernel reads
+    instead of computing sines and cosines."""
     _gpu(w, "qkv weight"); _gpu(q_out, "q output")
     N, K = w.shape
     xp, rp, nd, npt, T = _activations(x, residual, norm_weight, K, "qkv_rope_cache")
@@ -339,10 +341,24 @@ def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_fr
             raise KernelError("qkv_rope_cache: bias size")
     _ints(positions, T, "positions"); _ints(slot_mapping, T, "slot_mapping"); _gpu(inv_freq, "inv_freq")
     _, page_size = _check_pools(k_pool, v_pool, nkv, hd, torch.bfloat16, "qkv_rope_cache")
+    if table is not None:
+        _gpu(table, "rotation table")
+        if table.dtype != torch.float32 or tuple(table.shape) != (T, hd // 2, 2) or rotary_dim != hd:
+            raise KernelError(f"qkv_rope_cache: the rotation table must be float32 [{T}, {hd // 2}, 2]")
     check(library().sp_qkv_rope_cache(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(),
                                       _code(bias, "bias") if bias is not None else 0, _ptr(bias), q_out.data_ptr(),
                                       positions.data_ptr(), inv_freq.data_ptr(), rotary_dim, slot_mapping.data_ptr(),
-                                      k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd, page_size))
+                                      k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd, page_size, _ptr(table)))
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, d] = (cos, sin) of positions[t] * inv_freq[d]; out float32 [T, len(inv_freq), 2]."""
+    _gpu(inv_freq, "inv_freq"); _gpu(out, "rotation table")
+    T, half = out.shape[0], inv_freq.numel()
+    _ints(positions, T, "positions")
+    if inv_freq.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (T, half, 2):
+        raise KernelError("rope_table: inv_freq float32 [half] and out float32 [T, half, 2] expected")
+    check(library().sp_rope_table(_stream(), positions.data_ptr(), inv_freq.data_ptr(), half, out.data_ptr(), T))
 
 
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0) -> None:

@@ -35,7 +35,8 @@ def _declare(lib):
         "sp_gemm_decode": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_void, c_int,
                            c_int, c_int],
         "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,
-                              c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int],
+                              c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+        "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
         "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int],
         "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int],
         "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],

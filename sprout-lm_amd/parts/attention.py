@@ -64,7 +64,7 @@ class Attention(Mixer):
         self.position.prepare(device, dtype)
 
     def _fused(self, T: int, cache, norm: bool) -> bool:
-        """Whether the decode-sized fused projection kernel takes this call."""
+        """Whether a projection kernel with bias, rotation and cache write folded in takes this call."""
         return (self.own_kv and cache.writes and self.w_qkv.dtype == torch.bfloat16
                 and ops.fused_supported(ops.FUSED_ROPE, T, self.w_qkv.shape[0], self.hidden, self.head_dim,
                                         self.position.rotary_dim, norm))
@@ -103,11 +103,13 @@ class Attention(Mixer):
 
     def forward(self, ctx, h, residual, cache):
         T = h.shape[0]
-        if ctx.act_dtype == torch.bfloat16 and T <= 64 and self._fused(T, cache, False):
+        if ctx.act_dtype == torch.bfloat16 and self._fused(T, cache, False):
             q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
+            # many tokens: the sines and cosines are the same in every layer, computed once per step
+            table = self.position.table(ctx) if T > 64 and hasattr(self.position, "table") else None
             ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq,
                                self.position.rotary_dim, cache.slot_mapping, cache.k, cache.v, self.heads,
-                               self.kv_heads, self.head_dim, x=h)
+                               self.kv_heads, self.head_dim, x=h, table=table)
             self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
             return
         nkv = self.kv_heads if (self.own_kv and cache.writes) else 0

@@ -34,6 +34,19 @@ class NeoxRotary(PositionEncoding):
         if dtype == torch.float32:
             self.inv_freq_tail = (exact - exact.to(torch.float32).to(torch.float64)).to(torch.float32).to(device)
 
+    def table(self, ctx) -> torch.Tensor:
+        """(cosine, sine) of every token's angles, float32 [T, rotary_dim / 2, 2]: the same in every layer, so
+        the first layer of a step that asks computes it and the others find it in the step's context."""
+        from .. import ops
+        key = ("rotary_neox", self.rotary_dim, float(self.theta))
+        found = ctx.shared.get(key)
+        if found is None:
+            found = ctx.buffer(f"rotation_table_{self.rotary_dim}_{float(self.theta)!r}",
+                               (ctx.n_tokens, self.rotary_dim // 2, 2), torch.float32)
+            ops.rope_table(ctx.positions, self.inv_freq, found)
+            ctx.shared[key] = found
+        return found
+
 
 @register_part("position", "none")
 class NoPosition(PositionEncoding):

@@ -433,17 +433,17 @@ def _normed(res, w, eps):
     return bf16(x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * w)
 
 
-@pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64])
+@pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64, 65, 200, 513])   # above 64: the tiled product's rotating epilogue
 # the last two: few rows with a long K, which eight waves of a block share instead of four
 @pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4),
                                               (4, 2, 128, 3584, 16), (3, 1, 64, 2120, 8), (4, 2, 16, 64, 16), (5, 5, 48, 240, 16),
-                                              (2, 1, 80, 160, 4)])
+                                              (2, 1, 80, 160, 4), (5, 1, 64, 320, 8), (3, 3, 128, 384, 16)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     from sprout_lm_amd import ops
     taken = ops.fused_supported(ops.FUSED_ROPE, T, (nq + 2 * nkv) * hd, K, hd, hd, norm)
     rng = np.random.default_rng(T * 7 + hd)
-    N, pages, theta, eps = (nq + 2 * nkv) * hd, 40, 10000.0, 1e-5
+    N, pages, theta, eps = (nq + 2 * nkv) * hd, max(40, -(-T // page) + 1), 10000.0, 1e-5
     w = bf16(rng.standard_normal((N, K)) / math.sqrt(K))
     b = bf16(rng.standard_normal(N) * 0.3)
     res = (rng.standard_normal((T, K)) * 2).astype(np.float32)
@@ -480,6 +480,17 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     written = np.zeros((pages, page), bool)
     written[[s // page for s in slots if s >= 0], [s % page for s in slots if s >= 0]] = True
     assert np.all((kp == 0) | written[:, None, :, None]) and np.all((vp == 0) | written[:, None, :, None])
+    if T > 64:   # with the step's table of cosines and sines the result is the same to the bit
+        table = torch.empty(T, hd // 2, 2, dtype=torch.float32, device=DEV)
+        ops.rope_table(t(pos, torch.int32), inv, table)
+        angles = pos[:, None].astype(np.float32) * inv.cpu().numpy()[None, :]
+        assert np.abs(table.cpu().numpy() - np.stack([np.cos(angles.astype(np.float64)), np.sin(angles.astype(np.float64))], -1)).max() < 1e-6
+        kp2, vp2, q2 = torch.zeros_like(t(kp, torch.bfloat16)), torch.zeros_like(t(vp, torch.bfloat16)), torch.zeros_like(q_out)
+        vp2 = torch.zeros(pages, nkv, hd, page, dtype=torch.bfloat16, device=DEV)
+        ops.qkv_rope_cache(t(w, torch.bfloat16), t(b, torch.bfloat16), q2, t(pos, torch.int32), inv, hd,
+                           t(slots, torch.int32), kp2, vp2, nq, nkv, hd, table=table, **args)
+        assert torch.equal(q2, q_out)
+        assert np.array_equal(kp2.float().cpu().numpy(), kp) and np.array_equal(vp2.float().cpu().numpy().transpose(0, 1, 3, 2), vp)
 
 
 @pytest.mark.parametrize("T,I,K", [(t_, i_, k_) for t_ in [1, 8, 16, 33, 64, 65, 200, 513]
