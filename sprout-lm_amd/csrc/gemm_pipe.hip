@@ -224,7 +224,7 @@ static const PipeShape kPipeShapes[] = {
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
 // kernels, so large tiles win whenever they still fill the chip; products with few tiles (narrow outputs)
 // take small tiles or, when accumulating, a split of K, whose float atomics are charged per element.
-static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, bool paired_columns = false) {
+static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits) {
   const int steps = K / 64;
   float best = 1e30f;
   *shape = 2;
@@ -247,7 +247,6 @@ static void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* sp
     return;
   }
   for (int c : {0, 1, 2, 3, 6}) {
-    if (paired_columns && c == 3) continue;     // one tile column per wave: nothing to pair
     const PipeShape& p = kPipeShapes[c];
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
@@ -303,21 +302,23 @@ template <typename TB>
 static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const TB* bias, void* q_out, int T, int N, int K,
                      const RopeArgs& rope) {
   int shape, splits;
-  pipe_choice(T, N, K, false, &shape, &splits, true);
-  if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  pipe_choice(T, N, K, false, &shape, &splits);
   if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
-  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
-  return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 2) return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  set_error("sp_qkv_rope_cache: no rotating epilogue for %d tokens, %d rows, K = %d", T, N, K);
+  return 1;
 }
 
-// Taken where the plain product would not run on blocks of 64 x 64 (one tile column per wave: no lane holds both
-// of a pair): with few tokens those fill the chip better than anything larger, and a rotation kernel of its own
-// after them costs less than that (256 tokens at 14 + 2 + 2 heads of 64: 7.6 + 5 us against 17).
+// Taken where the plain product would run on blocks of 256 x 128 or 128 x 128.  Blocks of 64 x 64 have one tile
+// column per wave (no lane holds both of a pair), and with few tokens they fill the chip better than anything
+// larger (256 tokens at 14 + 2 + 2 heads of 64: 7.6 us and a rotation kernel of 5 against 17).  The blocks of
+// 8 waves hold 128 sums per lane, all the registers a lane has there: the epilogue's own would be spilled
+// (measured at 28 + 4 + 4 heads of 128, 2,048 tokens: 332 us against 106 and a rotation kernel of 18).
 bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
   if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
-  return shape != 3;
+  return shape == 1 || shape == 2;
 }
 
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
