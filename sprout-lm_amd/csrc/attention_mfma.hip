@@ -99,7 +99,7 @@ __device__ __forceinline__ float max_over_quarters(float x) {
 // MASKED false: every key of the step is visible to every existing row (the caller has checked), and
 // rows that do not exist compute values nobody reads.  The running maximum m is in log2 units and
 // starts at kNoKeyYet.
-template <int DT, int NQT, bool MASKED>
+template <int DT, int NQT, bool MASKED, bool LAZY>
 __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                                  floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT],
                                                  int key0, int k_lo, const int (&qpos)[NQT], int window,
@@ -136,9 +136,13 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
     float raw = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
     raw = vmax3(raw, s[qt][0][3], s[qt][1][0]);
     raw = vmax3(raw, s[qt][1][1], s[qt][1][2]);
-    raw = max_over_quarters(vmax(raw, s[qt][1][3]));
-    const float top = raw * scale2;                          // -inf when the row sees no key of the step
-    if (__builtin_amdgcn_ballot_w64(top > m[qt] + kRescaleStep) != 0) {
+    raw = vmax(raw, s[qt][1][3]);
+    // LAZY: the lane's own 8 keys decide whether anything has to be done about the maximum, and the row's other
+    // three lanes are asked only then (-inf when the lane sees no key of the step): ten instructions less per
+    // step and tile of rows.  Otherwise the row's maximum is formed first.
+    if (!LAZY) raw = max_over_quarters(raw);
+    if (__builtin_amdgcn_ballot_w64(raw * scale2 > m[qt] + kRescaleStep) != 0) {
+      const float top = (LAZY ? max_over_quarters(raw) : raw) * scale2;
       const float mx = top > m[qt] + kRescaleStep ? top : m[qt];   // finite: m starts finite
       const float alpha = __builtin_amdgcn_exp2f(m[qt] - mx);
       m[qt] = mx;
@@ -168,15 +172,15 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 
 // `first_pos`: smallest position among the rows that exist; a step whose 32 keys all lie at or before
 // it (and inside [k_lo, ...) with no window) needs no masking.
-template <int DT, int NQT>
+template <int DT, int NQT, bool LAZY = true>
 __device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                             floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT], int key0,
                                             int k_lo, const int (&qpos)[NQT], int window, float scale2,
                                             int first_pos) {
   if (window <= 0 && key0 >= k_lo && key0 + 31 <= first_pos)
-    attend_step_impl<DT, NQT, false>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step_impl<DT, NQT, false, LAZY>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
   else
-    attend_step_impl<DT, NQT, true>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step_impl<DT, NQT, true, LAZY>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
 }
 
 template <int DT>
@@ -422,7 +426,9 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
 #pragma unroll
           for (int kt = 0; kt < 2; ++kt)
             r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[(16 * dt + lr) * VP + skey + 16 * kt + 4 * lj]);
-        attend_step<DT, NQT>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+        // (the unpaired block of 16 waves has no register to spare: the lazy form made it spill 36 instead of 2,
+        // 529 -> 690 us for 2,048 queries over 32,768 keys; the paired one gained with it, 290 -> 264 us at 8,192)
+        attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED)>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
       }
     }
   }
