@@ -7,6 +7,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
 
@@ -78,8 +79,19 @@ def build(folder: str | None = None, verbose: bool = True, jobs: int | None = No
 
     if verbose:
         print(f"[sprout build] compiling {len(names)} HIP sources for {ARCH} ...", file=sys.stderr, flush=True)
-    with ThreadPoolExecutor(max_workers=jobs or min(8, os.cpu_count() or 4)) as pool:
-        objects = list(pool.map(compile_one, names))
+    done_compiling = threading.Event()
+
+    def heartbeat() -> None:      # the largest source takes most of a minute: say that the build is alive
+        while not done_compiling.wait(10.0):
+            print(f"[sprout build] still compiling ({time.time() - started:.0f}s) ...", file=sys.stderr, flush=True)
+
+    if verbose:
+        threading.Thread(target=heartbeat, daemon=True).start()
+    try:
+        with ThreadPoolExecutor(max_workers=jobs or min(8, os.cpu_count() or 4)) as pool:
+            objects = list(pool.map(compile_one, names))
+    finally:
+        done_compiling.set()
     tmp = library_path(folder) + f".tmp{os.getpid()}"
     done = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp, *objects],
                           capture_output=True, text=True)

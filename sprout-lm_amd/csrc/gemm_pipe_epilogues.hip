@@ -1,0 +1,56 @@
+// The pipelined tiled product with the gated (gate/up + SiLU) and the rotating (q/k/v + rotation + cache write)
+// epilogue: the kernel of gemm_pipe.h in the shapes that gemm_pipe.hip's cost model picks.
+#include "gemm_pipe.h"
+
+namespace sprout {
+
+// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T): a block's weight rows are half gate rows, half the matching up rows.
+int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
+  const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
+  int shape, splits;
+  pipe_choice(T, 2 * I, K, false, &shape, &splits);
+  if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  return launch_pipe_mode<2, 2, 2, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+}
+
+// q, k, v = x . w^T + bias with w [(nq + 2 nkv) * hd, K]; q and k heads rotated; q to q_out [T, nq * hd], k and v
+// into the paged pools.  Head sizes that are multiples of 64, more than 64 tokens.
+template <typename TB>
+static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const TB* bias, void* q_out, int T, int N, int K,
+                     const RopeArgs& rope) {
+  int shape, splits;
+  pipe_choice(T, N, K, false, &shape, &splits);
+  if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 2) return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  set_error("sp_qkv_rope_cache: no rotating epilogue for %d tokens, %d rows, K = %d", T, N, K);
+  return 1;
+}
+
+// Taken where the plain product would run on blocks of 256 x 128 or 128 x 128.  Blocks of 64 x 64 have one tile
+// column per wave (no lane holds both of a pair), and with few tokens they fill the chip better than anything
+// larger (256 tokens at 14 + 2 + 2 heads of 64: 7.6 us and a rotation kernel of 5 against 17).  The blocks of
+// 8 waves hold 128 sums per lane, all the registers a lane has there: the epilogue's own would be spilled
+// (measured at 28 + 4 + 4 heads of 128, 2,048 tokens: 332 us against 106 and a rotation kernel of 18).
+bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
+  if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
+  int shape, splits;
+  pipe_choice(T, N, K, false, &shape, &splits);
+  return shape == 1 || shape == 2;
+}
+
+int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
+                        const int32_t* positions, const float* inv_freq, const int32_t* slot_mapping, void* k_pool,
+                        void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, const float* table) {
+  RopeArgs rope = {positions, inv_freq, slot_mapping, (uint16_t*)k_pool, (uint16_t*)v_pool, nq, nkv, hd, page_size,
+                   reinterpret_cast<const float2*>(table)};
+  const int N = (nq + 2 * nkv) * hd;
+  if (bias && bias_dtype == kBF16)
+    return pipe_rope<bf16_t>(s, (const uint16_t*)x, (const uint16_t*)w, (const bf16_t*)bias, q_out, T, N, K, rope);
+  return pipe_rope<float>(s, (const uint16_t*)x, (const uint16_t*)w, (const float*)bias, q_out, T, N, K, rope);
+}
+
+}  // namespace sprout
