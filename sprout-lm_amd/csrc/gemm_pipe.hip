@@ -22,6 +22,7 @@ static const PipeShape kPipeShapes[] = {
     {64, 256, 1, 0.75f},    // 8 waves, 3 stages (few tokens)
     {64, 128, 2, 0.7f},     // 4 waves, 3 stages (few tokens)
     {384, 256, 1, 3.3f},    // 8 waves, 2 stages (all of the LDS): where it saves a round of blocks
+    {64, 64, 2, 0.45f},     // 2 waves with two tile columns each, 4 stages (few tokens: most blocks)
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -36,13 +37,17 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits) {
     // Few tokens: the weights are read once from memory, which bounds the product from below; a block's
     // steps follow each other at memory latency, so K is split until the blocks are short enough.
     const float stream_us = float(N) * float(K) * 2.f / 4.5e6f;
-    for (int c = 4; c < 6; ++c) {
+    for (int c : {4, 5, 7}) {
       const PipeShape& p = kPipeShapes[c];
       const int tiles = (N + p.bn - 1) / p.bn, slots = 256 * p.per_cu;
       for (int sp : {1, 2, 4, 8, 16}) {
         if (sp > 1 && (!may_split || steps / sp < 8)) break;
+        // blocks of two waves do badly on a long walk along K (37,888 x 3,584 at 64 tokens: 66 us against 59)
+        if (c == 7 && steps / sp > 24) continue;
         const int rounds = (tiles * sp + slots - 1) / slots;
-        float t = fmaxf(stream_us, rounds * float((steps + sp - 1) / sp) * p.step_us) + 2.0f;
+        // a CU pulls about 30 GB/s of weight rows, however many blocks it holds: the CU with the most blocks
+        const float pull_us = float((tiles * sp + 255) / 256) * float(p.bn) * float(K / sp) * 2.f / 30e3f;
+        float t = fmaxf(fmaxf(stream_us, pull_us), rounds * float((steps + sp - 1) / sp) * p.step_us) + 2.0f;
         if (sp > 1) t += 2.7e-6f * float(T) * float(N) * sp;
         if (t < best) { best = t; *shape = c; *splits = sp; }
       }

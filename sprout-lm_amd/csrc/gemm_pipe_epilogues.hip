@@ -14,6 +14,7 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
   if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 7) return launch_pipe_mode<1, 2, 2, 1, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   return launch_pipe_mode<2, 2, 2, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
 }
 
