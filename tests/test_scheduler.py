@@ -326,3 +326,13 @@ def test_lookahead_under_random_arrivals_cancellations_and_pressure(seed):
             assert result["status"] == "finished" and result["output"] == want, id
     engine.cache.clear_prefixes()
     assert engine.cache.free_pages() == [num_blocks]
+
+
+def test_mean_walk_of_a_steps_tiles():
+    """The hint that the attention kernels get of how unequal the walks of a step's tiles are."""
+    from sprout_lm_amd.ops import mean_tile_walk
+    assert mean_tile_walk([2048], [2048]) == 1040            # a prompt's first portion: 32, 64, ..., 2,048 keys
+    assert mean_tile_walk([2048], [4096]) == 2048 + 1040     # the same after 2,048 earlier tokens
+    assert mean_tile_walk([1, 1, 1], [5, 600, 7]) == 0       # decoded tokens have no tiles
+    assert mean_tile_walk([1, 40], [900, 40]) == (32 + 64) // 2   # the last tile counts as a whole one
+    assert mean_tile_walk([], []) == 0
