@@ -7,7 +7,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-REFERENCE_FIXTURE = "/root/reference/test/fixtures/qwen-tiny"
+# the reference checkout's own fixture; SPROUT_REFERENCE_FIXTURE names a copy where the checkout is not mounted
+REFERENCE_FIXTURE = os.environ.get("SPROUT_REFERENCE_FIXTURE", "/root/reference/test/fixtures/qwen-tiny")
 
 
 def pytest_configure(config):
