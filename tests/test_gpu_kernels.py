@@ -23,7 +23,9 @@ def bf16(x):
                                    (130, 257, 64), (200, 96, 192), (129, 300, 1024), (1000, 130, 128), (300, 331, 320),
                                    (700, 896, 4864), (65, 2100, 448),
                                    (300, 4608, 3584), (40, 3584, 18944), (24, 3584, 3584), (520, 9728, 896),
-                                   (1100, 13400, 192)])   # the last: blocks of 384 tokens save a round of blocks
+                                   (1100, 13400, 192),    # blocks of 384 tokens save a round of blocks
+                                   # few tiles and a long K
+                                   (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
