@@ -3,6 +3,9 @@
 // One block works on 16 queries of one sequence and one head, walking the keys 32 at a time with a
 // running maximum and sum (all float32).  Keys are always walked from a multiple of 32, so the order
 // of the sums at a position does not depend on how the tokens were cut into steps.
+// A step of few tiles and long contexts (decoding) would leave most of the chip idle: the keys are then
+// shared out in chunks (a multiple of 32 keys each) over gridDim.z blocks, which leave their maxima, sums
+// and unnormalised outputs in a workspace, and a second kernel joins them in the order of the chunks.
 #include "common.h"
 #include "sprout_hip.h"
 
@@ -76,7 +79,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
-    T* __restrict__ out, int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale) {
+    T* __restrict__ out, int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale,
+    float* __restrict__ part, int chunk) {
   extern __shared__ float lds[];
   // rows one float longer than their content: the four query rows that a wave reads at the same column
   // then lie in different LDS banks
@@ -105,6 +109,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   src.nkv = nkv; src.g = h / (nq / nkv); src.hd = hd; src.page_size = page_size; src.num_pages = num_pages;
   src.k_end = pos0 + nvalid;  // one past the last visible key of the tile
   src.k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int n_chunks = gridDim.z, first_key = blockIdx.z * chunk;   // this block's keys: first_key .. + chunk - 1
+  if (blockIdx.z + 1 < n_chunks) src.k_end = min(src.k_end, first_key + chunk);   // the last chunk: all that is left
   src.by_hd.set(hd);
   src.by_page.set(page_size);
   const int k_lo = src.k_lo, k_end = src.k_end;
@@ -116,7 +122,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   // The keys and values of a tile are requested while the tile before it is still being summed: the walk
   // waits for memory once per tile, not once per element.
   float ktile[2 * MAXD], vtile[2 * MAXD];
-  const int kb0 = (k_lo / AK) * AK;
+  const int kb0 = max((k_lo / AK) * AK, first_key);
   if (kb0 < k_end) {
     load_tile<T, MAXD, false>(src, k_pool, kb0, ktile);
     load_tile<T, MAXD, true>(src, v_pool, kb0, vtile);
@@ -174,6 +180,18 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       }
     }
   }
+  if (n_chunks > 1) {
+    // [tile][row][head][chunk][hd + 2]: the unnormalised output, the maximum and the sum; rows past the tile's
+    // queries and chunks without a visible key leave zeros and a maximum of -inf
+    float* p = part + (((size_t(blockIdx.x) * AQ + r) * nq + h) * n_chunks + blockIdx.z) * (hd + 2);
+#pragma unroll
+    for (int i = 0; i < MAXD; ++i) {
+      const int d = c16 + 16 * i;
+      if (d < hd) p[d] = acc[i];
+    }
+    if (c16 == 0) { p[hd] = m; p[hd + 1] = l; }
+    return;
+  }
   if (r < nvalid) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     T* o = out + size_t(qs + q_off + r) * (size_t(nq) * hd) + h * hd;
@@ -185,39 +203,92 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   }
 }
 
+// Joins the chunks of one query row and head: grid (tiles * AQ rows, heads), 64 threads over the head's dimensions.
+template <typename T>
+__global__ __launch_bounds__(64) void attention_generic_merge_kernel(
+    const float* __restrict__ part, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+    const int32_t* __restrict__ tiles, T* __restrict__ out, int nq, int hd, int n_chunks) {
+  const int tile = blockIdx.x / AQ, r = blockIdx.x % AQ, h = blockIdx.y;
+  const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
+  if (r >= q_len[seq] - q_off) return;
+  const float* p = part + ((size_t(blockIdx.x) * nq + h) * n_chunks) * (hd + 2);
+  float m = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c) m = fmaxf(m, p[size_t(c) * (hd + 2) + hd]);
+  float l = 0.f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float mc = p[size_t(c) * (hd + 2) + hd];
+    if (mc != -INFINITY) l += expf(mc - m) * p[size_t(c) * (hd + 2) + hd + 1];
+  }
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  T* o = out + size_t(q_start[seq] + q_off + r) * (size_t(nq) * hd) + h * hd;
+  for (int d = threadIdx.x; d < hd; d += 64) {
+    float sum = 0.f;
+    for (int c = 0; c < n_chunks; ++c) {
+      const float mc = p[size_t(c) * (hd + 2) + hd];
+      if (mc != -INFINITY) sum = fmaf(expf(mc - m), p[size_t(c) * (hd + 2) + d], sum);
+    }
+    o[d] = from_float<T>(sum * inv);
+  }
+}
+
+// How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
+// and long contexts; at most 32 chunks of at least 512 keys, whole groups of 32 keys each.
+static void generic_chunks(int n_tiles, int nq, int max_tile_ctx, int* n_chunks, int* chunk) {
+  *n_chunks = 1;
+  *chunk = 0;
+  if (n_tiles * nq >= 1024 || max_tile_ctx < 1024) return;
+  const int keys = max(512, ((max_tile_ctx + 31) / 32 + AK - 1) / AK * AK);
+  *chunk = keys;
+  *n_chunks = (max_tile_ctx + keys - 1) / keys;
+}
+
+size_t attention_generic_workspace_floats(int n_tiles, int nq, int hd, int max_tile_ctx) {
+  int n_chunks, chunk;
+  generic_chunks(n_tiles, nq, max_tile_ctx, &n_chunks, &chunk);
+  return n_chunks > 1 ? size_t(n_tiles) * AQ * nq * n_chunks * (hd + 2) : 0;
+}
+
 template <typename T>
 int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                              const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                              const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
                              void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
-                             float scale) {
+                             float scale, int max_tile_ctx, float* workspace) {
   const size_t lds = sizeof(float) * (size_t(AQ + AK) * (hd + 1) + AQ * (AK + 1));
-  dim3 grid(n_tiles, nq);
+  int n_chunks, chunk;
+  generic_chunks(n_tiles, nq, max_tile_ctx, &n_chunks, &chunk);
+  if (!workspace) n_chunks = 1;
+  dim3 grid(n_tiles, nq, n_chunks);
 #define SP_ATT(MAXD)                                                                                        \
   attention_generic_kernel<T, MAXD><<<grid, 256, lds, s>>>(                                                 \
       (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len, \
-      ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale)
+      ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk)
   if (hd <= 64) SP_ATT(4);
   else if (hd <= 128) SP_ATT(8);
   else SP_ATT(16);
 #undef SP_ATT
-  return check_launch("sp_attention (generic)");
+  if (check_launch("sp_attention (generic)")) return 1;
+  if (n_chunks == 1) return 0;
+  attention_generic_merge_kernel<T><<<dim3(n_tiles * AQ, nq), 64, 0, s>>>(workspace, q_start, q_len, tiles, (T*)out, nq, hd,
+                                                                          n_chunks);
+  return check_launch("sp_attention (generic, merge)");
 }
 
 int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, const void* k_pool,
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
-                      int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale) {
+                      int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
+                      float* workspace) {
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,
-                                           num_pages, window, scale);
+                                           num_pages, window, scale, max_tile_ctx, workspace);
   return launch_attention_generic<bf16_t>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                           q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages,
-                                          window, scale);
+                                          window, scale, max_tile_ctx, workspace);
 }
 
 }  // namespace sprout

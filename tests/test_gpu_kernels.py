@@ -317,21 +317,27 @@ def test_attention_long_prompts_whose_tiles_are_taken_in_pairs(nq, nkv, hd, page
     assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
 
 
-@pytest.mark.parametrize("far", [0, 127, 128, 1000, 2047, 2999])
-def test_attention_split_walk_finds_one_far_key(far):
-    got, want = run_attention(torch.bfloat16, 4, 2, 64, 16, [(3000, 1), (3000, 9)], kind=0, spike=(1, far), seed=far)
-    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+@pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, 0), (torch.float32, 1)])
+@pytest.mark.parametrize("far", [0, 127, 128, 511, 512, 1000, 2047, 2999])
+def test_attention_split_walk_finds_one_far_key(far, dtype, kind):
+    """Both kernels share the keys of these few tiles out over several blocks (the float32 one in chunks of 512)."""
+    got, want = run_attention(dtype, 4, 2, 64, 16, [(3000, 1), (3000, 9)], kind=kind, spike=(1, far), seed=far)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
 
 
 @pytest.mark.parametrize("nq,nkv,hd,page", [(14, 2, 64, 16), (8, 2, 128, 16), (3, 1, 32, 8)])
 @pytest.mark.parametrize("window", [None, 5000])
-def test_attention_decodes_over_long_contexts(nq, nkv, hd, page, window):
+@pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, 0), (torch.float32, 1)])
+def test_attention_decodes_over_long_contexts(nq, nkv, hd, page, window, dtype, kind):
     """One query each over thousands of keys: more chunks than one wave of the merge kernel takes in a trip
-    (several waves share them, unevenly), beside a short sequence whose chunks are nearly all empty."""
+    (several waves share them, unevenly), beside a short sequence whose chunks are nearly all empty.  The
+    float32 kernel shares the keys out in 32 chunks of 640."""
     seqs = [(9000, 1), (100, 1), (20000, 1), (4097, 1)]
-    got, want = run_attention(torch.bfloat16, nq, nkv, hd, page, seqs, window=window, kind=0, seed=hd)
+    got, want = run_attention(dtype, nq, nkv, hd, page, seqs, window=window, kind=kind, seed=hd)
     assert not np.isnan(got).any()
-    assert np.abs(got - want).max() <= 2e-2 * (1 + np.abs(want).max())
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
 
 
 @pytest.mark.parametrize("nq,nkv,hd,page,hidden", [(14, 2, 64, 16, 896), (3, 1, 32, 8, 100), (4, 4, 128, 16, 264),
