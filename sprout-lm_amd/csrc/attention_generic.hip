@@ -232,12 +232,12 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
 }
 
 // How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
-// and long contexts; at most 32 chunks of at least 512 keys, whole groups of 32 keys each.
+// and long contexts; at most 32 chunks of at least 256 keys, whole groups of 32 keys each.
 static void generic_chunks(int n_tiles, int nq, int max_tile_ctx, int* n_chunks, int* chunk) {
   *n_chunks = 1;
   *chunk = 0;
-  if (n_tiles * nq >= 1024 || max_tile_ctx < 1024) return;
-  const int keys = max(512, ((max_tile_ctx + 31) / 32 + AK - 1) / AK * AK);
+  if (n_tiles * nq >= 1024 || max_tile_ctx < 512) return;
+  const int keys = max(256, ((max_tile_ctx + 31) / 32 + AK - 1) / AK * AK);
   *chunk = keys;
   *n_chunks = (max_tile_ctx + keys - 1) / keys;
 }

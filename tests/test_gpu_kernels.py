@@ -318,9 +318,9 @@ def test_attention_long_prompts_whose_tiles_are_taken_in_pairs(nq, nkv, hd, page
 
 
 @pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, 0), (torch.float32, 1)])
-@pytest.mark.parametrize("far", [0, 127, 128, 511, 512, 1000, 2047, 2999])
+@pytest.mark.parametrize("far", [0, 127, 128, 255, 256, 511, 512, 1000, 2047, 2999])
 def test_attention_split_walk_finds_one_far_key(far, dtype, kind):
-    """Both kernels share the keys of these few tiles out over several blocks (the float32 one in chunks of 512)."""
+    """Both kernels share the keys of these few tiles out over several blocks (the float32 one in chunks of 256)."""
     got, want = run_attention(dtype, 4, 2, 64, 16, [(3000, 1), (3000, 9)], kind=kind, spike=(1, far), seed=far)
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
