@@ -27,11 +27,12 @@ static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const 
   pipe_choice(T, N, K, false, &shape, &splits);
   if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 2) return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   set_error("sp_qkv_rope_cache: no rotating epilogue for %d tokens, %d rows, K = %d", T, N, K);
   return 1;
 }
 
-// Taken where the plain product would run on blocks of 256 x 128 or 128 x 128.  Blocks of 64 x 64 have one tile
+// Taken where the plain product would run on blocks of 256 x 128, 128 x 128 or 64 x 128 (4 waves, two tile columns each).  Blocks of 64 x 64 have one tile
 // column per wave (no lane holds both of a pair), and with few tokens they fill the chip better than anything
 // larger (256 tokens at 14 + 2 + 2 heads of 64: 7.6 us and a rotation kernel of 5 against 17).  The blocks of
 // 8 waves hold 128 sums per lane, all the registers a lane has there: the epilogue's own would be spilled
@@ -40,7 +41,7 @@ bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
   if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
-  return shape == 1 || shape == 2;
+  return shape == 1 || shape == 2 || shape == 5;
 }
 
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
