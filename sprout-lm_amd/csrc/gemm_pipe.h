@@ -196,7 +196,8 @@ inline int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const 
 
 bool gemm_pipe_takes(int T, int N, int K);
 // Picks the shape (index into the list in gemm_pipe.hip) and the split of K with the least estimated time.
-void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits);
+// `paired`: the epilogue pairs tile columns, so shapes with one tile column a wave are left out.
+void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, bool paired = false);
 
 template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, typename TB>
 inline int launch_pipe(hipStream_t s, const void* x, const void* w, const void* bias, int mode, void* out, int T, int N,

@@ -28,7 +28,7 @@ static const PipeShape kPipeShapes[] = {
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
 // kernels, so large tiles win whenever they still fill the chip; products with few tiles (narrow outputs)
 // take small tiles or, when accumulating, a split of K, whose float atomics are charged per element.
-void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits) {
+void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, bool paired) {
   const int steps = K / 64;
   float best = 1e30f;
   *shape = 2;
@@ -55,15 +55,17 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits) {
     return;
   }
   for (int c : {0, 1, 2, 3, 5, 6}) {
-    // 64 x 128 on a short K only, where it fills the chip when 128 x 128 leaves CUs idle and 64 x 64 needs a second
-    // round (2,048 tokens, 1,152 rows, K = 896: 14.8 us against 17.2 and 15.1); not measured on a long K
-    if (c == 5 && steps > 16) continue;
+    // (64 x 128 fills the chip where 128 x 128 leaves CUs idle and 64 x 64 needs a second round: 2,048 tokens,
+    // 1,152 rows, K = 896: 14.8 us against 17.2 and 15.1)
+    if (c == 3 && paired) continue;   // one tile column a wave: no lane holds both of a pair
     const PipeShape& p = kPipeShapes[c];
+    // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
+    const float step_us = (c == 5 && steps > 16) ? 0.8f : p.step_us;
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;
       const int blocks = tiles * sp, full = blocks / slots, rest = blocks % slots;
-      const float per_block = float((steps + sp - 1) / sp) * p.step_us + 1.0f;
+      const float per_block = float((steps + sp - 1) / sp) * step_us + 1.0f;
       // a round that does not fill the chip runs somewhat faster: fewer blocks share the caches
       float t = full * per_block + (rest ? per_block * (0.7f + 0.3f * float(rest) / slots) : 0.f);
       if (sp > 1) t += 2.7e-6f * float(T) * float(N) * sp;      // float atomics into the output

@@ -8,7 +8,7 @@ namespace sprout {
 int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
   const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
   int shape, splits;
-  pipe_choice(T, 2 * I, K, false, &shape, &splits);
+  pipe_choice(T, 2 * I, K, false, &shape, &splits, true);
   if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
