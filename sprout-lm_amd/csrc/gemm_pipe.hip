@@ -60,7 +60,11 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     if (c == 3 && paired) continue;   // one tile column a wave: no lane holds both of a pair
     const PipeShape& p = kPipeShapes[c];
     // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
-    const float step_us = (c == 5 && steps > 16) ? 0.8f : p.step_us;
+    // and blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
+    // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180
+    // on 256 x 256, for all the round of blocks they save; with one token tile, 264 tokens, 55,296 rows,
+    // K = 5,120, their 253 us are the best there is)
+    const float step_us = steps <= 16 ? p.step_us : c == 5 ? 0.8f : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.step_us;
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;
