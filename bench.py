@@ -105,15 +105,17 @@ def measure_decode(engine, cfg, batch, context, steps, warmup):
     return elapsed / steps, spread
 
 
-def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup):
-    """`batch` requests decode while one long prompt is prefilled beside them, `chunk` tokens a step."""
+def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup, multiple=1):
+    """`batch` requests decode while one long prompt is prefilled beside them, `chunk` tokens a step; with
+    `multiple` > 1 the portion is cut back so that the step holds a whole multiple of that many tokens."""
     import random
     from dataclasses import replace
     import torch
     from sprout_lm_amd.engine import Engine
     rng = random.Random(batch + chunk)
     steps = max(1, min(steps, context // chunk - warmup - 1))
-    mixed = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk))
+    mixed = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk, step_token_multiple=multiple))
+    portion = chunk if multiple == 1 or batch + chunk <= multiple else (batch + chunk) // multiple * multiple - batch
     # requests that finish their prompt early decode while the others still prefill: leave them room
     slack = -(-batch * context // engine.options.max_batch_tokens) + 2
     ahead = steps + warmup + slack
@@ -130,15 +132,15 @@ def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup):
     for _ in range(steps):
         report = mixed.step()
         work = {w["id"]: w for w in report.work}
-        assert len(work) == batch + 1 and work["long"]["tokens"] == chunk, "timed steps must hold the batch and a portion"
+        assert len(work) == batch + 1 and work["long"]["tokens"] == portion, "timed steps must hold the batch and a portion"
     torch.cuda.synchronize()
     elapsed = (time.perf_counter() - t0) / steps
     for rid in list(mixed.scheduler.requests):
         mixed.cancel(rid)
         mixed.forget(rid)
     mixed.close()
-    return {"chunk": chunk, "batch": batch, "steps": steps, "ms_per_step": round(elapsed * 1000, 4),
-            "decode_value": round(batch / elapsed, 1), "chunk_value": round(chunk / elapsed, 1)}
+    return {"chunk": portion, "batch": batch, "steps": steps, "ms_per_step": round(elapsed * 1000, 4),
+            "decode_value": round(batch / elapsed, 1), "chunk_value": round(portion / elapsed, 1)}
 
 
 def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
@@ -236,6 +238,9 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / s, 1)
     mixed = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2) \
         if args.mixed_chunk else None
+    # the same with the step cut back to a whole multiple of the chunk (step_token_multiple): 248 + 8 tokens
+    mixed_aligned = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2,
+                                  multiple=args.mixed_chunk) if args.mixed_chunk and args.batch < args.mixed_chunk else None
     prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
     portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 2, c), 1)
                 for c in (256, 512) if c < args.prefill_tokens and not args.no_points}
@@ -271,6 +276,8 @@ def main() -> int:
         line["prefill_in_portions"] = portions
     if mixed:
         line["mixed"] = mixed
+    if mixed_aligned:
+        line["mixed_aligned"] = mixed_aligned
     if pressure:
         line["pressure"] = pressure
     print(json.dumps(line))

@@ -19,6 +19,10 @@ class EngineOptions:
     record_trace        keep every event in `engine.trace`
     decode_lookahead    launch the next step of decoded tokens before the running one has been read back
                         (not in the reference; off: every step waits for its tokens first)
+    step_token_multiple a step that would hold more tokens than this is cut back to a whole multiple of it, by
+                        shortening the portion of a prompt that crosses the line (not in the reference; 1: off).
+                        The tiled kernels work on blocks of up to 256 tokens: a step of 264 costs nearly as much
+                        as one of 512.
     """
 
     block_size: int = 16
@@ -29,6 +33,7 @@ class EngineOptions:
     prefix_caching: bool = True
     record_trace: bool = False
     decode_lookahead: bool = True
+    step_token_multiple: int = 1
 
     def __post_init__(self):
         for f in fields(self):

@@ -156,6 +156,15 @@ class Scheduler:
             start = request.seq.length
             remaining = total - start - (phase == "recompute")
             count = min(budget, 1 if phase == "decode" else self.options.prefill_chunk_size, remaining)
+            multiple = self.options.step_token_multiple
+            if multiple > 1 and phase != "decode" and count < remaining:
+                # a portion that carries the step over a whole multiple is cut back to it and closes the step
+                # (a portion that ends its prompt is left alone: the request's first token is not held back)
+                used = sum(len(w.tokens) for w in planned.values())
+                aligned = (used + count) // multiple * multiple - used
+                if 0 < aligned < count:
+                    count = aligned
+                    budget = count
             if count <= 0:
                 continue
             ok, refund = self._reserve(request, start + count, planned)

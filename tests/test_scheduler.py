@@ -58,6 +58,36 @@ def test_decode_goes_first_and_budget_cuts_prompts():
     drain(engine)
 
 
+def test_a_step_is_cut_back_to_a_whole_multiple_of_tokens():
+    """step_token_multiple: the portion that carries a step over a multiple is shortened and closes the step;
+    a portion that ends its prompt is left alone; outputs do not change."""
+    texts = {"A": "ab", "B": "0123456789abcdefghijklm", "C": "zyxwvutsr"}
+    outputs = {}
+    for multiple in (1, 4):
+        engine = make(max_batch_tokens=16, prefill_chunk_size=6, max_sequences=3, step_token_multiple=multiple,
+                      prefix_caching=False)
+        engine.add("A", prompt(texts["A"]), 6)
+        engine.step()                                  # A prefilled (2 tokens) and sampled
+        engine.add("B", prompt(texts["B"]), 2)
+        engine.add("C", prompt(texts["C"]), 2)
+        report = engine.step()
+        work = [(w["id"], w["phase"], w["tokens"]) for w in report.work]
+        if multiple == 1:
+            assert work == [("A", "decode", 1), ("B", "prefill", 6), ("C", "prefill", 6)]
+        else:                                          # 1 + 6 = 7 crosses 4: B is cut to 3 and closes the step
+            assert work == [("A", "decode", 1), ("B", "prefill", 3)]
+        reports = [report] + drain(engine)
+        if multiple > 1:
+            for r in reports:                          # every other step: a whole multiple, or a prompt ends in it
+                total = sum(w["tokens"] for w in r.work)
+                ends = any(w["phase"] == "prefill" and w["from"] + w["tokens"] == len(texts[w["id"]]) for w in r.work)
+                assert total <= multiple or total % multiple == 0 or ends, (total, r.work)
+        outputs[multiple] = {rid: engine.result(rid)["output"] for rid in "ABC"}
+        for rid, n in (("A", 6), ("B", 2), ("C", 2)):
+            assert outputs[multiple][rid] == engine.model.greedy(prompt(texts[rid]), n)
+    assert outputs[1] == outputs[4]
+
+
 def test_prefix_sharing_reuses_pages_and_recomputes_the_last_prompt_token():
     engine = make(block_size=2, prefill_chunk_size=8)
     p = prompt("abcd")                             # exactly two full pages
