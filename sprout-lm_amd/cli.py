@@ -78,7 +78,8 @@ def cmd_generate(args) -> int:
         prompt = None
     runtime = create_runtime(args.model, args.dtype, max_context_tokens=args.kv_tokens, block_size=args.block_size,
                              max_sequences=args.max_sequences, max_batch_tokens=args.max_batch_tokens,
-                             prefill_chunk_size=args.prefill_chunk_size, prefix_caching=not args.no_prefix_caching)
+                             prefill_chunk_size=args.prefill_chunk_size, prefix_caching=not args.no_prefix_caching,
+                             step_token_multiple=args.step_token_multiple)
     engine = runtime.engine
     if prompt is None:
         prompt = [rng.randrange(engine.model.vocab_size) for _ in range(args.prompt_len)]
@@ -191,6 +192,8 @@ def main(argv=None) -> int:
     gen.add_argument("--max-sequences", type=int, default=_env_int("MAX_SEQUENCES", 4))
     gen.add_argument("--max-batch-tokens", type=int, default=2048)
     gen.add_argument("--prefill-chunk-size", type=int, default=_env_int("PREFILL_CHUNK_SIZE", 512))
+    gen.add_argument("--step-token-multiple", type=int, default=1,
+                     help="cut a step of more tokens than this back to a whole multiple of it (1: off)")
     gen.add_argument("--no-prefix-caching", action="store_true")
     gen.add_argument("--report", default=os.environ.get("REPORT_PATH"), help="write the full JSON report here")
     gen.add_argument("--quiet", action="store_true")

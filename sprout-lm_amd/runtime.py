@@ -27,7 +27,8 @@ class Runtime:
 
 def create_runtime(model_directory: str, dtype: str = "bfloat16", max_context_tokens: int = 2048,
                    block_size: int = 16, max_sequences: int = 4, max_batch_tokens: int = 2048,
-                   prefill_chunk_size: int = 512, prefix_caching: bool = True, record_trace: bool = False) -> Runtime:
+                   prefill_chunk_size: int = 512, prefix_caching: bool = True, record_trace: bool = False,
+                   step_token_multiple: int = 1) -> Runtime:
     """`max_context_tokens` sizes the cache pool (the reference's KV_TOKENS): ceil(tokens / block_size) pages."""
     from .engine.engine import Engine
     if isinstance(max_context_tokens, bool) or not isinstance(max_context_tokens, int) or max_context_tokens < 1:
@@ -35,7 +36,7 @@ def create_runtime(model_directory: str, dtype: str = "bfloat16", max_context_to
     options = EngineOptions(block_size=block_size, num_blocks=-(-max_context_tokens // block_size),
                             max_sequences=max_sequences, max_batch_tokens=max_batch_tokens,
                             prefill_chunk_size=prefill_chunk_size, prefix_caching=prefix_caching,
-                            record_trace=record_trace)
+                            record_trace=record_trace, step_token_multiple=step_token_multiple)
     engine = Engine.from_folder(model_directory, dtype, options)
     if max_context_tokens > engine.model.max_positions * max_sequences:
         pass  # a pool larger than one request can use is allowed: it serves several requests
