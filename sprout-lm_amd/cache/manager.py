@@ -15,6 +15,7 @@ from .pages import PageError, PagePool
 from .spec import PagedKVSpec, StateSpec
 
 FREED = -1  # block-table entry of a page that a window has passed
+_DTYPE_BYTES = {"float32": 4, "bfloat16": 2, "float16": 2, "int32": 4, "float64": 8, "int64": 8}
 
 
 @dataclass
@@ -43,6 +44,9 @@ class SequenceCache:
         SequenceCache._next_uid += 1
         self.uid = SequenceCache._next_uid      # never reused, unlike id(): caches keyed by it stay valid
         self.blocks: list[list[int]] = [[] for _ in manager.groups]
+        # bumped whenever a group's table changes (a page more, a page given back): mirrors of the table on
+        # the device are rewritten only then
+        self.table_versions: list[int] = [0 for _ in manager.groups]
         self.length = 0
         self.state_slot = state_slot
         self.released = False
@@ -111,13 +115,26 @@ class CacheManager:
             g.k = torch.zeros((n, self.num_blocks, kv, self.block_size, hd), dtype=dtype, device=device)
             g.v = torch.zeros((n, self.num_blocks, kv, hd, self.block_size), dtype=dtype, device=device)
         for g in self.state_groups:
-            g.data = torch.zeros((len(g.slots), self.max_sequences, *g.spec.shape),
+            # one slot more than requests can hold: `spare_state_slot`, where the padding rows of a recorded
+            # step keep their state, so that no part has to tell them from real rows
+            g.data = torch.zeros((len(g.slots), self.max_sequences + 1, *g.spec.shape),
                                  dtype=getattr(torch, g.spec.dtype), device=device)
 
+    @property
+    def spare_state_slot(self) -> int:
+        """A state slot that no request ever holds (the last row of every state tensor)."""
+        return self.max_sequences
+
     def storage_bytes(self, element_size: int) -> int:
+        """Device bytes of every pool and state tensor for cache elements of `element_size` bytes."""
         total = 0
         for g in self.groups:
             total += 2 * len(g.slots) * self.num_blocks * g.spec.kv_heads * self.block_size * g.spec.head_dim * element_size
+        for g in self.state_groups:
+            count = 1
+            for n in g.spec.shape:
+                count *= n
+            total += len(g.slots) * (self.max_sequences + 1) * count * _DTYPE_BYTES.get(g.spec.dtype, 4)
         return total
 
     # ------------------------------------------------------------------ sequences
@@ -156,8 +173,9 @@ class CacheManager:
             entry.last_used = self._clock
             for g, page in zip(self.groups, entry.pages):
                 g.pool.retain(page)
-            for blocks, page in zip(seq.blocks, entry.pages):
+            for gi, (blocks, page) in enumerate(zip(seq.blocks, entry.pages)):
                 blocks.append(page)
+                seq.table_versions[gi] += 1
             seq.prefix_keys.append(key)
             seq.length = end
             end += bs
@@ -228,8 +246,10 @@ class CacheManager:
                     for gj, p in reversed(taken):
                         self.groups[gj].pool.release(p)
                         seq.blocks[gj].pop()
+                        seq.table_versions[gj] += 1
                     return False
                 seq.blocks[gi].append(page)
+                seq.table_versions[gi] += 1
                 taken.append((gi, page))
         return True
 
@@ -239,7 +259,7 @@ class CacheManager:
         if new_length > min((len(b) for b in seq.blocks), default=new_length // self.block_size + 1) * self.block_size:
             raise PageError("Committed more tokens than pages were reserved for.")
         seq.length = new_length
-        for g, blocks in zip(self.groups, seq.blocks):
+        for gi, (g, blocks) in enumerate(zip(self.groups, seq.blocks)):
             if g.spec.window is None:
                 continue
             # the next token (position new_length) reads keys >= new_length - window + 1
@@ -248,6 +268,7 @@ class CacheManager:
                 if blocks[i] != FREED:
                     g.pool.release(blocks[i])
                     blocks[i] = FREED
+                    seq.table_versions[gi] += 1
 
     def release(self, seq: SequenceCache) -> None:
         if seq.released:

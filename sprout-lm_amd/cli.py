@@ -79,12 +79,14 @@ def cmd_generate(args) -> int:
     runtime = create_runtime(args.model, args.dtype, max_context_tokens=args.kv_tokens, block_size=args.block_size,
                              max_sequences=args.max_sequences, max_batch_tokens=args.max_batch_tokens,
                              prefill_chunk_size=args.prefill_chunk_size, prefix_caching=not args.no_prefix_caching,
-                             step_token_multiple=args.step_token_multiple)
+                             step_token_multiple=args.step_token_multiple, weight_limit_mib=args.weight_limit_mib,
+                             reserve_mib=args.reserve_mib, strict_tensors=args.strict_tensors)
     engine = runtime.engine
     if prompt is None:
         prompt = [rng.randrange(engine.model.vocab_size) for _ in range(args.prompt_len)]
     load_ms = (time.perf_counter() - started) * 1000
-    print(json.dumps({"phase": "ready", "name": runtime.name, "input": prompt, "load_ms": round(load_ms, 1)}), flush=True)
+    print(json.dumps({"phase": "ready", "name": runtime.name, "input": prompt, "load_ms": round(load_ms, 1),
+                      "notes": getattr(engine.model, "load_notes", [])}), flush=True)
     engine.add("cli", prompt, args.max_new_tokens, temperature=args.temperature, seed=args.seed,
                ignore_eos=args.ignore_eos)
     rounds, first_token_ms = [], None
@@ -195,6 +197,12 @@ def main(argv=None) -> int:
     gen.add_argument("--step-token-multiple", type=int, default=1,
                      help="cut a step of more tokens than this back to a whole multiple of it (1: off)")
     gen.add_argument("--no-prefix-caching", action="store_true")
+    gen.add_argument("--weight-limit-mib", type=int, default=_env_int("CUDA_WEIGHT_LIMIT_MIB", 0),
+                     help="most device memory the weights may take (0: no limit)")
+    gen.add_argument("--reserve-mib", type=int, default=_env_int("CUDA_RESERVE_MIB", 1024),
+                     help="device memory that must stay free after weights and cache pools")
+    gen.add_argument("--strict-tensors", action="store_true",
+                     help="refuse a checkpoint that holds tensors the model does not ask for")
     gen.add_argument("--report", default=os.environ.get("REPORT_PATH"), help="write the full JSON report here")
     gen.add_argument("--quiet", action="store_true")
     gen.set_defaults(run=cmd_generate)

@@ -59,7 +59,9 @@ class Engine:
         from .runner import ModelRunner
         options = EngineOptions(**{**(asdict(options) if options else {}), **overrides})
         runner = ModelRunner.from_folder(folder, dtype, block_size=options.block_size, num_blocks=options.num_blocks,
-                                         max_sequences=options.max_sequences, prefix_caching=options.prefix_caching)
+                                         max_sequences=options.max_sequences, prefix_caching=options.prefix_caching,
+                                         strict_tensors=options.strict_tensors,
+                                         weight_limit_mib=options.weight_limit_mib, reserve_mib=options.reserve_mib)
         return cls(runner, options)
 
     @classmethod
@@ -69,7 +71,8 @@ class Engine:
         options = EngineOptions(**{**(asdict(options) if options else {}), **overrides})
         runner = ModelRunner.from_config(config, seed, dtype, block_size=options.block_size,
                                          num_blocks=options.num_blocks, max_sequences=options.max_sequences,
-                                         prefix_caching=options.prefix_caching)
+                                         prefix_caching=options.prefix_caching,
+                                         weight_limit_mib=options.weight_limit_mib, reserve_mib=options.reserve_mib)
         return cls(runner, options)
 
     # ------------------------------------------------------------------ the reference's surface

@@ -97,8 +97,9 @@ class _DecodeGraph:
     def fill(self, entries, params, counters, sources=None) -> None:
         """Write this step's values into the pinned staging buffer.
 
-        Block-table rows are rewritten only when a row's sequence or its number of pages has changed
-        since the last step (a steady decode batch gains a page every `block_size` steps).
+        Block-table rows are rewritten only when a row's sequence or its table has changed since the last
+        step (a steady decode batch gains a page every `block_size` steps; a windowed group also gives pages
+        back, which the cache manager counts in the table's version).
         `sources[i] >= 0`: entry i's token is row sources[i] of an earlier step's sampled tokens, which
         the host does not know yet (its `tokens[0]` is None)."""
         cache, h, n, S = self.runner.cache, self.h, len(entries), self.S
@@ -115,8 +116,9 @@ class _DecodeGraph:
         h["temperature"].view(np.float32)[:n] = [p.temperature for p in params]
         h["seed"].view(np.int64)[:n] = [p.seed for p in params]
         if n != self._filled:
-            for name in ("token_ids", "positions", "state_slots", "temperature"):
+            for name in ("token_ids", "positions", "temperature"):
                 h[name][n:] = 0
+            h["state_slots"][n:] = cache.spare_state_slot     # dummy rows keep their state where no request lives
             h["feed_source"][n:] = -1
             h["ctx_len"][n:] = 1
             self._rows = [None] * S
@@ -130,10 +132,11 @@ class _DecodeGraph:
             pages = np.empty(n, dtype=np.int32)
             for i, e in enumerate(entries):
                 blocks = e.seq.blocks[g]
-                key = (e.seq.uid, g, len(blocks))
+                key = (e.seq.uid, g, e.seq.table_versions[g])
                 if self._rows[i] is None or self._rows[i].get(g) != key:
                     nb = min(len(blocks), self.max_blocks)
                     tables[i, :nb] = blocks[:nb]
+                    tables[i, nb:] = -1
                     if self._rows[i] is None:
                         self._rows[i] = {}
                     self._rows[i][g] = key
@@ -156,6 +159,11 @@ class _DecodeGraph:
             self.graph.replay()
 
     def _body(self):
+        # What a part computes once per step for all layers (the rotation table) belongs to one step: the
+        # context of a graph outlives its steps, so the table is forgotten here and its kernel is recorded
+        # with the rest.  (Kept, the eager run before the capture would leave a table that the capture then
+        # finds: the graph would hold no kernel for it and rotate every later step by the first step's angles.)
+        self.ctx.shared.clear()
         self.logits = self.runner.forward(self.ctx)
         ops.sample(self.logits, self.sampled, self.sample_ws, self.temperature, self.seed, self.counter)
 
@@ -191,7 +199,9 @@ class DecodeGraphs:
 
     def usable(self, entries) -> bool:
         runner = self.runner
-        return (runner.parts.graph_safe and not runner.cache.state_groups and len(entries) > 0
+        # the parts decide: a model whose parts all launch a one-token step from device-resident values alone
+        # replays, whatever its cache groups are (pages of a window, state of fixed size)
+        return (runner.parts.graph_safe and len(entries) > 0
                 and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries))
 
     def launch(self, entries, params, counters, feed=None) -> "PendingDecode":
@@ -219,7 +229,7 @@ class DecodeGraphs:
         state.fill(entries, params, counters, sources)
         state.launch(previous)
         self.replays += 1
-        pending = PendingDecode(state.sampled, n, self._host_tokens(S))
+        pending = PendingDecode(state.sampled, n, self._host_tokens(S), state.logits)
         for e in entries:
             runner.cache.commit(e.seq, e.seq.length + 1)
         return pending
@@ -241,8 +251,9 @@ class DecodeGraphs:
 class PendingDecode:
     """A launched decode step: the sampled tokens are on their way to the host."""
 
-    def __init__(self, sampled: torch.Tensor, n: int, host: torch.Tensor):
+    def __init__(self, sampled: torch.Tensor, n: int, host: torch.Tensor, logits: torch.Tensor | None = None):
         self.sampled, self.n = sampled, n       # the step's device buffer: valid until the same graph runs again
+        self.logits = logits                    # float32 [rows of the graph, vocab], likewise; rows 0 .. n - 1 count
         self._host = host
         host[:n].copy_(sampled[:n], non_blocking=True)
         self._done = torch.cuda.Event()

@@ -15,6 +15,7 @@ from ..registry import build_model_plan, load_config
 from ..weights.loader import load_named_tensors
 from ..weights.random_init import random_tensors
 from .batch import CacheSlotView, DescriptorStager, StepEntry, Workspace, build_context
+from .memory import MemoryBudget, check_budget, free_device_bytes, weight_bytes
 
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
@@ -44,11 +45,18 @@ class ModelRunner:
     """
 
     def __init__(self, plan: ModelPlan, tensors: dict, dtype: torch.dtype, device, block_size: int, num_blocks: int,
-                 max_sequences: int, prefix_caching: bool = False, stop_token_ids=None, use_graphs: bool = True):
+                 max_sequences: int, prefix_caching: bool = False, stop_token_ids=None, use_graphs: bool = True,
+                 budget: MemoryBudget | None = None, parts=None):
+        """`tensors`: the plan's tensors on the device, by checkpoint name (the dict is emptied as parts take
+        them).  The cache pools are counted against the free device memory before they are allocated."""
         self.plan, self.dtype, self.device = plan, dtype, device
-        self.parts = plan.instantiate()
-        self.parts.bind(tensors, device, dtype)
+        self.parts = parts if parts is not None else plan.instantiate()
+        self.budget = budget or MemoryBudget()
         self.cache = CacheManager(self.parts.cache_slot_specs, block_size, num_blocks, max_sequences, prefix_caching)
+        if torch.device(device).type == "cuda":
+            check_budget(0, self.cache.storage_bytes(dtype.itemsize), free_device_bytes(device), self.budget,
+                         "cache pools (the weights are resident already)")
+        self.parts.bind(tensors, device, dtype)
         self.cache.attach_storage(dtype, device)
         self.workspace = Workspace(device)
         self.stager = DescriptorStager(device)
@@ -56,27 +64,55 @@ class ModelRunner:
         self.attention_kind = 1 if dtype == torch.float32 else 0
         self.vocab_size, self.hidden_size, self.max_positions = plan.vocab_size, plan.hidden_size, plan.max_positions
         self.use_graphs = use_graphs
+        self.load_notes: list[str] = []    # what the loader saw and left alone (tensors nobody asked for)
         self._graphs = None
         self._sampler = None
 
     # ------------------------------------------------------------------ construction
+    @staticmethod
+    def preflight(parts, dtype: torch.dtype, device, block_size: int, num_blocks: int, max_sequences: int,
+                  budget: MemoryBudget, stored: dict | None = None) -> tuple[int, int]:
+        """Count the weights and the cache pools of a model that is not loaded yet against the device's free
+        memory; raises MemoryBudgetError if they do not fit.  Returns (weight bytes, pool bytes)."""
+        weights = weight_bytes(parts.expected_tensors(), dtype, stored)
+        pools = CacheManager(parts.cache_slot_specs, block_size, num_blocks, max_sequences, False).storage_bytes(dtype.itemsize)
+        check_budget(weights, pools, free_device_bytes(device), budget)
+        return weights, pools
+
     @classmethod
-    def from_folder(cls, folder: str, dtype="bfloat16", **cache_options) -> "ModelRunner":
+    def from_folder(cls, folder: str, dtype="bfloat16", strict_tensors: bool = False, weight_limit_mib: int = 0,
+                    reserve_mib: int | None = None, **cache_options) -> "ModelRunner":
+        """`strict_tensors`: tensors in the checkpoint that the model does not ask for are an error (by
+        default they are left unread, as the reference leaves them: src/safetensors.ts:70-83)."""
         device = require_gpu()
         dtype = parse_dtype(dtype)
         config = load_config(folder)
         plan = build_model_plan(config)
-        tensors = load_named_tensors(folder, plan.expected_tensors(), set(plan.ignorable_tensors), dtype, device)
-        return cls(plan, tensors, dtype, device, stop_token_ids=stop_ids_of_folder(folder, plan), **cache_options)
+        parts = plan.instantiate()
+        budget = MemoryBudget(weight_limit_mib, MemoryBudget().reserve_mib if reserve_mib is None else reserve_mib)
+        sizes = {k: cache_options[k] for k in ("block_size", "num_blocks", "max_sequences")}
+        notes: list[str] = []
+        tensors = load_named_tensors(
+            folder, parts.expected_tensors(), set(plan.ignorable_tensors), dtype, device, strict=strict_tensors,
+            notes=notes, before_read=lambda stored: cls.preflight(parts, dtype, device, budget=budget, stored=stored, **sizes))
+        runner = cls(plan, tensors, dtype, device, stop_token_ids=stop_ids_of_folder(folder, plan), budget=budget,
+                     parts=parts, **cache_options)
+        runner.load_notes = notes
+        return runner
 
     @classmethod
-    def from_config(cls, config, seed: int, dtype="bfloat16", **cache_options) -> "ModelRunner":
+    def from_config(cls, config, seed: int, dtype="bfloat16", weight_limit_mib: int = 0, reserve_mib: int | None = None,
+                    **cache_options) -> "ModelRunner":
         """Random weights drawn on the device (for benchmarks; a model folder is not written)."""
         device = require_gpu()
         dtype = parse_dtype(dtype)
         plan = build_model_plan(config)
-        tensors = random_tensors(plan.expected_tensors(), seed, dtype=dtype, device=device)
-        return cls(plan, tensors, dtype, device, **cache_options)
+        parts = plan.instantiate()
+        budget = MemoryBudget(weight_limit_mib, MemoryBudget().reserve_mib if reserve_mib is None else reserve_mib)
+        cls.preflight(parts, dtype, device, budget=budget,
+                      **{k: cache_options[k] for k in ("block_size", "num_blocks", "max_sequences")})
+        tensors = random_tensors(parts.expected_tensors(), seed, dtype=dtype, device=device)
+        return cls(plan, tensors, dtype, device, budget=budget, parts=parts, **cache_options)
 
     # ------------------------------------------------------------------ the step
     def _slot_view(self, ctx, call) -> CacheSlotView | None:

@@ -115,8 +115,20 @@ class ModelParts:
         return out
 
     def bind(self, tensors: dict, device, dtype) -> None:
+        """Hand every part its tensors.  They are taken out of `tensors` as they go: a part that joins
+        several of them into one (q, k and v; gate and up) then holds the only copy, and the separate ones
+        are freed layer by layer instead of all at the end."""
+        again: dict = {}        # tensors that two parts name (weights shared by name)
+        names = [prefix + local for prefix, part in self._named for local in part.tensors()]
+        shared = {n for n in names if names.count(n) > 1}
         for prefix, part in self._named:
-            part.bind({local: tensors[prefix + local] for local in part.tensors()})
+            mine = {}
+            for local in part.tensors():
+                name = prefix + local
+                mine[local] = again[name] if name in again else tensors.pop(name)
+                if name in shared:
+                    again[name] = mine[local]
+            part.bind(mine)
             part.prepare(device, dtype)
         if getattr(self.head, "tied", False):
             self.head.tie(self.embedding.w["weight"])

@@ -28,16 +28,18 @@ class Runtime:
 def create_runtime(model_directory: str, dtype: str = "bfloat16", max_context_tokens: int = 2048,
                    block_size: int = 16, max_sequences: int = 4, max_batch_tokens: int = 2048,
                    prefill_chunk_size: int = 512, prefix_caching: bool = True, record_trace: bool = False,
-                   step_token_multiple: int = 1) -> Runtime:
-    """`max_context_tokens` sizes the cache pool (the reference's KV_TOKENS): ceil(tokens / block_size) pages."""
+                   step_token_multiple: int = 1, weight_limit_mib: int = 0, reserve_mib: int = 1024,
+                   strict_tensors: bool = False) -> Runtime:
+    """`max_context_tokens` sizes the cache pool (the reference's KV_TOKENS): ceil(tokens / block_size) pages.
+    A pool larger than one request can use is allowed: it serves several requests.  `weight_limit_mib` and
+    `reserve_mib` are the reference's CUDA_WEIGHT_LIMIT_MIB and CUDA_RESERVE_MIB."""
     from .engine.engine import Engine
     if isinstance(max_context_tokens, bool) or not isinstance(max_context_tokens, int) or max_context_tokens < 1:
         raise ValueError("Invalid max_context_tokens.")
     options = EngineOptions(block_size=block_size, num_blocks=-(-max_context_tokens // block_size),
                             max_sequences=max_sequences, max_batch_tokens=max_batch_tokens,
                             prefill_chunk_size=prefill_chunk_size, prefix_caching=prefix_caching,
-                            record_trace=record_trace, step_token_multiple=step_token_multiple)
+                            record_trace=record_trace, step_token_multiple=step_token_multiple,
+                            weight_limit_mib=weight_limit_mib, reserve_mib=reserve_mib, strict_tensors=strict_tensors)
     engine = Engine.from_folder(model_directory, dtype, options)
-    if max_context_tokens > engine.model.max_positions * max_sequences:
-        pass  # a pool larger than one request can use is allowed: it serves several requests
     return Runtime(engine, f"{model_directory} ({engine.model.plan.architecture}, {dtype}, HIP forward + device KV)")

@@ -64,9 +64,15 @@ class Checkpoint:
     def info(self, name: str) -> TensorInfo:
         return self._infos[name][1]
 
-    def read(self, name: str) -> torch.Tensor:
+    def dtype(self, name: str) -> torch.dtype:
+        """The torch dtype `name` is stored in."""
+        from .safetensors_io import stored_dtype
+        return stored_dtype(self._infos[name][1].dtype)
+
+    def read(self, name: str, copy: bool = True) -> torch.Tensor:
+        """`copy=False`: a view of the file's mapping, to be used before the next tensor is read."""
         shard, _ = self._infos[name]
-        return self._file(shard).read(name)
+        return self._file(shard).read(name, copy)
 
     def close(self):
         for file in self._open.values():

@@ -9,7 +9,13 @@ from .checkpoint import Checkpoint
 
 
 class WeightError(ValueError):
-    """Lists missing tensors, unexpected tensors and wrong shapes of a checkpoint together."""
+    """Lists missing tensors, unexpected tensors and wrong shapes of a checkpoint together.
+
+    Tensors that nobody asked for are no error by themselves (the reference reads what it asks for and
+    nothing else, src/safetensors.ts:70-83); they are listed when something else is wrong, because a tensor
+    that is "missing" and one that is "unexpected" are often the same tensor under two names, and they are
+    an error of their own only for a strict load.
+    """
 
     def __init__(self, folder, missing, unexpected, wrong_shape, wrong_dtype=()):
         self.missing, self.unexpected = list(missing), list(unexpected)
@@ -56,8 +62,14 @@ def target_dtype(stored: torch.dtype, kind: str, compute: torch.dtype) -> torch.
 
 
 def load_named_tensors(folder: str, expected: dict[str, TensorSpec], ignorable: set[str],
-                       compute: torch.dtype, device) -> dict[str, torch.Tensor]:
-    """Read exactly the tensors in `expected`; anything else in the checkpoint must be in `ignorable`."""
+                       compute: torch.dtype, device, strict: bool = False, notes: list | None = None,
+                       before_read=None) -> dict[str, torch.Tensor]:
+    """Read exactly the tensors in `expected`, by name, each with the shape its part expects.
+
+    Other tensors in the checkpoint are left unread (a line in `notes` names them); with `strict` they are
+    an error unless `ignorable` lists them.  Everything wrong with the checkpoint is reported in one
+    WeightError.  `before_read(stored)`: called once the header has been checked and before any tensor is
+    read, with the dtype each expected tensor is stored in (the place to count memory)."""
     with Checkpoint(folder) as ckpt:
         present = set(ckpt.names())
         missing = sorted(n for n in expected if n not in present)
@@ -72,10 +84,20 @@ def load_named_tensors(folder: str, expected: dict[str, TensorSpec], ignorable: 
             is_int = info.dtype in ("I32", "I64")
             if is_int != (spec.kind == "int_table"):
                 wrong_dtype.append((name, info.dtype))
-        if missing or unexpected or wrong_shape or wrong_dtype:
+        if missing or wrong_shape or wrong_dtype or (strict and unexpected):
             raise WeightError(folder, missing, unexpected, wrong_shape, wrong_dtype)
+        if unexpected and notes is not None:
+            notes.append(f"{len(unexpected)} tensors of the checkpoint are not part of the model and were left "
+                         f"unread: " + ", ".join(unexpected[:8]) + (" ..." if len(unexpected) > 8 else ""))
+        if before_read is not None:
+            before_read({name: ckpt.dtype(name) for name in expected})
         out = {}
         for name, spec in expected.items():
-            t = ckpt.read(name)
-            out[name] = t.to(device=device, dtype=target_dtype(t.dtype, spec.kind, compute)).contiguous()
+            # straight from the file's mapping to the device: no copy on the host in between
+            view = ckpt.read(name, copy=False)
+            kept = view.to(device=device, dtype=target_dtype(view.dtype, spec.kind, compute)).contiguous()
+            if kept.data_ptr() == view.data_ptr():
+                kept = kept.clone()       # a host tensor of the stored dtype: it must not live in the mapping
+            out[name] = kept
+            del view
         return out

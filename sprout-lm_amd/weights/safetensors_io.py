@@ -33,6 +33,11 @@ _NAMES = {torch.float32: "F32", torch.bfloat16: "BF16", torch.float16: "F16",
 MAX_HEADER = 16 * 1024 * 1024
 
 
+def stored_dtype(name: str) -> torch.dtype:
+    """The torch dtype of a safetensors dtype name."""
+    return _DTYPES[name][1]
+
+
 @dataclass(frozen=True)
 class TensorInfo:
     dtype: str
@@ -86,7 +91,8 @@ class SafetensorsFile:
                 raise SafetensorsError(f"{path}: safetensors data size does not match its header.")
             self.entries = entries
             self._start = 8 + header_size
-            self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_READ) if size else None
+            # a private mapping: nothing is ever written to it, but tensors may then view its pages directly
+            self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_COPY) if size else None
         except Exception:
             self._file.close()
             raise
@@ -97,13 +103,14 @@ class SafetensorsFile:
     def info(self, name: str) -> TensorInfo:
         return self.entries[name]
 
-    def read(self, name: str) -> torch.Tensor:
-        """The tensor in its stored dtype, copied out of the mapping."""
+    def read(self, name: str, copy: bool = True) -> torch.Tensor:
+        """The tensor in its stored dtype.  `copy=False`: a view of the file's mapping (no host copy), which
+        must be dropped before the file is closed; meant for `view.to(device)` right away."""
         info = self.entries[name]
         _, torch_dtype, np_dtype = _DTYPES[info.dtype]
         count = (info.end - info.begin) // np_dtype.itemsize
         array = np.frombuffer(self._map, dtype=np_dtype, count=count, offset=self._start + info.begin)
-        tensor = torch.from_numpy(array.copy())
+        tensor = torch.from_numpy(array.copy() if copy else array)
         if info.dtype == "BF16":
             tensor = tensor.view(torch.bfloat16)
         return tensor.reshape(info.shape)

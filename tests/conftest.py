@@ -7,8 +7,9 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# the reference checkout's own fixture; SPROUT_REFERENCE_FIXTURE names a copy where the checkout is not mounted
-REFERENCE_FIXTURE = os.environ.get("SPROUT_REFERENCE_FIXTURE", "/root/reference/test/fixtures/qwen-tiny")
+# test vectors that the reference's own tests hold: the copy kept beside the tests, or the folder that
+# SPROUT_REFERENCE_FIXTURE names
+REFERENCE_FIXTURE = os.environ.get("SPROUT_REFERENCE_FIXTURE") or os.path.join(ROOT, "tests", "fixtures", "reference_qwen_tiny")
 
 
 def pytest_configure(config):
@@ -19,9 +20,8 @@ def pytest_configure(config):
 def reference_fixture():
     """The reference's own tiny Qwen2 with logits computed by an independent library.
 
-    Read in place (never copied); tests that need it are skipped where the
-    reference checkout is not mounted.
+    Tests that need it are skipped where the folder is not there.
     """
     if not os.path.isfile(os.path.join(REFERENCE_FIXTURE, "reference.json")):
-        pytest.skip("reference fixture not mounted")
+        pytest.skip(f"no reference fixture at {REFERENCE_FIXTURE}")
     return REFERENCE_FIXTURE

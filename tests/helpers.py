@@ -59,13 +59,13 @@ def plain_model(folder: str, dtype: str):
 _LOGIT_CACHE: dict = {}
 
 
-def plain_logits(folder: str, dtype: str, tokens) -> np.ndarray:
-    """Logits of the plain implementation at every position of `tokens` (cached per sequence)."""
-    key = (folder, dtype, tuple(tokens))
+def plain_logits(folder: str, dtype: str, tokens, rows=None) -> np.ndarray:
+    """Logits of the plain implementation at every position of `tokens`, or at `rows` only (cached per sequence)."""
+    key = (folder, dtype, tuple(tokens), None if rows is None else tuple(rows))
     if key not in _LOGIT_CACHE:
         cfg, w = plain_model(folder, dtype)
         store = P.bf16_round if dtype == "bfloat16" else P.f32
-        _LOGIT_CACHE[key] = P.forward_logits(w, cfg, list(tokens), store=store)
+        _LOGIT_CACHE[key] = P.forward_logits(w, cfg, list(tokens), store=store, rows=rows)
     return _LOGIT_CACHE[key]
 
 

@@ -126,8 +126,9 @@ def decoder_layer(x, w, layer, cfg, positions, store=f32):
     return x
 
 
-def forward_logits(w, cfg, tokens, store=f32, first_position=0):
-    """Logits [len(tokens), vocab] at every position (src/qwen.ts:158-204 over a whole sequence).
+def forward_logits(w, cfg, tokens, store=f32, first_position=0, rows=None):
+    """Logits [len(tokens), vocab] at every position (src/qwen.ts:158-204 over a whole sequence), or at the
+    positions `rows` only (the reference computes them where they are asked for, src/qwen.ts:203).
 
     The output matrix is the embedding when tie_word_embeddings (src/qwen.ts:152).
     """
@@ -136,6 +137,8 @@ def forward_logits(w, cfg, tokens, store=f32, first_position=0):
     x = f32(np.asarray(w["model.embed_tokens.weight"])[tokens])
     for layer in range(cfg["num_hidden_layers"]):
         x = decoder_layer(x, w, layer, cfg, positions, store)
+    if rows is not None:
+        x = x[np.asarray(rows, dtype=np.int64)]
     n = store(rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]))
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return linear(n, head)

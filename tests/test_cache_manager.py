@@ -73,6 +73,24 @@ def test_window_gives_pages_back_as_it_passes_them():
     assert cache.free_pages() == [5]
 
 
+def test_table_versions_change_exactly_when_a_table_changes():
+    """Mirrors of a block table on the device are rewritten when its version moves: it must move with every page
+    that is added or given back (also by a window, which leaves the table's length as it was), and only then."""
+    cache = CacheManager([FULL, WINDOWED], block_size=4, num_blocks=6, max_sequences=2, prefix_caching=False)
+    seq = cache.create()
+    seen = [(list(b), v) for b, v in zip(seq.blocks, seq.table_versions)]
+    for length in range(1, 25):
+        assert cache.reserve(seq, length)
+        cache.commit(seq, length)
+        for gi, (blocks, version) in enumerate(zip(seq.blocks, seq.table_versions)):
+            assert (blocks != seen[gi][0]) == (version != seen[gi][1]), f"group {gi} at length {length}"
+            seen[gi] = (list(blocks), version)
+    assert FREED in seq.blocks[1] and FREED not in seq.blocks[0]
+    other = cache.create()
+    assert not cache.reserve(other, 24)                    # group 0 has no page left: nothing is kept
+    assert other.blocks == [[], []]
+
+
 def test_prefix_reuse_leaves_the_last_token_to_compute():
     cache = CacheManager([FULL], block_size=2, num_blocks=8, max_sequences=4)
     tokens = [5, 6, 7, 8]                                   # exactly two pages

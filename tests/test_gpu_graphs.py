@@ -1,0 +1,117 @@
+"""Decode steps replayed from recorded HIP graphs, compared by their logits with the plain implementation.
+
+Generation runs every step of single tokens through `ModelRunner.launch_decode`; the other logits tests step
+eagerly.  Here the recorded path itself is held to the plain side: its own descriptor builder, padded rows,
+context buckets, and the kernels that only steps of decoded tokens take at real layer sizes."""
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+def plain_rows(folder, tokens, rows):
+    """bfloat16-rounded plain logits of `tokens` at `rows`, with the weights widened once (exactly) to float64."""
+    cfg, w = H.plain_model(folder, "bfloat16")
+    key = ("f64", folder)
+    if key not in H._PLAIN_CACHE:
+        H._PLAIN_CACHE[key] = {k: v.astype(np.float64) for k, v in w.items()}
+    return P.forward_logits(H._PLAIN_CACHE[key], cfg, list(tokens), store=P.bf16_round, rows=rows)
+
+
+def decode_through_graphs(runner, seqs, tokens, fed, steps, folder, label):
+    """Feed token `fed[r]` of every request r in `seqs` as one recorded step, `steps` times; compare the step's
+    logits with the plain implementation.  Returns the worst error as a fraction of the bound."""
+    from sprout_lm_amd.engine import StepEntry
+    from sprout_lm_amd.sampling import SamplingParams
+    worst = 0.0
+    for _ in range(steps):
+        names = list(seqs)
+        entries = []
+        for r in names:
+            assert runner.cache.reserve(seqs[r], fed[r] + 1)
+            entries.append(StepEntry(seqs[r], [tokens[r][fed[r]]], [0]))
+        pending = runner.launch_decode(entries, [SamplingParams()] * len(names), [0] * len(names))
+        assert pending is not None, "the step did not run from a recorded graph"
+        sampled = runner.finish_decode(pending)
+        got = pending.logits[:len(names)].cpu().numpy()
+        for i, r in enumerate(names):
+            want = plain_rows(folder, tokens[r][:fed[r] + 1], [fed[r]])[0]
+            err = float(np.abs(got[i] - want).max()) / H.tolerance("bfloat16", want)
+            worst = max(worst, err)
+            assert err <= 1.0, f"{label}: request {r} at position {fed[r]}: {err:.2f} of the bound"
+            if want.max() - np.partition(want, -2)[-2] > 2 * H.tolerance("bfloat16", want):
+                assert sampled[i] == int(np.argmax(want)), f"{label}: request {r} at position {fed[r]}: sampled token"
+            fed[r] += 1
+    return worst
+
+
+def test_recorded_steps_of_many_sequences_rotate_by_their_own_positions(tmp_path):
+    """More than 64 sequences in a step take the tiled q/k/v product whose epilogue rotates by a table of sines
+    and cosines that the first layer of a step computes.  A recorded step must compute that table anew at every
+    replay: 530 sequences at different positions, four replays, every logit row against the plain side."""
+    import sprout_lm_amd as S
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    raw = dict(model_type="qwen2", hidden_act="silu", hidden_size=1280, intermediate_size=256, num_hidden_layers=1,
+               num_attention_heads=10, num_key_value_heads=5, vocab_size=300, max_position_embeddings=64,
+               rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=True, eos_token_id=0)
+    n, steps = 530, 4
+    # the case this test is for: at the recorded step's 1,024 rows the projection rotates in its epilogue
+    assert ops.fused_supported(ops.FUSED_ROPE, 1024, (10 + 2 * 5) * 128, 1280, 128, 128, False)
+    folder = str(tmp_path / "wide")
+    write_model_folder(folder, S.config_from_dict(raw), seed=21, dtype=torch.bfloat16, std=0.03)
+    rng = np.random.default_rng(5)
+    tokens = {r: [int(t) for t in rng.integers(0, 300, int(rng.integers(1, 7)) + steps)] for r in range(n)}
+    runner = ModelRunner.from_folder(folder, "bfloat16", block_size=16, num_blocks=n + 8, max_sequences=n)
+    seqs = {r: runner.cache.create() for r in range(n)}
+    fed = {r: len(tokens[r]) - steps for r in range(n)}
+    entries = []
+    for r in range(n):
+        assert runner.cache.reserve(seqs[r], fed[r])
+        entries.append(StepEntry(seqs[r], tokens[r][:fed[r]], []))
+    assert runner.step(entries).shape[0] == 0                    # the prompts, eagerly, no logits wanted
+    worst = decode_through_graphs(runner, seqs, tokens, fed, steps, folder, "wide")
+    assert runner._graphs.replays == steps and list(runner._graphs.graphs) == [(1024, 256)]
+    print(f"recorded steps of {n} sequences: worst {worst:.2f} of the bound")
+
+
+def test_recorded_steps_at_real_layer_sizes_match_plain(tmp_path):
+    """Two layers with the sizes of Qwen2.5-0.5B, decoded through recorded graphs: a batch of three (one padded
+    row), a context that crosses 256 keys under way (another bucket: the chunks of keys are merged inside the
+    output projection from there on), a request that joins late and one that leaves.  With up to 16 tokens the
+    norms are folded into the products and the down product splits K between blocks."""
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    raw = dict(PRESETS["qwen2.5-0.5b"], num_hidden_layers=2)
+    folder = str(tmp_path / "half_b")
+    write_model_folder(folder, S.config_from_dict(raw), seed=9, dtype=torch.bfloat16, std=0.02)
+    lengths = {"a": 250, "c": 5, "d": 100, "b": 300}
+    tokens = {r: H.random_tokens(raw["vocab_size"], m + 24, 30 + i) for i, (r, m) in enumerate(lengths.items())}
+    runner = ModelRunner.from_folder(folder, "bfloat16", block_size=16, num_blocks=64, max_sequences=4)
+    seqs, fed = {}, {}
+
+    def admit(r):
+        seqs[r] = runner.cache.create()
+        assert runner.cache.reserve(seqs[r], lengths[r])
+        runner.step([StepEntry(seqs[r], tokens[r][:lengths[r]], [])])
+        fed[r] = lengths[r]
+
+    for r in "acd":
+        admit(r)
+    worst = decode_through_graphs(runner, seqs, tokens, fed, 10, folder, "three requests")       # a passes 256 keys
+    assert set(runner._graphs.graphs) == {(4, 256), (4, 512)}
+    admit("b")
+    worst = max(worst, decode_through_graphs(runner, seqs, tokens, fed, 4, folder, "four requests"))
+    seqs.pop("c").release()
+    worst = max(worst, decode_through_graphs(runner, seqs, tokens, fed, 4, folder, "three requests again"))
+    for s in seqs.values():
+        s.release()
+    assert runner.cache.free_pages() == [64]
+    print(f"recorded steps at real layer sizes: worst {worst:.2f} of the bound")

@@ -194,7 +194,13 @@ def register_toy():
 
     @register_part("mixer", "toy_running_mean")
     class RunningMean(Mixer):
-        """y_t = W . mean(h_0 .. h_t): the state per request is the running sum and the count."""
+        """y_t = W . mean(h_0 .. h_t): the state per request is the running sum and the count.
+
+        A step in which every request brings one token is computed from device-resident values alone (state
+        slots and rows are indexed on the device), so the part may be recorded into a graph; portions of
+        prompts are cut on the host."""
+
+        graph_safe = True
 
         def __init__(self, hidden):
             self.hidden = hidden
@@ -206,6 +212,17 @@ def register_toy():
             return {"proj.weight": TensorSpec((self.hidden, self.hidden))}
 
         def forward(self, ctx, h, residual, cache):
+            from sprout_lm_amd import ops
+            if ctx.max_q_len == 1:
+                # row i is request i's one token; padded rows of a recorded step point at the spare state slot
+                slots = ctx.state_slots.long()
+                state = cache.state.index_select(0, slots)
+                sums = state[:, :-1] + h.float()
+                counts = state[:, -1] + 1
+                mean = (sums / counts[:, None]).to(h.dtype).contiguous()
+                ops.gemm(mean, self.w["proj.weight"], residual, accumulate=True)
+                cache.state.index_copy_(0, slots, torch.cat([sums, counts[:, None]], dim=1))
+                return
             for start, n, slot in zip(ctx.host["q_start"], ctx.host["q_len"], ctx.host["state_slots"]):
                 state = cache.state[slot]
                 sums = torch.cumsum(h[start:start + n].float(), 0) + state[:-1]
@@ -309,7 +326,7 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
     write_model_folder(folder, S.config_from_dict(TOY), seed=3, dtype=torch.bfloat16, std=0.15)
     assert json.load(open(os.path.join(folder, "config.json")))["architectures"] == ["ToyMeanForCausalLM"]
     runner = ModelRunner.from_folder(folder, dtype, block_size=4, num_blocks=40, max_sequences=3)
-    assert not runner.parts.graph_safe                       # the toy mixer plans on the host: no graph replay
+    assert runner.parts.graph_safe                           # every part says so, the toy mixer included
     kinds = [(g.spec.window, g.slots) for g in runner.cache.groups]
     assert kinds == [(None, [0, 3]), (6, [2])] and runner.cache.state_groups[0].slots == [1]
     from safetensors.torch import load_file
@@ -345,6 +362,60 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
         s.release()
     assert runner.cache.free_pages() == [40, 40]
     print(f"toy {dtype}: worst error {worst:.3e}")
+
+
+def test_toy_architecture_decodes_through_recorded_graphs(tmp_path):
+    """What decides whether steps of single tokens are replayed from recorded graphs is the parts' own word
+    (`graph_safe`), not the kind of cache a model has: the toy model, with per-request state and a windowed
+    group that gives pages back under way, replays, and every replay's logits are the plain side's.  Three
+    requests make a step of four rows: the padded row keeps its state in the spare slot."""
+    register_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cache import FREED
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.sampling import SamplingParams
+    from sprout_lm_amd.weights import write_model_folder
+    folder = str(tmp_path / "toy")
+    write_model_folder(folder, S.config_from_dict(TOY), seed=3, dtype=torch.bfloat16, std=0.15)
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner.from_folder(folder, dtype, block_size=4, num_blocks=40, max_sequences=3)
+        store = P.bf16_round if dtype == "bfloat16" else P.f32
+        requests = {"a": H.random_tokens(97, 30, 11), "b": H.random_tokens(97, 19, 12), "c": H.random_tokens(97, 25, 13)}
+        want = {k: plain_toy_logits(w, t, store) for k, t in requests.items()}
+        tol = 3e-5 if dtype == "float32" else 5e-2
+        seqs = {k: runner.cache.create() for k in requests}
+        fed = {"a": 9, "b": 2, "c": 14}
+        for k, n in fed.items():                                # the prompts' first portions, eagerly
+            assert runner.cache.reserve(seqs[k], n)
+            runner.step([StepEntry(seqs[k], requests[k][:n], [])])
+        spare = runner.cache.spare_state_slot
+        state_before = runner.cache.state_groups[0].data[0, spare].clone()
+        steps = 0
+        while seqs:
+            names = list(seqs)
+            entries = []
+            for k in names:
+                assert runner.cache.reserve(seqs[k], fed[k] + 1)
+                entries.append(StepEntry(seqs[k], [requests[k][fed[k]]], [0]))
+            pending = runner.launch_decode(entries, [SamplingParams()] * len(names), [0] * len(names))
+            assert pending is not None
+            runner.finish_decode(pending)
+            got = pending.logits[:len(names)].cpu().numpy()
+            for row, k in zip(got, names):
+                err = np.abs(row - want[k][fed[k]]).max()
+                assert err <= tol * (1 + np.abs(want[k][fed[k]]).max()), f"{dtype} {k} position {fed[k]}: {err:.3e}"
+                fed[k] += 1
+                if fed[k] == len(requests[k]):
+                    seqs.pop(k).release()
+            steps += 1
+            if steps == 5:
+                assert FREED in seqs["a"].blocks[1]             # the window has given pages back under way
+        assert runner._graphs.replays == steps and steps == 21
+        # the padded row of the first steps ran like any other row; what it added up lies in the spare slot
+        assert not torch.equal(runner.cache.state_groups[0].data[0, spare], state_before)
+        assert runner.cache.free_pages() == [40, 40]
 
 
 # A second toy architecture: a feed-forward with routing and a position encoding of its own, both

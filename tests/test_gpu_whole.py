@@ -102,6 +102,27 @@ def test_reference_fixture_logits_fp32(reference_fixture):
         assert runner.cache.free_pages() == [12]
 
 
+def test_what_cannot_fit_is_refused_before_anything_is_allocated(folders):
+    """Weights and cache pools are counted against the free device memory before the first tensor is read
+    (reference: native/cuda-offload.cu:249-252): an absurd pool, or weights over their limit, are refused with a
+    message that names the numbers, and no device memory has been taken."""
+    import sprout_lm_amd as S
+    from sprout_lm_amd.engine import ModelRunner
+    from sprout_lm_amd.engine.memory import MemoryBudgetError
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    with pytest.raises(MemoryBudgetError, match=r"weights [\d,]+ MiB \+ cache pools [\d,]+ MiB \+ reserve 1,024 MiB = [\d,]+ MiB, free [\d,]+ MiB"):
+        ModelRunner.from_folder(folders["C"], "bfloat16", block_size=16, num_blocks=2_000_000_000, max_sequences=4)
+    with pytest.raises(MemoryBudgetError, match=r"Resident weight budget exceeded.*limit is 1 MiB"):
+        ModelRunner.from_folder(folders["C"], "bfloat16", block_size=16, num_blocks=8, max_sequences=4, weight_limit_mib=1)
+    with pytest.raises(MemoryBudgetError, match="reserve 400,000,000 MiB"):
+        ModelRunner.from_config(S.config_from_dict(H.CONFIGS["A"]), 1, "float32", block_size=16, num_blocks=8,
+                                max_sequences=4, reserve_mib=400_000_000)
+    assert torch.cuda.memory_allocated() == before
+    runner = ModelRunner.from_folder(folders["C"], "bfloat16", block_size=16, num_blocks=8, max_sequences=4, weight_limit_mib=2)
+    assert runner.cache.free_pages() == [8]
+
+
 def test_checkpoint_stored_in_32_bit_computed_in_bfloat16(tmp_path):
     """A tensor stored in 32-bit stays so: bfloat16 activations meet float32 weights (no rounding of the weights)."""
     import torch

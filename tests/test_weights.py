@@ -130,6 +130,43 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in text
 
 
+def test_tensors_nobody_asked_for_are_left_unread_unless_strict(tmp_path):
+    """The reference reads what it asks for and nothing else (src/safetensors.ts:70-83): a checkpoint that still
+    ships a buffer such as rotary_emb.inv_freq loads; a strict load refuses it, naming it."""
+    folder = model_folder(tmp_path)
+    from safetensors.torch import load_file, save_file
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, path)
+    plan = S.build_model_plan(S.load_config(folder))
+    notes = []
+    loaded = load_named_tensors(folder, plan.expected_tensors(), set(plan.ignorable_tensors), torch.bfloat16, "cpu",
+                                notes=notes)
+    assert set(loaded) == set(plan.expected_tensors()) and len(notes) == 1 and "inv_freq" in notes[0]
+    with pytest.raises(WeightError) as info:
+        load_named_tensors(folder, plan.expected_tensors(), set(plan.ignorable_tensors), torch.bfloat16, "cpu", strict=True)
+    assert info.value.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"] and not info.value.missing
+
+
+def test_loaded_tensors_do_not_live_in_the_file(tmp_path):
+    """Tensors go from the file's mapping to where they are kept without a host copy in between; a tensor kept
+    on the host in its stored dtype must still be a copy (the file is closed, and may change, afterwards)."""
+    folder = model_folder(tmp_path)
+    plan = S.build_model_plan(S.load_config(folder))
+    seen = {}
+    loaded = load_named_tensors(folder, plan.expected_tensors(), set(), torch.bfloat16, "cpu",
+                                before_read=lambda stored: seen.update(stored))
+    assert set(seen) == set(plan.expected_tensors()) and set(seen.values()) == {torch.bfloat16}
+    before = {k: v.clone() for k, v in loaded.items()}
+    path = os.path.join(folder, "model.safetensors")
+    size = os.path.getsize(path)
+    with open(path, "r+b") as f:          # scribble over the data region
+        f.seek(size // 2)
+        f.write(b"\xff" * (size - size // 2))
+    assert all(torch.equal(loaded[k].view(torch.int16), before[k].view(torch.int16)) for k in loaded)
+
+
 def test_tied_checkpoint_may_ship_the_output_matrix(tmp_path):
     folder = model_folder(tmp_path)
     from safetensors.torch import load_file, save_file
