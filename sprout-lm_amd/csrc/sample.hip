@@ -4,6 +4,8 @@
 // Temperature: argmax of logits / temperature + Gumbel noise.  The noise of a column comes from a
 // counter generator keyed by (seed, counter, column) only, so a request's draw does not depend on
 // what else is in the batch or on the row it lands in.
+#include <mutex>
+
 #include "common.h"
 #include "sprout_hip.h"
 
@@ -111,6 +113,42 @@ __global__ __launch_bounds__(64) void sample_stage2(const float* __restrict__ pa
   if (threadIdx.x == 0) out[r] = (bad || bi == 0x7fffffff) ? -1 : bi;
 }
 
+// The partial results of sp_sample_static: one copy of this array on every GPU that the library runs on, held
+// until the process ends.  In host code the name `scratch` is only a handle for hipGetSymbolAddress; the
+// address that kernels and copies take is the one that call returns, per device.
+constexpr int kStaticScratchFloats = 64 * 1024;   // 256 KiB
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_of[kMaxDevices];   // device -> address of that device's copy of `scratch` (null: not asked yet)
+static std::mutex g_scratch_lock;
+
+// The current device's copy of `scratch`.  The first call on a device asks the runtime for its address.
+static int static_scratch(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) {
+    set_error("sp_sample_static: no current device: %s", hipGetErrorString(e));
+    return 1;
+  }
+  if (device < 0 || device >= kMaxDevices) {
+    set_error("sp_sample_static: device %d is outside the %d devices the library keeps scratch for", device, kMaxDevices);
+    return 1;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_of[device]) {
+    void* address = nullptr;
+    e = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !address) {
+      set_error("sp_sample_static: cannot find the scratch array on device %d: %s", device, hipGetErrorString(e));
+      return 1;
+    }
+    g_scratch_of[device] = static_cast<float*>(address);
+  }
+  *ptr = g_scratch_of[device];
+  return 0;
+}
+
 }  // namespace sprout
 
 using namespace sprout;
@@ -132,4 +170,29 @@ extern "C" int sp_sample(void* stream, const float* logits, const float* tempera
   sample_stage1<<<dim3(chunks, R), 256, 0, s>>>(logits, temperature, seed, counter, part_value, part_index, V, chunks);
   sample_stage2<<<R, 64, 0, s>>>(part_value, part_index, out, chunks);
   return check_launch("sp_sample");
+}
+
+extern "C" int sp_sample_static_max_floats() { return kStaticScratchFloats; }
+
+// sp_sample with the partial results in the library's own device array: nothing is allocated.
+extern "C" int sp_sample_static(void* stream, const float* logits, const float* temperature, const int64_t* seed,
+                                const int32_t* counter, int32_t* out, int R, int V) {
+  SP_REQUIRE(R >= 0 && V > 0, "sp_sample_static: bad sizes R=%d V=%d", R, V);
+  SP_REQUIRE(logits && out, "sp_sample_static: null argument");
+  if (R == 0) return 0;
+  const int chunks = (V + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+  const long long need = 2LL * R * chunks;
+  SP_REQUIRE(need <= kStaticScratchFloats,
+             "sp_sample_static: %d rows of %d logits need %lld floats of scratch, the static array holds %d "
+             "(use sp_sample with a workspace of the caller's)", R, V, need, kStaticScratchFloats);
+  float* ws = nullptr;
+  if (static_scratch(&ws)) return 1;
+  hipStream_t s = (hipStream_t)stream;
+  // Every slot that the second stage reads is written by the first stage of the same call: nothing has to
+  // start at zero, and what an earlier call left in the array is never read.
+  float* part_value = ws;
+  int* part_index = reinterpret_cast<int*>(ws + size_t(R) * chunks);
+  sample_stage1<<<dim3(chunks, R), 256, 0, s>>>(logits, temperature, seed, counter, part_value, part_index, V, chunks);
+  sample_stage2<<<R, 64, 0, s>>>(part_value, part_index, out, chunks);
+  return check_launch("sp_sample_static");
 }

@@ -107,4 +107,16 @@ int sp_feed_tokens(void* stream, int32_t* tokens, const int32_t* previous, const
 int sp_sample(void* stream, const float* logits, const float* temperature, const int64_t* seed,
               const int32_t* counter, int32_t* out, float* workspace, int R, int V);
 int sp_sample_workspace_floats(int R, int V);
+
+// sp_sample for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+// harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The partial results of the first
+// stage go to a device array of the library's own (sp_sample_static_max_floats() floats, 256 KiB, one copy on
+// every GPU the library is used on, kept until the process ends) instead of a workspace; the call allocates and
+// frees nothing.  Sizes whose partial results (sp_sample_workspace_floats(R, V)) do not fit are refused.  The
+// device of `stream` must be the current device.  All calls on one GPU share that GPU's array: calls whose
+// kernels may overlap (different streams, no ordering between them) race; calls on one stream do not.  What an
+// earlier call left in the array is never read.
+int sp_sample_static(void* stream, const float* logits, const float* temperature, const int64_t* seed,
+                     const int32_t* counter, int32_t* out, int R, int V);
+int sp_sample_static_max_floats();
 }
