@@ -2,8 +2,12 @@
 // folded in.  One block of four waves owns TILES tiles of 16 weight rows; the waves split K between
 // them (64 elements at a time, interleaved), so that even a matrix with few rows keeps many loads in
 // flight, and their partial sums meet in LDS.  What can be folded in:
-//   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from
-//                    the float32 residual and kept in LDS (no separate norm kernel, no round trip)
+//   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from the
+//                    float32 residual (up to 16 tokens).  The scale 1 / sqrt(mean(x^2) + eps) of a token is one
+//                    number, so it is applied to the sums after the product: the lanes turn x * weight into
+//                    matrix-core operands as the rows arrive, add up x^2 on the side, and the squares meet in
+//                    the same exchange through LDS as the partial products.  Nothing waits for the norm: the
+//                    residual rows travel together with the weights.
 //   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
 //             kEpiRope   the block's rows are rotation partners (dims d and d + head/2 of one head): two tiles
 //                        of 16, or (NT = 1, up to 16 tokens) one tile of 8 dimensions and their 8 partners, so
@@ -39,10 +43,86 @@ struct FusedArgs {
   int nq, nkv, hd, page_size, rotary_dim;
 };
 
-__device__ __forceinline__ float load_param(const void* p, int is_bf16, int i) {
-  return is_bf16 ? __uint_as_float(uint32_t(reinterpret_cast<const uint16_t*>(p)[i]) << 16)
-                 : reinterpret_cast<const float*>(p)[i];
+// A bias value as it lies in memory (bfloat16 bits or float32 bits), and its value.  The two are kept apart
+// because turning the bits into a number waits for the load, and loads return in the order of their requests:
+// done where the bias is asked for, it would wait for the weights asked for before it.
+__device__ __forceinline__ uint32_t load_param_bits(const void* p, int is_bf16, int i) {
+  return is_bf16 ? uint32_t(reinterpret_cast<const uint16_t*>(p)[i]) : reinterpret_cast<const uint32_t*>(p)[i];
 }
+__device__ __forceinline__ float param_value(uint32_t bits, int is_bf16) {
+  return __uint_as_float(is_bf16 ? bits << 16 : bits);
+}
+
+__device__ __forceinline__ float4 ldg_f4(const float* __restrict__ p) { return *reinterpret_cast<const float4*>(p); }
+
+// The norm prologue's inputs of one pass as they come from memory: for each of the wave's UN steps the lane's 16
+// values of its token (two groups of 8 along K, starting at k0 + 64 * step) and the norm's weights for them.
+// `request` asks for all of them; `operands` turns them into x * norm weight in bfloat16 and adds the squares of
+// x to `square_sum`.  Groups past the end of K are read from the start of the row instead (a valid address) and
+// count for nothing.  Lanes whose token is past the step's last one (`active` false) request nothing: with a
+// single token that is 15 of 16 lanes.
+template <int UN>
+struct NormInputs {
+  float4 xf[UN][2][2];
+  uint4 nw[UN][2][2];   // the norm's weights as stored: 8 bfloat16 in [0], or 8 float32 in [0] and [1]
+
+  __device__ __forceinline__ void request(const float* __restrict__ row, const void* __restrict__ norm_w, bool BF, int k0,
+                                          int k_end, int s0, int steps, bool active) {
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        xf[u][h][0] = xf[u][h][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+        nw[u][h][0] = nw[u][h][1] = make_uint4(0, 0, 0, 0);
+      }
+    if (!active) return;
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int k = k0 + 64 * (s0 + 4 * u) + 8 * h;
+        const int at = (s0 + 4 * u < steps && k < k_end) ? k : 0;
+        xf[u][h][0] = ldg_f4(row + at);
+        xf[u][h][1] = ldg_f4(row + at + 4);
+        if (BF) {
+          nw[u][h][0] = ldg128(reinterpret_cast<const uint16_t*>(norm_w) + at);
+        } else {
+          nw[u][h][0] = ldg128(reinterpret_cast<const float*>(norm_w) + at);
+          nw[u][h][1] = ldg128(reinterpret_cast<const float*>(norm_w) + at + 4);
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void operands(bool BF, int k0, int k_end, int s0, int steps, uint4 (&xb)[UN][1][2],
+                                           float& square_sum) const {
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int k = k0 + 64 * (s0 + 4 * u) + 8 * h;
+        const float in = (s0 + 4 * u < steps && k < k_end) ? 1.f : 0.f;
+        const float4 x0 = xf[u][h][0], x1 = xf[u][h][1];
+        float4 w0, w1;
+        const uint4 b = nw[u][h][0], c = nw[u][h][1];
+        if (BF) {
+          w0 = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
+                           __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
+          w1 = make_float4(__uint_as_float(b.z << 16), __uint_as_float(b.z & 0xffff0000u),
+                           __uint_as_float(b.w << 16), __uint_as_float(b.w & 0xffff0000u));
+        } else {
+          w0 = make_float4(__uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w));
+          w1 = make_float4(__uint_as_float(c.x), __uint_as_float(c.y), __uint_as_float(c.z), __uint_as_float(c.w));
+        }
+        float sq = fmaf(x0.x, x0.x, fmaf(x0.y, x0.y, fmaf(x0.z, x0.z, x0.w * x0.w)));
+        sq = fmaf(x1.x, x1.x, fmaf(x1.y, x1.y, fmaf(x1.z, x1.z, fmaf(x1.w, x1.w, sq))));
+        square_sum = fmaf(in, sq, square_sum);
+        // (the weights of a group past the end of K are zeros: what stands here for it does not count)
+        xb[u][0][h] = make_uint4(pack_bf16x2(x0.x * w0.x, x0.y * w0.y), pack_bf16x2(x0.z * w0.z, x0.w * w0.w),
+                                 pack_bf16x2(x1.x * w1.x, x1.y * w1.y), pack_bf16x2(x1.z * w1.z, x1.w * w1.w));
+      }
+  }
+};
 
 // First row of tile `which` (0 or 1) of block `b`.
 template <int EPI, int NT>
@@ -61,10 +141,9 @@ template <int TN, int EPI, bool NORM, int NT = 2>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   static_assert(NT == 2 || EPI == kEpiRope, "one gathered tile a block only for the rotation");
   extern __shared__ uint4 lds[];
-  // reduction buffer [4 waves][NT tiles][TN][64 lanes] float4, then (NORM) activations [TN * 16][K / 8 + 1] uint4
+  // reduction buffer [4 waves][NT tiles][TN][64 lanes] float4, then (NORM) sums of squares [4 waves][16 tokens]
   float4* red = reinterpret_cast<float4*>(lds);
-  uint4* xs = lds + 4 * NT * TN * 64;
-  const int LD = a.K / 8 + 1;
+  float* squares = reinterpret_cast<float*>(lds + 4 * NT * TN * 64);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const int k_begin = blockIdx.y * a.k_per_split;
   const int k_end = min(a.K, k_begin + a.k_per_split);
@@ -97,58 +176,23 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       }
     }
   };
-  // RMSNorm of up to 16 tokens: 16 threads per token, each owning every 16th group of four columns,
-  // so that a token's loads are all in flight together and its sum closes with four lane exchanges.
-  const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
-  const float* row = NORM ? a.residual + size_t(min(t, a.T - 1)) * a.K : nullptr;   // rows past T repeat the last one
-  float4 v[16], wn[16];
-  auto load_values = [&](int k0) {
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int k = k0 + 4 * part + 64 * j;
-      v[j] = k < a.K ? *reinterpret_cast<const float4*>(row + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-  };
-  auto load_norm_weights = [&](int k0) {   // one vector load per group of four columns
-    if (a.norm_w_bf16) {
-      const uint16_t* nw = reinterpret_cast<const uint16_t*>(a.norm_w);
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int k = k0 + 4 * part + 64 * j;
-        const uint2 b = k < a.K ? *reinterpret_cast<const uint2*>(nw + k) : make_uint2(0, 0);
-        wn[j] = make_float4(__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xffff0000u),
-                            __uint_as_float(b.y << 16), __uint_as_float(b.y & 0xffff0000u));
-      }
-    } else {
-      const float* nw = reinterpret_cast<const float*>(a.norm_w);
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int k = k0 + 4 * part + 64 * j;
-        wn[j] = k < a.K ? *reinterpret_cast<const float4*>(nw + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    }
-  };
-  // Loads return in the order of their requests.  The residual rows (close by, in L2) are therefore asked for
-  // before the weights (far, in memory): they arrive early, and the norm is computed while the weights are
-  // still on their way.  (With the weights first, the norm waited for them and stood between them and the
-  // products: it then cost as much as a kernel of its own.)
-  if (NORM) {
-    load_values(0);
-    load_norm_weights(0);
-  }
+  // The norm prologue's rows are requested right after the weights; both are then on their way together.
+  NormInputs<NORM ? UN : 1> normed;
+  const float* norm_row = NORM ? a.residual + size_t(min(lr, a.T - 1)) * a.K : nullptr;
   load_weights(wave);
+  if constexpr (NORM) normed.request(norm_row, a.norm_w, a.norm_w_bf16, k_begin + 16 * lj, k_end, wave, steps, lr < a.T);
   __builtin_amdgcn_sched_barrier(0);   // keep these requests ahead of everything below
   // What the epilogue reads per output (bias, position, rotation frequency, cache slot) is requested now
   // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
   // thread -> (token et of a tile, row ei of the tile), as in the epilogue below
   const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
   const int er = NT == 1 ? (ei & 7) : ei;   // one gathered tile: threads ei < 8 own dimension er and its partner
-  float bias_of[2] = {0.f, 0.f};
+  uint32_t bias_bits[2] = {0u, 0u};   // zero bits are zero in either dtype
   if (a.bias && blockIdx.y == 0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int n = NT == 1 ? row0[0] + er + i * a.partner : row0[i] + ei;
-      if (n < a.N) bias_of[i] = load_param(a.bias, a.bias_bf16, n);
+      if (n < a.N) bias_bits[i] = load_param_bits(a.bias, a.bias_bf16, n);
     }
   }
   int position_of[TN], slot_of[TN];
@@ -164,34 +208,6 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     }
   }
 
-  if (NORM) {
-    float sum = 0.f;
-    for (int k0 = 0; k0 < a.K; k0 += 1024) {
-      if (k0 > 0) load_values(k0);                         // the first 1024 columns were requested above
-#pragma unroll
-      for (int j = 0; j < 16; ++j) sum = fmaf(v[j].x, v[j].x, fmaf(v[j].y, v[j].y, fmaf(v[j].z, v[j].z, fmaf(v[j].w, v[j].w, sum))));
-    }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-    const float scale = rsqrtf(sum / float(a.K) + a.eps);
-    for (int k0 = 0; k0 < a.K; k0 += 1024) {
-      if (a.K > 1024) {                                    // wide rows: the values are read again
-        load_values(k0);
-        load_norm_weights(k0);
-      }
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int k = k0 + 4 * part + 64 * j;
-        if (k < a.K) {
-          uint2* dst = reinterpret_cast<uint2*>(xs + t * LD) + (k >> 2);
-          *dst = make_uint2(pack_bf16x2(v[j].x * scale * wn[j].x, v[j].y * scale * wn[j].y),
-                            pack_bf16x2(v[j].z * scale * wn[j].z, v[j].w * scale * wn[j].w));
-        }
-      }
-    }
-    __syncthreads();
-  }
-
   floatx4 acc[NT][TN];
 #pragma unroll
   for (int i = 0; i < NT; ++i)
@@ -199,20 +215,27 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // this wave's steps of 64 along K: wave, wave + 4, ...; UN steps are loaded before they are multiplied
+  static_assert(!NORM || TN == 1, "the norm prologue takes one tile of 16 tokens");
+  float square_sum = 0.f;   // NORM: this lane's share of the sum of squares of token lr
   for (int s0 = wave; s0 < steps; s0 += 4 * UN) {
-    if (s0 != wave) load_weights(s0);
+    if (s0 != wave) {
+      load_weights(s0);
+      if constexpr (NORM) normed.request(norm_row, a.norm_w, a.norm_w_bf16, k_begin + 16 * lj, k_end, s0, steps, lr < a.T);
+    }
     uint4 xb[UN][TN][2];
+    if constexpr (NORM) {
+      // Lane (lr, lj) needs 16 values of token lr per step, as the matrix cores take them.  They come straight
+      // from the float32 residual, times the norm's weights (the same for every token), rounded to bfloat16;
+      // the token's scale follows in the epilogue.  Lanes of rows past T load nothing and hold zeros.
+      normed.operands(a.norm_w_bf16, k_begin + 16 * lj, k_end, s0, steps, xb, square_sum);
+    } else {
 #pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
-      const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
+      for (int u = 0; u < UN; ++u) {
+        const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
+        const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn) {
-        const int t = tn * 16 + lr;
-        if (NORM) {
-          xb[u][tn][0] = in0 ? xs[t * LD + (k >> 3)] : make_uint4(0, 0, 0, 0);
-          xb[u][tn][1] = in1 ? xs[t * LD + (k >> 3) + 1] : make_uint4(0, 0, 0, 0);
-        } else {
+        for (int tn = 0; tn < TN; ++tn) {
+          const int t = tn * 16 + lr;
           const bool row = t < a.T;
           xb[u][tn][0] = (row && in0) ? ldg128(a.x + size_t(t) * a.K + k) : make_uint4(0, 0, 0, 0);
           xb[u][tn][1] = (row && in1) ? ldg128(a.x + size_t(t) * a.K + k + 8) : make_uint4(0, 0, 0, 0);
@@ -235,10 +258,18 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
       red[((wave * NT + i) * TN + tn) * 64 + lane] = make_float4(acc[i][tn][0], acc[i][tn][1], acc[i][tn][2], acc[i][tn][3]);
+  if (NORM) {   // the four lanes of a token hold a quarter of the wave's steps each
+    square_sum += __shfl_xor(square_sum, 16, 64);
+    square_sum += __shfl_xor(square_sum, 32, 64);
+    if (lj == 0) squares[wave * 16 + lr] = square_sum;
+  }
   __syncthreads();
 
   // thread -> (token t of the tile, row i of the tile); the MFMA lane that holds it is (i / 4) * 16 + t, element i % 4
   const int src_lane = (ei >> 2) * 16 + et, src_r = ei & 3;
+  // NORM: 1 / sqrt(mean(x^2) + eps) of this thread's token, from the four waves' shares of the sum
+  const float scale_of = NORM ? rsqrtf((squares[et] + squares[16 + et] + squares[32 + et] + squares[48 + et]) / float(a.K) + a.eps)
+                              : 1.f;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     const int t = tn * 16 + et;
@@ -254,7 +285,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
         for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * NT + i) * TN + tn) * 64 + src_lane])[src_r];
       }
-      v[i] = sum + bias_of[i];
+      v[i] = (NORM ? sum * scale_of : sum) + param_value(bias_bits[i], a.bias_bf16);
     }
     if (t >= a.T || (NT == 1 && ei >= 8)) continue;
     if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
@@ -311,13 +342,13 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   }
 }
 
-static size_t fused_lds_bytes(int TN, bool norm, int K, int NT = 2) {
-  return sizeof(float4) * 4 * NT * TN * 64 + (norm ? sizeof(uint4) * size_t(TN) * 16 * (K / 8 + 1) : 0);
+static size_t fused_lds_bytes(int TN, bool norm, int NT = 2) {
+  return sizeof(float4) * 4 * NT * TN * 64 + (norm ? sizeof(float) * 4 * 16 : 0);
 }
 
 template <int TN, int EPI, bool NORM, int NT = 2>
 static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
-  const size_t lds = fused_lds_bytes(TN, NORM, a.K, NT);
+  const size_t lds = fused_lds_bytes(TN, NORM, NT);
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fused_kernel<TN, EPI, NORM, NT>),
@@ -340,16 +371,23 @@ static bool rope_one_tile(int T, int hd) { return T <= 16 || hd % 32 != 0; }
 
 template <int EPI, bool NORM>
 static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
-  if (EPI == kEpiRope && rope_one_tile(a.T, a.hd)) {
+  if constexpr (NORM) {   // one tile of up to 16 tokens (fused_shape_ok)
     if constexpr (EPI == kEpiRope) {
-      if (a.T <= 16) return launch_fused<1, EPI, NORM, 1>(s, a, blocks, splits);
-      if (a.T <= 32) return launch_fused<2, EPI, NORM, 1>(s, a, blocks, splits);
-      return launch_fused<4, EPI, NORM, 1>(s, a, blocks, splits);
+      if (rope_one_tile(a.T, a.hd)) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);
     }
+    return launch_fused<1, EPI, true>(s, a, blocks, splits);
+  } else {
+    if (EPI == kEpiRope && rope_one_tile(a.T, a.hd)) {
+      if constexpr (EPI == kEpiRope) {
+        if (a.T <= 16) return launch_fused<1, EPI, false, 1>(s, a, blocks, splits);
+        if (a.T <= 32) return launch_fused<2, EPI, false, 1>(s, a, blocks, splits);
+        return launch_fused<4, EPI, false, 1>(s, a, blocks, splits);
+      }
+    }
+    if (a.T <= 16) return launch_fused<1, EPI, false>(s, a, blocks, splits);
+    if (a.T <= 32) return launch_fused<2, EPI, false>(s, a, blocks, splits);
+    return launch_fused<4, EPI, false>(s, a, blocks, splits);
   }
-  if (a.T <= 16) return launch_fused<1, EPI, NORM>(s, a, blocks, splits);
-  if (a.T <= 32) return launch_fused<2, EPI, NORM>(s, a, blocks, splits);
-  return launch_fused<4, EPI, NORM>(s, a, blocks, splits);
 }
 
 template <int EPI>
@@ -358,12 +396,10 @@ static int fused_norm(hipStream_t s, const FusedArgs& a, bool norm, int blocks, 
 }
 
 // Whether the fused kernels take this shape.  K in 16-byte rows, T <= 64; the norm prologue takes up to
-// 16 tokens, whose normalised activations must fit into LDS beside the reduction buffer.
+// 16 tokens (one tile).
 static bool fused_shape_ok(int T, int K, bool norm) {
   if (T < 1 || T > 64 || K % 8) return false;
-  if (norm && T > 16) return false;   // the prologue normalises one tile of 16 tokens
-  const int TN = T <= 16 ? 1 : T <= 32 ? 2 : 4;
-  return fused_lds_bytes(TN, norm, K) <= 150 * 1024;
+  return !(norm && T > 16);
 }
 
 }  // namespace sprout
