@@ -29,13 +29,14 @@ constexpr int kDecodeWaveKeys = 64; // keys per wave of a decode block
 struct PagedKV {
   const uint16_t* k;     // key pool, already offset to the key/value head: + page * page_stride + slot * HD + d
   const uint16_t* v;     // value pool, offset to the head: + page * page_stride + d * page_size + slot
-  const int32_t* table;  // this sequence's block table
+  const int32_t* table;  // this sequence's block table, from entry `table_first` on
   int page_size, num_pages;
   size_t page_stride;    // elements between pages: nkv * page_size * HD
+  int table_first = 0;   // the table entry that table[0] is (a copy of a part of the table starts later)
 };
 
 __device__ __forceinline__ int page_of(const PagedKV& kv, int key) {
-  const int page = kv.table[key / kv.page_size];
+  const int page = kv.table[key / kv.page_size - kv.table_first];
   return min(max(page, 0), kv.num_pages - 1);   // a bad table entry must not become a wild address
 }
 
@@ -534,11 +535,19 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   __shared__ float s_o[4][16][HD + 1];
   __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ int32_t s_table[kDecodeChunk / 4 + 4];      // the chunk's page numbers (pages of 4 tokens or more)
   const int split = blockIdx.x, g = blockIdx.y, di = blockIdx.z;
   const int seq = decode_seqs ? decode_seqs[di] : di;   // no list: the batch is one-query sequences only, in order
+  const int chunk0 = split * kDecodeChunk;
+  // The page numbers of this chunk do not depend on how long the sequence is: they are asked for together with
+  // its length (entries past the sequence's pages are never used), so that the keys are one trip further, not two.
+  const int table_first = chunk0 / page_size, table_count = (chunk0 + kDecodeChunk - 1) / page_size - table_first + 1;
+  if (int(threadIdx.x) < table_count)
+    s_table[threadIdx.x] = block_tables[size_t(seq) * max_blocks + min(table_first + int(threadIdx.x), max_blocks - 1)];
+  // without a list, sequence i's one query is row i
+  const int q_row = decode_seqs ? q_start[seq] : seq;
   const int ctx = ctx_len[seq], pos = ctx - 1;
   const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int chunk0 = split * kDecodeChunk;
   const int G = nq / nkv;
   if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) {
     // no visible key in this chunk: the merge kernel reads every chunk's (maximum, sum) without looking at
@@ -558,11 +567,13 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   kv.page_stride = size_t(nkv) * page_size * HD;
   kv.k = k_pool + size_t(g) * page_size * HD;
   kv.v = v_pool + size_t(g) * page_size * HD;
-  kv.table = block_tables + size_t(seq) * max_blocks;
+  kv.table = s_table;
+  kv.table_first = table_first;
 
   bf16x8 qop[1][HC];
   int qpos[1] = {lr < G ? pos : -1};
-  load_q_operand<DT>(qop[0], lr < G ? q + size_t(q_start[seq]) * q_stride + (g * G + lr) * HD : nullptr);
+  load_q_operand<DT>(qop[0], lr < G ? q + size_t(q_row) * q_stride + (g * G + lr) * HD : nullptr);
+  __syncthreads();   // the page numbers are in LDS
   floatx4 o[1][DT];
   float m[1] = {kNoKeyYet}, lsum[1] = {0.f};
 #pragma unroll
@@ -605,7 +616,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     }
     const int head = g * G + qh;
     if (n_splits == 1) {
-      out[size_t(q_start[seq]) * (size_t(nq) * HD) + head * HD + d] = f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
+      out[size_t(q_row) * (size_t(nq) * HD) + head * HD + d] = f32_to_bf16_bits(den > 0.f ? num / den : 0.f);
     } else {
       const size_t slot = (size_t(di) * nq + head) * n_splits + split;
       part_o[slot * HD + d] = num;
@@ -702,7 +713,8 @@ __global__ __launch_bounds__(256) void attention_merge_project_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ decode_seqs, const uint16_t* __restrict__ w_o, float* __restrict__ residual,
     int n_decode, int n_splits, int nq, int hidden) {
-  constexpr int HD = 16 * DT, HC = (DT + 1) / 2, XP = HD + 8, GROUP = 8;
+  // GROUP chunks are requested together: the 16 chunks of a context of 4,096 keys in one trip to memory
+  constexpr int HD = 16 * DT, HC = (DT + 1) / 2, XP = HD + 8, GROUP = 16;
   __shared__ __attribute__((aligned(16))) uint16_t xs[16 * TN][XP];
   __shared__ int32_t s_row[16 * TN];
   const int head = blockIdx.x, n_begin = blockIdx.y * (64 * TPW);

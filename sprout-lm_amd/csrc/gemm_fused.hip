@@ -1,5 +1,5 @@
 // Skinny bfloat16 products for decoding (T <= 64) with the work of the neighbouring small kernels
-// folded in.  One block of four waves owns TILES tiles of 16 weight rows; the waves split K between
+// folded in.  One block of four waves owns NT tiles of 16 weight rows; the waves split K between
 // them (64 elements at a time, interleaved), so that even a matrix with few rows keeps many loads in
 // flight, and their partial sums meet in LDS.  What can be folded in:
 //   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from the
@@ -13,8 +13,14 @@
 //                        of 16, or (NT = 1, up to 16 tokens) one tile of 8 dimensions and their 8 partners, so
 //                        that the few rows of q, k and v are spread over twice the blocks; adds the bias,
 //                        rotates q and k heads, writes q and scatters k, v into the paged cache
-//             kEpiSilu   the two tiles are gate rows and the matching up rows: writes silu(gate) * up
+//             kEpiSilu   the block owns `rows_per_block` inner columns: their gate rows and the matching up rows
+//                        fill its tiles one after the other (two tiles hold 16 of each; three hold up to 24, which
+//                        lets a matrix be cut into a whole number of blocks per CU); writes silu(gate) * up
 // Accumulating products may also be split along K over several blocks (hardware float atomics).
+//
+// A step of decoded tokens spends a few microseconds in each of these kernels, and a wave's every vector
+// instruction is four cycles of them: with K in whole steps of 64 (K64) the loads carry no bounds of their
+// own, whole steps are switched by scalar branches, and addresses are one base per pass plus constants.
 #include "mfma.h"
 #include "sprout_hip.h"
 
@@ -33,7 +39,8 @@ struct FusedArgs {
   int bias_bf16;
   void* out;                 // [T, N] (store / accumulate); [T, N / 2] for kEpiSilu; q rows [T, nq * hd] for kEpiRope
   int T, N, K, k_per_split;
-  int partner;               // rows between a tile and its partner tile (kEpiRope: hd / 2, kEpiSilu: N / 2)
+  int partner;               // rows between a row and its partner (kEpiRope: hd / 2, kEpiSilu: N / 2)
+  int rows_per_block;        // kEpiSilu: inner columns a block owns (at most 8 * NT)
   // kEpiRope
   const int32_t* positions;
   const float* inv_freq;
@@ -56,52 +63,55 @@ __device__ __forceinline__ float param_value(uint32_t bits, int is_bf16) {
 __device__ __forceinline__ float4 ldg_f4(const float* __restrict__ p) { return *reinterpret_cast<const float4*>(p); }
 
 // The norm prologue's inputs of one pass as they come from memory: for each of the wave's UN steps the lane's 16
-// values of its token (two groups of 8 along K, starting at k0 + 64 * step) and the norm's weights for them.
-// `request` asks for all of them; `operands` turns them into x * norm weight in bfloat16 and adds the squares of
-// x to `square_sum`.  Groups past the end of K are read from the start of the row instead (a valid address) and
-// count for nothing.  Lanes whose token is past the step's last one (`active` false) request nothing: with a
-// single token that is 15 of 16 lanes.
-template <int UN>
+// values of its token (two groups of 8 along K) and the norm's weights for them.  `request` asks for all of
+// them; `operands` turns them into x * norm weight in bfloat16 and adds the squares of x to `square_sum`.
+// `row` and `norm_w` point at the lane's first value of the pass (step s0); step s0 + 4 u lies 256 u values on.
+// K64: K is whole steps, a step is there or not for the whole wave (`steps_left` of them from s0 on, every
+// fourth).  Otherwise groups past the end of K are read from `safe_row` / `safe_w` instead (valid addresses:
+// the starts of the row and of the norm's weights) and count for nothing.
+template <int UN, bool K64>
 struct NormInputs {
   float4 xf[UN][2][2];
   uint4 nw[UN][2][2];   // the norm's weights as stored: 8 bfloat16 in [0], or 8 float32 in [0] and [1]
 
-  __device__ __forceinline__ void request(const float* __restrict__ row, const void* __restrict__ norm_w, bool BF, int k0,
-                                          int k_end, int s0, int steps, bool active) {
-#pragma unroll
-    for (int u = 0; u < UN; ++u)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        xf[u][h][0] = xf[u][h][1] = make_float4(0.f, 0.f, 0.f, 0.f);
-        nw[u][h][0] = nw[u][h][1] = make_uint4(0, 0, 0, 0);
-      }
-    if (!active) return;
+  __device__ __forceinline__ void request(const float* __restrict__ row, const void* __restrict__ norm_w, bool BF,
+                                          int steps_left, int k_left, const float* __restrict__ safe_row,
+                                          const void* __restrict__ safe_w) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
+      if (K64 && 4 * u >= steps_left) {   // the same for every lane of the wave: a scalar branch
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          xf[u][h][0] = xf[u][h][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+          nw[u][h][0] = nw[u][h][1] = make_uint4(0, 0, 0, 0);
+        }
+        continue;
+      }
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int k = k0 + 64 * (s0 + 4 * u) + 8 * h;
-        const int at = (s0 + 4 * u < steps && k < k_end) ? k : 0;
-        xf[u][h][0] = ldg_f4(row + at);
-        xf[u][h][1] = ldg_f4(row + at + 4);
+        const int at = 256 * u + 8 * h;
+        const bool there = K64 || (4 * u < steps_left && at < k_left);
+        const float* xp = there ? row + at : safe_row;
+        xf[u][h][0] = ldg_f4(xp);
+        xf[u][h][1] = ldg_f4(xp + 4);
+        nw[u][h][1] = make_uint4(0, 0, 0, 0);
         if (BF) {
-          nw[u][h][0] = ldg128(reinterpret_cast<const uint16_t*>(norm_w) + at);
+          nw[u][h][0] = ldg128(there ? reinterpret_cast<const uint16_t*>(norm_w) + at : reinterpret_cast<const uint16_t*>(safe_w));
         } else {
-          nw[u][h][0] = ldg128(reinterpret_cast<const float*>(norm_w) + at);
-          nw[u][h][1] = ldg128(reinterpret_cast<const float*>(norm_w) + at + 4);
+          const float* wp = there ? reinterpret_cast<const float*>(norm_w) + at : reinterpret_cast<const float*>(safe_w);
+          nw[u][h][0] = ldg128(wp);
+          nw[u][h][1] = ldg128(wp + 4);
         }
       }
     }
   }
 
-  __device__ __forceinline__ void operands(bool BF, int k0, int k_end, int s0, int steps, uint4 (&xb)[UN][1][2],
+  __device__ __forceinline__ void operands(bool BF, int steps_left, int k_left, uint4 (&xb)[UN][1][2],
                                            float& square_sum) const {
 #pragma unroll
     for (int u = 0; u < UN; ++u)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int k = k0 + 64 * (s0 + 4 * u) + 8 * h;
-        const float in = (s0 + 4 * u < steps && k < k_end) ? 1.f : 0.f;
         const float4 x0 = xf[u][h][0], x1 = xf[u][h][1];
         float4 w0, w1;
         const uint4 b = nw[u][h][0], c = nw[u][h][1];
@@ -116,7 +126,8 @@ struct NormInputs {
         }
         float sq = fmaf(x0.x, x0.x, fmaf(x0.y, x0.y, fmaf(x0.z, x0.z, x0.w * x0.w)));
         sq = fmaf(x1.x, x1.x, fmaf(x1.y, x1.y, fmaf(x1.z, x1.z, fmaf(x1.w, x1.w, sq))));
-        square_sum = fmaf(in, sq, square_sum);
+        if (K64) square_sum += sq;                     // a step that is not there holds zeros
+        else square_sum = fmaf((4 * u < steps_left && 256 * u + 8 * h < k_left) ? 1.f : 0.f, sq, square_sum);
         // (the weights of a group past the end of K are zeros: what stands here for it does not count)
         xb[u][0][h] = make_uint4(pack_bf16x2(x0.x * w0.x, x0.y * w0.y), pack_bf16x2(x0.z * w0.z, x0.w * w0.w),
                                  pack_bf16x2(x1.x * w1.x, x1.y * w1.y), pack_bf16x2(x1.z * w1.z, x1.w * w1.w));
@@ -124,82 +135,116 @@ struct NormInputs {
   }
 };
 
-// First row of tile `which` (0 or 1) of block `b`.
+// The weight row that lane-row `lr` of tile `i` of block `b` multiplies (an existing row also where the tile
+// has no row for the lane: what it computes there is not used).
 template <int EPI, int NT>
-__device__ __forceinline__ int tile_row0(const FusedArgs& a, int b, int which) {
+__device__ __forceinline__ int weight_row(const FusedArgs& a, int b, int i, int lr) {
+  int row;
   if (EPI == kEpiRope) {
     const int dims = NT == 1 ? 8 : 16;                    // dimensions of a head's first half that a block takes
     const int per_head = a.hd / (2 * dims);
-    const int head = b / per_head, j = b % per_head;
-    return head * a.hd + dims * j + which * a.partner;
+    const int first = (b / per_head) * a.hd + dims * (b % per_head);
+    // one gathered tile: rows 0..7 are dims first .. + 7 of the head, rows 8..15 their partners half a head on
+    row = NT == 1 ? first + (lr < 8 ? lr : a.partner + lr - 8) : first + i * a.partner + lr;
+  } else if (EPI == kEpiSilu) {
+    // the block's gate rows, then its up rows, fill the tiles one after the other
+    const int slot = 16 * i + lr, r = a.rows_per_block;
+    row = slot < r ? b * r + slot : a.partner + b * r + slot - r;
+  } else {
+    row = 16 * (NT * b + i) + lr;
   }
-  if (EPI == kEpiSilu) return 16 * b + which * a.partner;
-  return 16 * (2 * b + which);
+  return min(a.N - 1, row);
 }
 
-template <int TN, int EPI, bool NORM, int NT = 2>
+template <int TN, int EPI, bool NORM, int NT, bool K64>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
-  static_assert(NT == 2 || EPI == kEpiRope, "one gathered tile a block only for the rotation");
+  static_assert(NT == 2 || EPI == kEpiRope || EPI == kEpiSilu, "one or three tiles a block only where rows are paired");
+  static_assert(!NORM || TN == 1, "the norm prologue takes one tile of 16 tokens");
   extern __shared__ uint4 lds[];
   // reduction buffer [4 waves][NT tiles][TN][64 lanes] float4, then (NORM) sums of squares [4 waves][16 tokens]
   float4* red = reinterpret_cast<float4*>(lds);
   float* squares = reinterpret_cast<float*>(lds + 4 * NT * TN * 64);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for the whole wave: a scalar
+  const int lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const int k_begin = blockIdx.y * a.k_per_split;
   const int k_end = min(a.K, k_begin + a.k_per_split);
+  const int steps = (k_end - k_begin + 63) / 64;
 
-  int row0[2];
-  row0[0] = tile_row0<EPI, NT>(a, blockIdx.x, 0);
-  row0[1] = tile_row0<EPI, NT>(a, blockIdx.x, 1);
+  // the lane's first weight of each tile, and of the activations, at step 0
   const uint16_t* wrow[NT];
-  if (NT == 1) {   // rows 0..7 of the tile: dims row0[0] .. + 7 of the head; rows 8..15: their partners, half a head on
-    wrow[0] = a.w + size_t(min(a.N - 1, row0[0] + (lr < 8 ? lr : a.partner + lr - 8))) * a.K;
-  } else {
 #pragma unroll
-    for (int i = 0; i < NT; ++i) wrow[i] = a.w + size_t(min(a.N - 1, row0[i] + lr)) * a.K;
-  }
+  for (int i = 0; i < NT; ++i) wrow[i] = a.w + size_t(weight_row<EPI, NT>(a, blockIdx.x, i, lr)) * a.K + k_begin + 16 * lj;
+  const float* norm_row = NORM ? a.residual + size_t(min(lr, a.T - 1)) * a.K + k_begin + 16 * lj : nullptr;
+  const char* norm_w0 = NORM ? reinterpret_cast<const char*>(a.norm_w) + size_t(k_begin + 16 * lj) * (a.norm_w_bf16 ? 2 : 4) : nullptr;
+  const uint16_t* xrow[TN];
+#pragma unroll
+  for (int tn = 0; tn < TN; ++tn)   // rows past T repeat the last one: their sums are not used
+    xrow[tn] = NORM ? nullptr : a.x + size_t(min(tn * 16 + lr, a.T - 1)) * a.K + k_begin + 16 * lj;
 
   // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
-  // of this wave together.
+  // of this wave together (steps s0, s0 + 4, ...).
   constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
-  const int steps = (k_end - k_begin + 63) / 64;
   uint4 wa[UN][NT][2];
   auto load_weights = [&](int s0) {
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
-      const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
-      const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
+      const bool step_there = s0 + 4 * u < steps;
+      if (K64) {
+        if (step_there) {   // a scalar branch
 #pragma unroll
-      for (int i = 0; i < NT; ++i) {
-        wa[u][i][0] = in0 ? ldg128(wrow[i] + k) : make_uint4(0, 0, 0, 0);
-        wa[u][i][1] = in1 ? ldg128(wrow[i] + k + 8) : make_uint4(0, 0, 0, 0);
+          for (int i = 0; i < NT; ++i) {
+            wa[u][i][0] = ldg128(wrow[i] + 64 * s0 + 256 * u);
+            wa[u][i][1] = ldg128(wrow[i] + 64 * s0 + 256 * u + 8);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < NT; ++i) wa[u][i][0] = wa[u][i][1] = make_uint4(0, 0, 0, 0);
+        }
+      } else {
+        const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
+        const bool in0 = step_there && k < k_end, in1 = step_there && k + 8 < k_end;
+#pragma unroll
+        for (int i = 0; i < NT; ++i) {
+          wa[u][i][0] = in0 ? ldg128(wrow[i] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
+          wa[u][i][1] = in1 ? ldg128(wrow[i] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
+        }
       }
     }
   };
   // The norm prologue's rows are requested right after the weights; both are then on their way together.
-  NormInputs<NORM ? UN : 1> normed;
-  const float* norm_row = NORM ? a.residual + size_t(min(lr, a.T - 1)) * a.K : nullptr;
+  NormInputs<NORM ? UN : 1, K64> normed;
+  auto request_rows = [&](int s0) {
+    normed.request(norm_row + 64 * s0, norm_w0 + size_t(64 * s0) * (a.norm_w_bf16 ? 2 : 4), a.norm_w_bf16, steps - s0,
+                   k_end - (k_begin + 16 * lj + 64 * s0), a.residual, a.norm_w);
+  };
   load_weights(wave);
-  if constexpr (NORM) normed.request(norm_row, a.norm_w, a.norm_w_bf16, k_begin + 16 * lj, k_end, wave, steps, lr < a.T);
+  if constexpr (NORM) request_rows(wave);
   __builtin_amdgcn_sched_barrier(0);   // keep these requests ahead of everything below
   // What the epilogue reads per output (bias, position, rotation frequency, cache slot) is requested now
   // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
-  // thread -> (token et of a tile, row ei of the tile), as in the epilogue below
+  // thread -> (token et of a tile, row ei of a tile), as in the epilogue below
   const int et = threadIdx.x >> 4, ei = threadIdx.x & 15;
-  const int er = NT == 1 ? (ei & 7) : ei;   // one gathered tile: threads ei < 8 own dimension er and its partner
+  const int er = (EPI == kEpiRope && NT == 1) ? (ei & 7) : ei;   // one gathered tile: threads ei < 8 own a dimension and its partner
+  // the output rows this thread finishes: kEpiRope dimension er of the block and its partner; kEpiSilu the
+  // block's inner columns ei and 16 + ei; otherwise row ei of either tile
+  constexpr int OUTS = EPI == kEpiSilu ? (NT + 1) / 2 : 2;
   uint32_t bias_bits[2] = {0u, 0u};   // zero bits are zero in either dtype
-  if (a.bias && blockIdx.y == 0) {
+  if (EPI != kEpiSilu && a.bias && blockIdx.y == 0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int n = NT == 1 ? row0[0] + er + i * a.partner : row0[i] + ei;
+      const int n = EPI == kEpiRope ? weight_row<EPI, NT>(a, blockIdx.x, NT == 1 ? 0 : i, NT == 1 ? er + 8 * i : er)
+                                    : 16 * (NT * blockIdx.x + i) + ei;
       if (n < a.N) bias_bits[i] = load_param_bits(a.bias, a.bias_bf16, n);
     }
   }
   int position_of[TN], slot_of[TN];
   float frequency = 0.f;
+  int rope_head = 0, rope_dim = 0;
   if (EPI == kEpiRope) {
-    const int d = row0[0] % a.hd + er;
-    if (d < a.rotary_dim / 2) frequency = a.inv_freq[d];
+    const int dims = NT == 1 ? 8 : 16, per_head = a.hd / (2 * dims);
+    rope_head = blockIdx.x / per_head;
+    rope_dim = dims * (blockIdx.x % per_head) + er;           // < hd / 2; the partner is hd / 2 further
+    if (rope_dim < a.rotary_dim / 2) frequency = a.inv_freq[rope_dim];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
       const int t = min(tn * 16 + et, a.T - 1);
@@ -215,30 +260,37 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // this wave's steps of 64 along K: wave, wave + 4, ...; UN steps are loaded before they are multiplied
-  static_assert(!NORM || TN == 1, "the norm prologue takes one tile of 16 tokens");
   float square_sum = 0.f;   // NORM: this lane's share of the sum of squares of token lr
   for (int s0 = wave; s0 < steps; s0 += 4 * UN) {
     if (s0 != wave) {
       load_weights(s0);
-      if constexpr (NORM) normed.request(norm_row, a.norm_w, a.norm_w_bf16, k_begin + 16 * lj, k_end, s0, steps, lr < a.T);
+      if constexpr (NORM) request_rows(s0);
     }
     uint4 xb[UN][TN][2];
     if constexpr (NORM) {
       // Lane (lr, lj) needs 16 values of token lr per step, as the matrix cores take them.  They come straight
       // from the float32 residual, times the norm's weights (the same for every token), rounded to bfloat16;
-      // the token's scale follows in the epilogue.  Lanes of rows past T load nothing and hold zeros.
-      normed.operands(a.norm_w_bf16, k_begin + 16 * lj, k_end, s0, steps, xb, square_sum);
+      // the token's scale follows in the epilogue.
+      normed.operands(a.norm_w_bf16, steps - s0, k_end - (k_begin + 16 * lj + 64 * s0), xb, square_sum);
     } else {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
+        const bool step_there = s0 + 4 * u < steps;
         const int k = k_begin + 64 * (s0 + 4 * u) + 16 * lj;
-        const bool in0 = s0 + 4 * u < steps && k < k_end, in1 = s0 + 4 * u < steps && k + 8 < k_end;
+        const bool in0 = step_there && (K64 || k < k_end), in1 = step_there && (K64 || k + 8 < k_end);
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) {
-          const int t = tn * 16 + lr;
-          const bool row = t < a.T;
-          xb[u][tn][0] = (row && in0) ? ldg128(a.x + size_t(t) * a.K + k) : make_uint4(0, 0, 0, 0);
-          xb[u][tn][1] = (row && in1) ? ldg128(a.x + size_t(t) * a.K + k + 8) : make_uint4(0, 0, 0, 0);
+          if (K64) {
+            if (step_there) {
+              xb[u][tn][0] = ldg128(xrow[tn] + 64 * s0 + 256 * u);
+              xb[u][tn][1] = ldg128(xrow[tn] + 64 * s0 + 256 * u + 8);
+            } else {
+              xb[u][tn][0] = xb[u][tn][1] = make_uint4(0, 0, 0, 0);
+            }
+          } else {
+            xb[u][tn][0] = in0 ? ldg128(xrow[tn] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
+            xb[u][tn][1] = in1 ? ldg128(xrow[tn] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
+          }
         }
       }
     }
@@ -265,33 +317,46 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   }
   __syncthreads();
 
-  // thread -> (token t of the tile, row i of the tile); the MFMA lane that holds it is (i / 4) * 16 + t, element i % 4
-  const int src_lane = (ei >> 2) * 16 + et, src_r = ei & 3;
+  // The sum of the four waves for (tile, row of the tile, token tile tn, token et): row r of a tile lies in
+  // MFMA lane (r / 4) * 16 + token, element r % 4.
+  auto summed = [&](int tile, int row, int tn) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+      sum += reinterpret_cast<const float*>(&red[((w * NT + tile) * TN + tn) * 64 + (row >> 2) * 16 + et])[row & 3];
+    return sum;
+  };
   // NORM: 1 / sqrt(mean(x^2) + eps) of this thread's token, from the four waves' shares of the sum
   const float scale_of = NORM ? rsqrtf((squares[et] + squares[16 + et] + squares[32 + et] + squares[48 + et]) / float(a.K) + a.eps)
                               : 1.f;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     const int t = tn * 16 + et;
+    if (EPI == kEpiSilu) {
+      const int r = a.rows_per_block;
+#pragma unroll
+      for (int o = 0; o < OUTS; ++o) {
+        const int p = 16 * o + ei, n = blockIdx.x * r + p;     // inner column p of the block
+        if (p >= r || n >= a.partner || t >= a.T) continue;
+        const int gate = p, up = p + r;                         // their places among the block's rows
+        const float gv = summed(gate >> 4, gate & 15, tn) * scale_of, uv = summed(up >> 4, up & 15, tn) * scale_of;
+        // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
+        const float g = to_float(bf16_t{f32_to_bf16_bits(gv)}), u = to_float(bf16_t{f32_to_bf16_bits(uv)});
+        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
+      }
+      continue;
+    }
     float v[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      float sum = 0.f;
-      if (NT == 1) {   // row er of the one tile (i = 0) and its partner, row 8 + er (i = 1)
-        const int row = er + 8 * i, lane_of = (row >> 2) * 16 + et;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[(w * TN + tn) * 64 + lane_of])[row & 3];
-      } else {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) sum += reinterpret_cast<const float*>(&red[((w * NT + i) * TN + tn) * 64 + src_lane])[src_r];
-      }
+      const float sum = (EPI == kEpiRope && NT == 1) ? summed(0, er + 8 * i, tn) : summed(i, ei, tn);
       v[i] = (NORM ? sum * scale_of : sum) + param_value(bias_bits[i], a.bias_bf16);
     }
-    if (t >= a.T || (NT == 1 && ei >= 8)) continue;
+    if (t >= a.T || (EPI == kEpiRope && NT == 1 && ei >= 8)) continue;
     if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const int n = row0[i] + ei;
+        const int n = 16 * (NT * blockIdx.x + i) + ei;
         if (n >= a.N) continue;
         const size_t o = size_t(t) * a.N + n;
         if (EPI == kEpiStore) reinterpret_cast<uint16_t*>(a.out)[o] = f32_to_bf16_bits(v[i]);
@@ -299,15 +364,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         else if (gridDim.y == 1) reinterpret_cast<float*>(a.out)[o] += v[i];
         else unsafeAtomicAdd(reinterpret_cast<float*>(a.out) + o, v[i]);
       }
-    } else if (EPI == kEpiSilu) {
-      const int n = row0[0] + ei;
-      if (n < a.partner) {
-        // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
-        const float g = to_float(bf16_t{f32_to_bf16_bits(v[0])}), u = to_float(bf16_t{f32_to_bf16_bits(v[1])});
-        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
-      }
     } else {  // kEpiRope
-      const int head = row0[0] / a.hd, d = row0[0] % a.hd + er;      // d < hd / 2; partner dim d + hd / 2
+      const int head = rope_head, d = rope_dim;      // d < hd / 2; partner dim d + hd / 2
       // projections are kept as bfloat16 before the rotation, as in the unfused path
       float lo = to_float(bf16_t{f32_to_bf16_bits(v[0])}), hi = to_float(bf16_t{f32_to_bf16_bits(v[1])});
       const int half = a.hd / 2;
@@ -348,18 +406,11 @@ static size_t fused_lds_bytes(int TN, bool norm, int NT = 2) {
 
 template <int TN, int EPI, bool NORM, int NT = 2>
 static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
-  const size_t lds = fused_lds_bytes(TN, NORM, NT);
-  static bool raised = false;
-  if (lds > 48 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_fused_kernel<TN, EPI, NORM, NT>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) {
-      set_error("sp_gemm_fused: cannot raise the LDS limit: %s", hipGetErrorString(e));
-      return 1;
-    }
-    raised = true;
-  }
-  gemm_fused_kernel<TN, EPI, NORM, NT><<<dim3(blocks, splits), 256, lds, s>>>(a);
+  const size_t lds = fused_lds_bytes(TN, NORM, NT);     // at most 48 KB (four token tiles of three tiles)
+  if (a.K % 64 == 0 && a.k_per_split % 64 == 0)
+    gemm_fused_kernel<TN, EPI, NORM, NT, true><<<dim3(blocks, splits), 256, lds, s>>>(a);
+  else
+    gemm_fused_kernel<TN, EPI, NORM, NT, false><<<dim3(blocks, splits), 256, lds, s>>>(a);
   return check_launch("sp_gemm_fused");
 }
 
@@ -371,6 +422,9 @@ static bool rope_one_tile(int T, int hd) { return T <= 16 || hd % 32 != 0; }
 
 template <int EPI, bool NORM>
 static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+  if constexpr (EPI == kEpiSilu) {   // up to 16 tokens: a block may own up to 24 inner columns (three tiles)
+    if (a.rows_per_block > 16) return launch_fused<1, EPI, NORM, 3>(s, a, blocks, splits);
+  }
   if constexpr (NORM) {   // one tile of up to 16 tokens (fused_shape_ok)
     if constexpr (EPI == kEpiRope) {
       if (rope_one_tile(a.T, a.hd)) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);
@@ -388,6 +442,24 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
     if (a.T <= 32) return launch_fused<2, EPI, false>(s, a, blocks, splits);
     return launch_fused<4, EPI, false>(s, a, blocks, splits);
   }
+}
+
+// Inner columns a block of the gated product owns.  A CU pulls its blocks' rows at about the same rate however
+// many blocks it holds, so the matrix is cut for the CU that gets the most: bytes a block asks for (its gate and
+// up rows, and the activations, which every block reads whole) times blocks per CU, rounded up.  4,864 inner
+// columns: 256 blocks of 19 instead of 304 of 16, of which 48 CUs held two.  More than 16 columns (three tiles)
+// only with up to 16 tokens.
+static int silu_rows_per_block(int T, int I, int K, bool norm) {
+  const int most = T <= 16 ? 24 : 16;
+  int best_rows = 16;
+  double best = 1e30;
+  for (int r = 4; r <= most; ++r) {
+    const int blocks = (I + r - 1) / r;
+    const double bytes = 4.0 * r * K + (norm ? 4.0 * min(T, 16) * K + 2.0 * K : 2.0 * T * K);
+    const double cost = double((blocks + 255) / 256) * bytes;
+    if (cost <= best) { best = cost; best_rows = r; }
+  }
+  return best_rows;
 }
 
 template <int EPI>
@@ -517,5 +589,6 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.out = out;
   a.T = T; a.N = 2 * I; a.K = K; a.k_per_split = (K + 63) / 64 * 64; a.partner = I;
-  return fused_norm<kEpiSilu>((hipStream_t)stream, a, residual != nullptr, (I + 15) / 16, 1);
+  a.rows_per_block = silu_rows_per_block(T, I, K, residual != nullptr);
+  return fused_norm<kEpiSilu>((hipStream_t)stream, a, residual != nullptr, (I + a.rows_per_block - 1) / a.rows_per_block, 1);
 }

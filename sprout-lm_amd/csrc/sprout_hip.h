@@ -58,8 +58,8 @@ int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, 
 // sp_attention_plan tells how the caller must list the work: tiles [n_tiles][2] = (sequence, first
 // query of the tile within the sequence's tokens) of plan[0] queries each, over every sequence
 // (plan[1] == 1) or over the sequences with more than one query only, the others being listed in
-// decode_seqs (plan[1] == 0; a null decode_seqs stands for sequences 0 .. n_decode - 1, which saves the kernels
-// one dependent read).  max_decode_ctx: largest ctx_len among decode_seqs; max_tile_ctx: largest
+// decode_seqs (plan[1] == 0; a null decode_seqs stands for sequences 0 .. n_decode - 1, each of one query, so that
+// q_start[s] == s, which saves the kernels two dependent reads).  max_decode_ctx: largest ctx_len among decode_seqs; max_tile_ctx: largest
 // ctx_len among the sequences of the tile list (it only guides how a long walk over the keys is shared out
 // between blocks: a smaller value than the truth costs time, not correctness); mean_tile_walk: the mean over
 // the tiles of the keys a tile walks (likewise a hint, 0 if unknown: where the longest walk is much longer than

@@ -252,7 +252,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     if n_decode:
         if decode is not None:         # None: sequences 0 .. n_decode - 1
             _ints(decode, n_decode, "decode_seqs")
-        elif n_decode != n_seqs:
+        elif n_decode != n_seqs or n_tiles:
+            # the kernels then take sequence i's query to be row i
             raise KernelError("attention: without a decode list every sequence must bring one query")
         if max_decode_ctx > block_tables.shape[1] * page_size:
             raise KernelError("attention: a decode context is longer than its block table")
