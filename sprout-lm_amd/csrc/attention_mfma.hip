@@ -33,10 +33,22 @@ struct PagedKV {
   int page_size, num_pages;
   size_t page_stride;    // elements between pages: nkv * page_size * HD
   int table_first = 0;   // the table entry that table[0] is (a copy of a part of the table starts later)
+  int page_shift = 0;    // POW2: page_size == 1 << page_shift
 };
 
+// Which page of the sequence a key lies in, and where in that page.  A division by a number that only the
+// launch knows is some forty vector instructions; pages of a power of two of tokens (POW2) need a shift.
+template <bool POW2>
+__device__ __forceinline__ int page_index(const PagedKV& kv, int key) {
+  return POW2 ? key >> kv.page_shift : key / kv.page_size;
+}
+template <bool POW2>
+__device__ __forceinline__ int page_offset(const PagedKV& kv, int key) {
+  return POW2 ? key & (kv.page_size - 1) : key % kv.page_size;
+}
+template <bool POW2>
 __device__ __forceinline__ int page_of(const PagedKV& kv, int key) {
-  const int page = kv.table[key / kv.page_size - kv.table_first];
+  const int page = kv.table[page_index<POW2>(kv, key) - kv.table_first];
   return min(max(page, 0), kv.num_pages - 1);   // a bad table entry must not become a wild address
 }
 
@@ -49,14 +61,14 @@ struct KVStep {
 
 // Requests the 32 keys starting at key0 (a multiple of 32).  Loads are clamped to keys in [k_lo, k_hi];
 // what lies outside is masked by position when the step is used.
-template <int DT>
+template <int DT, bool POW2 = false>
 __device__ __forceinline__ void load_step(KVStep<DT>& r, const PagedKV& kv, int key0, int k_lo, int k_hi) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   const int lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
 #pragma unroll
   for (int kt = 0; kt < 2; ++kt) {
     const int key = min(max(key0 + 16 * kt + lr, k_lo), k_hi);
-    const uint16_t* krow = kv.k + size_t(page_of(kv, key)) * kv.page_stride + size_t(key % kv.page_size) * HD;
+    const uint16_t* krow = kv.k + size_t(page_of<POW2>(kv, key)) * kv.page_stride + size_t(page_offset<POW2>(kv, key)) * HD;
 #pragma unroll
     for (int c = 0; c < HC; ++c) {
       const int d0 = 32 * c + 8 * lj;
@@ -68,7 +80,7 @@ __device__ __forceinline__ void load_step(KVStep<DT>& r, const PagedKV& kv, int 
   for (int kt = 0; kt < 2; ++kt) {
     int kb = key0 + 16 * kt + 4 * lj;
     kb = min(max(kb, (k_lo >> 2) << 2), (k_hi >> 2) << 2);
-    const uint16_t* vbase = kv.v + size_t(page_of(kv, kb)) * kv.page_stride + kb % kv.page_size;
+    const uint16_t* vbase = kv.v + size_t(page_of<POW2>(kv, kb)) * kv.page_stride + page_offset<POW2>(kv, kb);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
       r.va[dt][kt] = *reinterpret_cast<const uint2*>(vbase + size_t(16 * dt + lr) * kv.page_size);
@@ -525,7 +537,7 @@ __global__ __launch_bounds__(256) void attention_prefill_merge_kernel(
 // ------------------------------------------------------------------------------------------ decode
 // Partial results of a block, for the merge kernel: part_o [seq][head][split][HD] (not yet divided),
 // part_ml [seq][head][split][2] = (running maximum in log2 units, sum).
-template <int DT>
+template <int DT, bool POW2>
 __global__ __launch_bounds__(256) void attention_decode_kernel(
     const uint16_t* __restrict__ q, int q_stride, const uint16_t* __restrict__ k_pool,
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
@@ -541,7 +553,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   const int chunk0 = split * kDecodeChunk;
   // The page numbers of this chunk do not depend on how long the sequence is: they are asked for together with
   // its length (entries past the sequence's pages are never used), so that the keys are one trip further, not two.
-  const int table_first = chunk0 / page_size, table_count = (chunk0 + kDecodeChunk - 1) / page_size - table_first + 1;
+  int page_shift = 0;
+  if (POW2) page_shift = 31 - __builtin_clz(page_size);
+  const int table_first = POW2 ? chunk0 >> page_shift : chunk0 / page_size;
+  const int table_count = (POW2 ? (chunk0 + kDecodeChunk - 1) >> page_shift : (chunk0 + kDecodeChunk - 1) / page_size) - table_first + 1;
   if (int(threadIdx.x) < table_count)
     s_table[threadIdx.x] = block_tables[size_t(seq) * max_blocks + min(table_first + int(threadIdx.x), max_blocks - 1)];
   // without a list, sequence i's one query is row i
@@ -569,6 +584,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   kv.v = v_pool + size_t(g) * page_size * HD;
   kv.table = s_table;
   kv.table_first = table_first;
+  kv.page_shift = page_shift;
 
   bf16x8 qop[1][HC];
   int qpos[1] = {lr < G ? pos : -1};
@@ -587,7 +603,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i) {
     const int key0 = w0 + 32 * i;
     live[i] = key0 <= pos && key0 + 32 > k_lo;
-    if (live[i]) load_step<DT>(steps[i], kv, key0, k_lo, pos);
+    if (live[i]) load_step<DT, POW2>(steps[i], kv, key0, k_lo, pos);
   }
 #pragma unroll
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i)
@@ -926,9 +942,14 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
     const int n_splits = max(1, (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk);
     float* part_o = workspace;
     float* part_ml = workspace ? workspace + size_t(n_decode) * nq * n_splits * HD : nullptr;
-    attention_decode_kernel<DT><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
-        qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
-        n_splits, nq, nkv, page_size, num_pages, window, scale2);
+    if ((page_size & (page_size - 1)) == 0)
+      attention_decode_kernel<DT, true><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
+          n_splits, nq, nkv, page_size, num_pages, window, scale2);
+    else
+      attention_decode_kernel<DT, false><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+          qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
+          n_splits, nq, nkv, page_size, num_pages, window, scale2);
     if (check_launch("sp_attention (decode)")) return 1;
     if (n_splits > 1) {
       if (n_splits <= 16)
@@ -981,9 +1002,14 @@ static int launch_decode_project(hipStream_t s, const void* q, int q_stride, con
   const int n_splits = (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk;
   float* part_o = workspace;
   float* part_ml = workspace + size_t(n_decode) * nq * n_splits * HD;
-  attention_decode_kernel<DT><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
-      (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
-      ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
+  if ((page_size & (page_size - 1)) == 0)
+    attention_decode_kernel<DT, true><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+        (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
+  else
+    attention_decode_kernel<DT, false><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+        (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
   if (check_launch("sp_attention_decode_project (decode)")) return 1;
   const dim3 grid(nq, (hidden + 63) / 64);
 #define SP_PROJECT(TN)                                                                                          \

@@ -48,6 +48,7 @@ struct FusedArgs {
   uint16_t* k_pool;
   uint16_t* v_pool;
   int nq, nkv, hd, page_size, rotary_dim;
+  int page_shift;            // page_size == 1 << page_shift, or -1 where it is no power of two
 };
 
 // A bias value as it lies in memory (bfloat16 bits or float32 bits), and its value.  The two are kept apart
@@ -384,7 +385,14 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       } else {
         const int slot = slot_of[tn];
         if (slot >= 0) {
-          const int page = slot / a.page_size, off = slot % a.page_size;
+          int page, off;
+          if (a.page_shift >= 0) {      // the same for every thread: a scalar branch, and no division
+            page = slot >> a.page_shift;
+            off = slot & (a.page_size - 1);
+          } else {
+            page = slot / a.page_size;
+            off = slot % a.page_size;
+          }
           if (head < a.nq + a.nkv) {
             uint16_t* k = a.k_pool + ((size_t(page) * a.nkv + (head - a.nq)) * a.page_size + off) * a.hd;
             k[d] = blo;
@@ -572,6 +580,9 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.positions = positions; a.inv_freq = inv_freq; a.slot_mapping = slot_mapping;
   a.k_pool = (uint16_t*)k_pool; a.v_pool = (uint16_t*)v_pool;
   a.nq = nq; a.nkv = nkv; a.hd = hd; a.page_size = page_size; a.rotary_dim = rotary_dim;
+  a.page_shift = -1;
+  if (page_size > 0 && (page_size & (page_size - 1)) == 0)
+    for (a.page_shift = 0; (1 << a.page_shift) < page_size;) ++a.page_shift;
   const int blocks = (nq + 2 * nkv) * (hd / (rope_one_tile(T, hd) ? 16 : 32));
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
