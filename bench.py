@@ -28,25 +28,18 @@ HBM_PEAK_GBS = 8000.0                     # MI355X HBM3E, published
 MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense, published
 
 
-def weight_bytes_per_step(cfg, element: int) -> int:
-    """Every weight a decode step uses, read once (the embedding rows it gathers are negligible)."""
-    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
-    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
-    layer = H * (Q + 2 * KV) + (Q + 2 * KV) + Q * H + 3 * H * I + 2 * H
-    return (L * layer + V * H + H) * element
+# What a step has to read and to compute is asked of the model's parts (`ModelParts.weight_bytes`,
+# `.cache_bytes_per_context_token`, `.flops`): nothing here knows an architecture.
+
+def decode_step_bytes(parts, batch: int, context: int, element: int) -> int:
+    """Every weight a decode step uses, read once, and the cache of `batch` requests at `context` tokens."""
+    return parts.weight_bytes(element) + batch * context * parts.cache_bytes_per_context_token(element)
 
 
-def kv_bytes(cfg, batch: int, context: int, element: int) -> int:
-    KV = cfg.num_key_value_heads * cfg.head_dim
-    return batch * context * 2 * cfg.num_hidden_layers * KV * element
-
-
-def prefill_flops(cfg, T: int) -> float:
-    H, I, V, L = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.num_hidden_layers
-    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
-    linear = 2.0 * T * L * (H * (Q + 2 * KV) + Q * H + 3 * H * I)
-    attention = 2.0 * L * Q * T * T          # causal: half of 4 Q T^2
-    return linear + attention + 2.0 * V * H  # logits of the last position only
+def prefill_flops(parts, T: int) -> float:
+    """Matrix products of one fresh prompt of T tokens: every (query, key) pair of a causal prompt counted as
+    half of T x T, and the logits of the last position only."""
+    return parts.flops(T, T * T // 2, 1)
 
 
 def make_engine(cfg, dtype, batch, context, prefill_tokens, pages=None):
@@ -228,6 +221,7 @@ def main() -> int:
 
     biggest = max(args.batch, 1 if args.no_points else 64)
     engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
+    parts = engine.model.parts
     warmup = max(args.warmup, 1)
 
     step_s, spread = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
@@ -250,9 +244,9 @@ def main() -> int:
         del engine
         pressure = measure_pressure(cfg, dtype, args.batch, 512, 256, args.pressure)
 
-    read = weight_bytes_per_step(cfg, element) + kv_bytes(cfg, args.batch, args.context, element)
+    read = decode_step_bytes(parts, args.batch, args.context, element)
     achieved = read / step_s / 1e9
-    flops = prefill_flops(cfg, args.prefill_tokens)
+    flops = prefill_flops(parts, args.prefill_tokens)
     value = args.batch / step_s
     line = {
         "metric": f"decode tok/s at batch {args.batch} ({args.preset} sizes, context {args.context}); "

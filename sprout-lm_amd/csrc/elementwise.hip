@@ -287,7 +287,8 @@ extern "C" int sp_rmsnorm(void* stream, const float* x, const int32_t* rows, int
   return check_launch("sp_rmsnorm");
 }
 
-extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I) {
+extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation) {
+  SP_REQUIRE(activation == 0, "sp_silu_mul: no kernel for activation %d (0 = SiLU)", activation);
   SP_REQUIRE(T >= 0 && I > 0, "sp_silu_mul: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
@@ -324,7 +325,8 @@ extern "C" int sp_rope_table(void* stream, const int32_t* positions, const float
 extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions,
                              const float* inv_freq, const float* inv_freq_tail, int rotary_dim,
                              const int32_t* slot_mapping, void* k_pool,
-                             void* v_pool, int T, int nq, int nkv, int hd, int page_size, int num_pages) {
+                             void* v_pool, int T, int nq, int nkv, int hd, int page_size, int num_pages, int pairing) {
+  SP_REQUIRE(pairing == 0, "sp_rope_cache: no kernel for pairing %d (0 = halves of the rotated dimensions)", pairing);
   SP_REQUIRE(T >= 0 && nq > 0 && nkv >= 0 && hd > 0, "sp_rope_cache: bad sizes");
   SP_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0,
              "sp_rope_cache: rotary_dim %d must be even and at most head size %d", rotary_dim, hd);

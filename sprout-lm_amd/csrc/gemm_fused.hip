@@ -499,7 +499,8 @@ int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dt
                         void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, const float* table);
 }
 
-extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm) {
+extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm, int variant) {
+  if (variant != 0) return 0;   // the one pairing (halves) and the one activation (SiLU) these kernels have
   if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0;   // the tiled kernel's gated epilogue
   if (kind == kEpiRope && T > 64) return !norm && rotary_dim == hd && gemm_pipe_rope_takes(T, N, K, hd);   // and its rotating one
   if (!fused_shape_ok(T, K, norm != 0)) return 0;
@@ -564,9 +565,10 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
                                  const void* norm_w, float eps, const void* w, int bias_dtype, const void* bias,
                                  void* q_out, const int32_t* positions, const float* inv_freq, int rotary_dim,
                                  const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int K, int nq,
-                                 int nkv, int hd, int page_size, const float* cos_sin) {
+                                 int nkv, int hd, int page_size, const float* cos_sin, int pairing) {
   const int N = (nq + 2 * nkv) * hd;
-  SP_REQUIRE(sp_fused_supported(kEpiRope, T, N, K, hd, rotary_dim, residual != nullptr),
+  SP_REQUIRE(pairing == 0, "sp_qkv_rope_cache: no kernel for pairing %d (0 = halves of the rotated dimensions)", pairing);
+  SP_REQUIRE(sp_fused_supported(kEpiRope, T, N, K, hd, rotary_dim, residual != nullptr, pairing),
              "sp_qkv_rope_cache: shape T=%d K=%d hd=%d rotary=%d is not taken", T, K, hd, rotary_dim);
   SP_REQUIRE((x || residual) && w && q_out && positions && inv_freq && slot_mapping && k_pool && v_pool,
              "sp_qkv_rope_cache: null operand");
@@ -589,8 +591,10 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
 
 // out[T, I] = silu(x . w_gate^T) * (x . w_up^T) with w = [gate rows; up rows] of [2 I, K].
 extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype,
-                               const void* norm_w, float eps, const void* w, void* out, int T, int I, int K) {
-  SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr),
+                               const void* norm_w, float eps, const void* w, void* out, int T, int I, int K,
+                               int activation) {
+  SP_REQUIRE(activation == 0, "sp_gate_up_silu: no kernel for activation %d (0 = SiLU)", activation);
+  SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr, activation),
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
   // many tokens, or a few with whole steps of 64 along K: the tiled kernels stream the weights better

@@ -1,6 +1,10 @@
 // C interface of libsprout_hip.so.  Every function returns 0 on success; otherwise
 // sp_last_error() gives the reason.  Pointers are device pointers unless named host_*.
 // dtype codes: 0 = float32, 1 = bfloat16.  All launches go to `stream`.
+// Variants of an operation that parts may ask for are numbered, one `int` each; a number that no kernel
+// implements is refused with an error, so another variant is an addition here and in the kernels, never a guess:
+//   pairing of a rotation     0 = halves of the rotated dimensions (d with d + rotary_dim / 2, "neox")
+//   activation of a gated product   0 = SiLU (x / (1 + exp(-x)))
 #pragma once
 #include <stdint.h>
 
@@ -25,7 +29,8 @@ int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, const void* w
 // Decode-sized products (T <= 64, bfloat16) with neighbouring work folded in.  Activations are x
 // [T, K] bfloat16, or, with residual != null, rmsnorm(residual [T, K] float32) * norm_w computed inside.
 // sp_fused_supported(kind, ...): kind 0..2 = plain modes of sp_gemm, 3 = sp_qkv_rope_cache, 4 = sp_gate_up_silu.
-int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm);
+// `variant`: the pairing (kind 3) or the activation (kind 4) asked for; 0 otherwise.
+int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm, int variant);
 // Whether folding the norm into the product (norm = 1 above) is faster than a norm kernel before it.
 int sp_fused_norm_pays(int T, int N, int K);
 int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
@@ -37,12 +42,12 @@ int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int no
                       float eps, const void* w, int bias_dtype, const void* bias, void* q_out,
                       const int32_t* positions, const float* inv_freq, int rotary_dim, const int32_t* slot_mapping,
                       void* k_pool, void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size,
-                      const float* cos_sin);
+                      const float* cos_sin, int pairing);
 // out [T][half][2] = (cosine, sine) of positions[t] * inv_freq[d]: the same for every layer of a step.
 int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T);
 // out [T, I] = silu(x . w[:I]^T) * (x . w[I:]^T)
 int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
-                    const void* w, void* out, int T, int I, int K);
+                    const void* w, void* out, int T, int I, int K, int activation);
 
 // Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
 // inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
@@ -50,7 +55,7 @@ int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm
 // The key pool is [pages][nkv][page_size][hd], the value pool [pages][nkv][hd][page_size], of `dtype`.
 int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, const float* inv_freq,
                   const float* inv_freq_tail, int rotary_dim, const int32_t* slot_mapping, void* k_pool, void* v_pool, int T, int nq,
-                  int nkv, int hd, int page_size, int num_pages);
+                  int nkv, int hd, int page_size, int num_pages, int pairing);
 
 // Causal attention of a mixed batch over the paged pools.
 // q: [T, q_stride] (head h at column h * hd), out: [T, nq * hd].
@@ -89,8 +94,8 @@ int sp_attention_decode_project(void* stream, const void* q, int q_stride, const
                                 int hidden, int nq, int nkv, int hd, int page_size, int num_pages, int window,
                                 float scale);
 
-// out[t, i] = silu(gu[t, i]) * gu[t, I + i]
-int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I);
+// out[t, i] = act(gu[t, i]) * gu[t, I + i]
+int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation);
 
 // dst (dst_dtype) = src (src_dtype), n elements
 int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n);

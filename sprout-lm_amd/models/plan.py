@@ -107,6 +107,33 @@ class ModelParts:
         every += [getattr(b.mixer, "position", None) for b in self.blocks if hasattr(b, "mixer")]
         self.graph_safe = all(getattr(part, "graph_safe", False) for part in every if part is not None)
 
+    # ------------------------------------------------------------------ what a step costs, summed over the parts
+    def _calls(self):
+        """(block, cache slot) of every entry of the run order: a layer that runs twice counts twice."""
+        return [self.blocks[call.layer] for call in self.plan.schedule]
+
+    def weight_bytes(self, element_size: int) -> int:
+        """Bytes of weights that one step reads: every tensor of every part that runs, once."""
+        seen, total = set(), 0
+        parts = [self.final_norm, self.head] + [p for block in self._calls() for p in block.parts().values()]
+        for part in parts:
+            if id(part) not in seen:       # a layer that runs twice reads its weights twice, but from the caches
+                seen.add(id(part))
+                total += part.weight_elements()
+        return total * element_size
+
+    def cache_bytes_per_context_token(self, element_size: int) -> int:
+        """Cache bytes that one decoded token reads per token of its context, over all calls of the run order."""
+        return sum(block.mixer.cache_elements_per_token() for block in self._calls() if hasattr(block, "mixer")) * element_size
+
+    def flops(self, tokens: int, pairs: int, logit_rows: int) -> float:
+        """Matrix-product operations of a step of `tokens` tokens with `pairs` (query, key) pairs in every
+        mixer and `logit_rows` rows of logits."""
+        total = self.head.flops(logit_rows)
+        for block in self._calls():
+            total += sum(part.flops(tokens, pairs) for part in block.parts().values())
+        return total
+
     def expected_tensors(self) -> dict[str, TensorSpec]:
         out = {}
         for prefix, part in self._named:

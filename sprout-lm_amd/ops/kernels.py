@@ -59,6 +59,30 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+# Variants of an operation that a part may ask for, as the C interface numbers them.  Only the listed ones have
+# kernels; anything else is refused (KernelError) before a launch.
+ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox")
+GATE_ACTIVATIONS = {"silu": 0}
+MAX_HEAD_DIM = 256                       # the largest head size any attention kernel takes
+
+
+def variant_code(table: dict, name: str, what: str) -> int:
+    try:
+        return table[name]
+    except KeyError:
+        raise KernelError(f"No kernel for {what} {name!r}; there are kernels for: {sorted(table)}.") from None
+
+
+def check_attention_sizes(heads: int, kv_heads: int, head_dim: int) -> None:
+    """Raises KernelError unless some attention kernel takes these sizes (any page size goes with them).
+    Head sizes of 16 ... 96 in steps of 16 and 128 run on the matrix cores in bfloat16, every other size up to
+    256, and everything in float32, on the general kernel."""
+    if kv_heads <= 0 or heads <= 0 or heads % kv_heads:
+        raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key/value heads")
+    if not 0 < head_dim <= MAX_HEAD_DIM:
+        raise KernelError(f"attention: head size {head_dim} is outside 1..{MAX_HEAD_DIM}, the sizes the kernels take")
+
+
 def _check_pools(k_pool, v_pool, nkv: int, hd: int, dtype, what: str) -> tuple[int, int]:
     """Keys [pages, nkv, page_size, hd] and values [pages, nkv, hd, page_size]; returns (pages, page_size)."""
     _gpu(k_pool, "key pool"); _gpu(v_pool, "value pool")
@@ -124,10 +148,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: torch.Tensor
 
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rotary_dim: int, nq: int, nkv: int,
                hd: int, slot_mapping: torch.Tensor | None = None, k_pool: torch.Tensor | None = None,
-               v_pool: torch.Tensor | None = None, inv_freq_tail: torch.Tensor | None = None) -> None:
+               v_pool: torch.Tensor | None = None, inv_freq_tail: torch.Tensor | None = None, pairing: str = "halves") -> None:
     """Rotate q and k heads of qkv in place and write k, v into the pools (keys [pages, nkv, page, hd], values
     [pages, nkv, hd, page]).  `inv_freq_tail` (float32 qkv only): the float64 table minus `inv_freq`; with it
-    angles, sines and cosines are computed in float64."""
+    angles, sines and cosines are computed in float64.  `pairing`: which dimensions turn together."""
+    pairing_code = variant_code(ROTARY_PAIRINGS, pairing, "rotation pairing")
     _gpu(qkv, "qkv")
     T = qkv.shape[0]
     if qkv.shape[1] != (nq + 2 * nkv) * hd:
@@ -146,7 +171,7 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tenso
         num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, qkv.dtype, "rope_cache")
     check(library().sp_rope_cache(_stream(), _code(qkv, "qkv"), qkv.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(),
                                   _ptr(inv_freq_tail), rotary_dim, _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool), T, nq, nkv, hd, page_size,
-                                  num_pages))
+                                  num_pages, pairing_code))
 
 
 TILE_SIZES = (16, 32, 64)   # query-tile sizes an attention kernel may ask for
@@ -235,8 +260,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         raise KernelError("attention: bad q row stride")
     if nkv <= 0 or nq % nkv:
         raise KernelError(f"attention: {nq} query heads do not divide into {nkv} groups")
-    if not 0 < hd <= 256:
-        raise KernelError(f"attention: head size {hd} is outside 1..256")
+    check_attention_sizes(nq, nkv, hd)
     num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, q.dtype, "attention")
     _gpu(block_tables, "block tables")
     n_seqs = batch.n_seqs
@@ -300,9 +324,14 @@ def feed_tokens(tokens: torch.Tensor, previous: torch.Tensor, source: torch.Tens
 FUSED_ROPE, FUSED_SILU = 3, 4
 
 
-def fused_supported(kind: int, T: int, N: int, K: int, hd: int = 0, rotary_dim: int = 0, norm: bool = False) -> bool:
-    """Whether the decode-sized fused kernels take this shape (see sprout_hip.h)."""
-    return bool(library().sp_fused_supported(kind, T, N, K, hd, rotary_dim, int(norm)))
+def fused_supported(kind: int, T: int, N: int, K: int, hd: int = 0, rotary_dim: int = 0, norm: bool = False,
+                    variant: str | None = None) -> bool:
+    """Whether the fused kernels take this shape (see sprout_hip.h).  `variant`: the rotation's pairing
+    (FUSED_ROPE) or the gate's activation (FUSED_SILU) by name; one without a kernel is not taken."""
+    code = 0
+    if variant is not None:
+        code = (ROTARY_PAIRINGS if kind == FUSED_ROPE else GATE_ACTIVATIONS).get(variant, -1)
+    return bool(library().sp_fused_supported(kind, T, N, K, hd, rotary_dim, int(norm), code))
 
 
 def fused_norm_pays(T: int, N: int, K: int) -> bool:
@@ -325,7 +354,7 @@ def _activations(x, residual, norm_weight, K: int, what: str):
 
 def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_freq, rotary_dim: int, slot_mapping,
                    k_pool, v_pool, nq: int, nkv: int, hd: int, x=None, residual=None, norm_weight=None,
-                   eps: float = 0.0, table=None) -> None:
+                   eps: float = 0.0, table=None, pairing: str = "halves") -> None:
     """q, k, v = activations . w^T + bias; rotate q and k; q to q_out, k and v into the paged pools.
 
     Activations are x (bfloat16) or rmsnorm(residual) * norm_weight computed inside the kernel.
@@ -349,7 +378,8 @@ def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_fr
     check(library().sp_qkv_rope_cache(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(),
                                       _code(bias, "bias") if bias is not None else 0, _ptr(bias), q_out.data_ptr(),
                                       positions.data_ptr(), inv_freq.data_ptr(), rotary_dim, slot_mapping.data_ptr(),
-                                      k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd, page_size, _ptr(table)))
+                                      k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd, page_size, _ptr(table),
+                                      variant_code(ROTARY_PAIRINGS, pairing, "rotation pairing")))
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> None:
@@ -362,23 +392,26 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tenso
     check(library().sp_rope_table(_stream(), positions.data_ptr(), inv_freq.data_ptr(), half, out.data_ptr(), T))
 
 
-def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0) -> None:
-    """out = silu(a . w[:I]^T) * (a . w[I:]^T) for activations a as in `qkv_rope_cache`."""
+def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,
+                 activation: str = "silu") -> None:
+    """out = act(a . w[:I]^T) * (a . w[I:]^T) for activations a as in `qkv_rope_cache`."""
     _gpu(w, "gate/up weight"); _gpu(out, "gated output")
     N, K = w.shape
     xp, rp, nd, npt, T = _activations(x, residual, norm_weight, K, "gate_up_silu")
     if w.dtype != torch.bfloat16 or N % 2 or tuple(out.shape) != (T, N // 2) or out.dtype != torch.bfloat16:
         raise KernelError("gate_up_silu: weight [2 I, K] and output [T, I] bfloat16 expected")
-    check(library().sp_gate_up_silu(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), out.data_ptr(), T, N // 2, K))
+    check(library().sp_gate_up_silu(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), out.data_ptr(), T, N // 2, K,
+                                    variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
-def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, i] = silu(gu[t, i]) * gu[t, I + i]."""
+def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """out[t, i] = act(gu[t, i]) * gu[t, I + i]."""
     _gpu(gu, "gate/up"); _gpu(out, "gated output")
     T, I = out.shape
     if tuple(gu.shape) != (T, 2 * I) or gu.dtype != out.dtype:
         raise KernelError(f"silu_mul: shapes do not fit: gu {tuple(gu.shape)}, out {tuple(out.shape)}")
-    check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I))
+    check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I,
+                                variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
 def cast(src: torch.Tensor, dst: torch.Tensor) -> None:

@@ -21,7 +21,7 @@ def _declare(lib):
         "sp_rmsnorm": [c_void, c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int],
         "sp_gemm": [c_void, c_int, c_void, c_int, c_void, c_int, c_void, c_int, c_int, c_void, c_int, c_int, c_int],
         "sp_rope_cache": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int,
-                          c_int, c_int, c_int, c_int],
+                          c_int, c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
                          c_int, c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
                          c_int, c_int, c_float, c_int],
@@ -30,15 +30,15 @@ def _declare(lib):
                                         c_int, c_int, c_void, c_i64, c_void, c_void, c_int, c_int, c_int, c_int, c_int,
                                         c_int, c_int, c_float],
         "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
-        "sp_fused_supported": [c_int] * 7,
+        "sp_fused_supported": [c_int] * 8,
         "sp_fused_norm_pays": [c_int] * 3,
         "sp_gemm_decode": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_void, c_int,
                            c_int, c_int],
         "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,
-                              c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+                              c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_int],
         "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
-        "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int],
-        "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int],
+        "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
+        "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int, c_int],
         "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],

@@ -7,6 +7,7 @@ import torch
 
 from .. import ops
 from ..cache.spec import PagedKVSpec
+from ..config.base import ConfigError
 from ..weights.loader import TensorSpec
 from .norm import RMSNorm
 from .base import Mixer, register_part
@@ -29,8 +30,12 @@ class Attention(Mixer):
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
                  out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None):
-        if heads % kv_heads:
-            raise ValueError(f"{heads} query heads do not divide into {kv_heads} key/value heads.")
+        try:      # sizes no kernel takes are refused when the part is built, not at the first step
+            ops.check_attention_sizes(heads, kv_heads, head_dim)
+        except ops.KernelError as error:
+            raise ConfigError(str(error)) from None
+        if head_dim % 2 and getattr(position, "rotary_dim", 0):
+            raise ConfigError(f"A rotation needs an even head size, got {head_dim}.")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.position, self.qkv_bias, self.out_bias = position, qkv_bias, out_bias
         self.window, self.own_kv = window, own_kv
@@ -38,6 +43,14 @@ class Attention(Mixer):
 
     def cache_spec(self):
         return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
+
+    def cache_elements_per_token(self) -> int:
+        return 2 * self.kv_heads * self.head_dim
+
+    def flops(self, tokens: int, pairs: int = 0) -> float:
+        q, kv = self.heads * self.head_dim, (self.kv_heads * self.head_dim if self.own_kv else 0)
+        projections = 2.0 * tokens * self.hidden * (q + 2 * kv) + 2.0 * tokens * q * self.hidden
+        return projections + 4.0 * q * pairs          # scores and weighted values: two products over every pair
 
     def tensors(self):
         q, kv = self.heads * self.head_dim, self.kv_heads * self.head_dim
@@ -67,7 +80,7 @@ class Attention(Mixer):
         """Whether a projection kernel with bias, rotation and cache write folded in takes this call."""
         return (self.own_kv and cache.writes and self.w_qkv.dtype == torch.bfloat16
                 and ops.fused_supported(ops.FUSED_ROPE, T, self.w_qkv.shape[0], self.hidden, self.head_dim,
-                                        self.position.rotary_dim, norm))
+                                        self.position.rotary_dim, norm, variant=self.position.pairing))
 
     # Folding the norm into the projection kernel (up to 16 tokens) saves a launch; the kernel asks for the
     # residual rows before its weights, so the norm is computed while the weights are on their way.  Every
@@ -85,7 +98,7 @@ class Attention(Mixer):
         q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
         ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                            cache.slot_mapping, cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
-                           residual=residual, norm_weight=norm.w["weight"], eps=norm.eps)
+                           residual=residual, norm_weight=norm.w["weight"], eps=norm.eps, pairing=self.position.pairing)
         self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
         return True
 
@@ -109,7 +122,7 @@ class Attention(Mixer):
             table = self.position.table(ctx) if T > 64 and hasattr(self.position, "table") else None
             ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq,
                                self.position.rotary_dim, cache.slot_mapping, cache.k, cache.v, self.heads,
-                               self.kv_heads, self.head_dim, x=h, table=table)
+                               self.kv_heads, self.head_dim, x=h, table=table, pairing=self.position.pairing)
             self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
             return
         nkv = self.kv_heads if (self.own_kv and cache.writes) else 0
@@ -123,5 +136,6 @@ class Attention(Mixer):
         ops.rope_cache(qkv, ctx.positions, self.position.inv_freq, self.position.rotary_dim, self.heads, nkv,
                        self.head_dim, cache.slot_mapping if nkv else None, cache.k if nkv else None,
                        cache.v if nkv else None,
-                       inv_freq_tail=getattr(self.position, "inv_freq_tail", None) if qkv.dtype == torch.float32 else None)
+                       inv_freq_tail=getattr(self.position, "inv_freq_tail", None) if qkv.dtype == torch.float32 else None,
+                       pairing=self.position.pairing)
         self._attend(ctx, qkv, width, residual, cache)

@@ -61,6 +61,23 @@ class Part:
     def prepare(self, device, dtype) -> None:
         """Build device-side constants (tables of frequencies and the like).  Called once."""
 
+    # What a part costs, for measurement: the engine's bench adds these up over the model's parts and
+    # knows no architecture.
+    def weight_elements(self) -> int:
+        """Elements of the part's tensors that one step reads (every weight once, whatever the batch)."""
+        total = 0
+        for spec in self.tensors().values():
+            count = 1
+            for n in spec.shape:
+                count *= n
+            total += count
+        return total
+
+    def flops(self, tokens: int, pairs: int = 0) -> float:
+        """Floating-point operations of `forward` on `tokens` tokens (a multiply-add counts two).  `pairs`: the
+        number of (query, key) pairs of the step, for parts that mix tokens.  Matrix products only."""
+        return 0.0
+
 
 class Norm(Part):
     def forward(self, ctx, x, out, rows=None):
@@ -69,7 +86,14 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Turns positions into something a mixer applies to its queries and keys."""
+    """Turns positions into something a mixer applies to its queries and keys.
+
+    A rotary part provides `inv_freq` (float32 [rotary_dim / 2] on the device after `prepare`), `rotary_dim`
+    (0: nothing turns) and `pairing`: which dimensions turn together, by the name the kernels know it under
+    (`ops.ROTARY_PAIRINGS`; a pairing without a kernel is refused when the step is launched)."""
+
+    rotary_dim = 0
+    pairing = "halves"
 
 
 class Mixer(Part):
@@ -78,6 +102,10 @@ class Mixer(Part):
     def cache_spec(self):
         """A PagedKVSpec, a StateSpec, or None if the mixer keeps nothing between steps."""
         return None
+
+    def cache_elements_per_token(self) -> int:
+        """Cache elements that a decoded token reads per token of its context (keys and values)."""
+        return 0
 
     def forward(self, ctx, h, residual, cache):
         """residual += mixer(h).  `cache` is this call's cache slot view (engine.batch.CacheSlotView) or None."""

@@ -19,6 +19,9 @@ class TokenEmbedding(Part):
     def forward(self, ctx, tokens, residual):
         ops.embed(self.w["weight"], tokens, residual)
 
+    def weight_elements(self) -> int:
+        return 0      # a step gathers one row per token: nothing beside the matrices
+
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
@@ -43,3 +46,9 @@ class LinearHead(Part):
 
     def forward(self, ctx, h, logits):
         ops.gemm(h, self.table, logits)
+
+    def weight_elements(self) -> int:
+        return self.vocab * self.hidden      # the output matrix is read whole, also where it is the embedding table
+
+    def flops(self, tokens: int, pairs: int = 0) -> float:
+        return 2.0 * tokens * self.vocab * self.hidden

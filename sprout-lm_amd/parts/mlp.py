@@ -16,9 +16,13 @@ class GatedMLP(FeedForward):
     graph_safe = True
 
     def __init__(self, hidden: int, inner: int, activation: str = "silu"):
-        if activation != "silu":
-            raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; only 'silu'.")
+        if activation not in ops.GATE_ACTIVATIONS:     # refused when the part is built, not at the first step
+            raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; "
+                             f"there are kernels for {sorted(ops.GATE_ACTIVATIONS)}.")
         self.hidden, self.inner, self.activation = hidden, inner, activation
+
+    def flops(self, tokens: int, pairs: int = 0) -> float:
+        return 2.0 * tokens * 3 * self.hidden * self.inner
 
     def tensors(self):
         return {"gate_proj.weight": TensorSpec((self.inner, self.hidden)),
@@ -32,7 +36,7 @@ class GatedMLP(FeedForward):
 
     def _fused(self, T: int, norm: bool) -> bool:
         return self.w_gate_up.dtype == torch.bfloat16 and ops.fused_supported(ops.FUSED_SILU, T, 2 * self.inner,
-                                                                               self.hidden, norm=norm)
+                                                                               self.hidden, norm=norm, variant=self.activation)
 
     fuse_input_norm = True    # see Attention.fuse_input_norm
 
@@ -45,7 +49,8 @@ class GatedMLP(FeedForward):
         if not ops.fused_norm_pays(T, 2 * self.inner, self.hidden):
             return False
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=norm.w["weight"], eps=norm.eps)
+        ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=norm.w["weight"], eps=norm.eps,
+                         activation=self.activation)
         ops.gemm(act, self.w_down, residual, accumulate=True)
         return True
 
@@ -53,9 +58,9 @@ class GatedMLP(FeedForward):
         T = h.shape[0]
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
         if ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
-            ops.gate_up_silu(self.w_gate_up, act, x=h)
+            ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation)
         else:
             gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
             ops.gemm(h, self.w_gate_up, gu)
-            ops.silu_mul(gu, act)
+            ops.silu_mul(gu, act, activation=self.activation)
         ops.gemm(act, self.w_down, residual, accumulate=True)

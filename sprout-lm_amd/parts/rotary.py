@@ -18,6 +18,7 @@ class NeoxRotary(PositionEncoding):
     """
 
     graph_safe = True
+    pairing = "halves"      # which dimensions turn together, as the kernels name it (ops.ROTARY_PAIRINGS)
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
         self.head_dim, self.theta = head_dim, theta
@@ -53,6 +54,7 @@ class NoPosition(PositionEncoding):
     """No position encoding: queries and keys are used as projected."""
 
     rotary_dim = 0
+    pairing = "halves"      # nothing turns; the kernels are asked for the pairing they have
 
     graph_safe = True
 

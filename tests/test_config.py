@@ -76,3 +76,19 @@ def test_load_config_from_folder(tmp_path):
     assert S.load_config(str(tmp_path)).vocab_size == 256
     with pytest.raises(ConfigError):
         S.load_config(str(tmp_path / "missing"))
+
+
+def test_sizes_that_no_kernel_takes_are_refused_when_the_parts_are_built():
+    """Not at the first step: a head size beyond what the attention kernels take, or a feed-forward activation
+    or a rotation pairing without a kernel, fail where the model is put together from config.json."""
+    from sprout_lm_amd.config.base import ConfigError
+    from sprout_lm_amd.models.plan import PartPlan
+    from sprout_lm_amd import ops
+    raw = dict(H.TINY_A, hidden_size=1024, num_attention_heads=2, num_key_value_heads=1)     # head size 512
+    with pytest.raises(ConfigError, match="head size 512 is outside 1..256"):
+        S.build_model_plan(S.config_from_dict(raw)).instantiate()
+    with pytest.raises(ValueError, match="'gelu' has no kernel"):
+        PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "gelu"}).make()
+    with pytest.raises(ops.KernelError, match="rotation pairing 'interleaved'"):
+        ops.kernels.variant_code(ops.ROTARY_PAIRINGS, "interleaved", "rotation pairing")
+    assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0}

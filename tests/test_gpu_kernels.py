@@ -375,6 +375,82 @@ def test_attention_refuses_what_it_cannot_take():
         ops.attention(big, 512, pool, pool.transpose(2, 3).contiguous(), table, batch, torch.empty_like(big), 1, 1, 512, None, 0.1, kind=1)
 
 
+@pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, 0), (torch.float32, 1)])
+@pytest.mark.parametrize("seqs", [[(300, 1), (1, 1), (257, 1), (520, 1), (33, 1)], [(200, 200)], [(330, 70), (40, 1), (64, 64)]])
+def test_attention_at_the_head_counts_of_the_largest_model(dtype, kind, seqs):
+    """40 query heads in 8 groups of head size 128 (the 32B sizes): decoded tokens, a whole prompt, a mixed step."""
+    got, want = run_attention(dtype, 40, 8, 128, 16, seqs, kind=kind, seed=len(seqs))
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("T", [1, 8, 40, 300])
+@pytest.mark.parametrize("what", ["down", "gate_up", "qkv", "head"])
+def test_products_at_the_widths_of_the_largest_model(T, what):
+    """The products of the 32B sizes (a width of 5,120, 27,648 inner columns, 40 + 8 + 8 heads of 128) against a
+    float32 product of the same bfloat16 operands: every kernel that generation takes at these widths."""
+    from sprout_lm_amd import ops
+    gen = torch.Generator(device=DEV).manual_seed(T)
+    H, I, V = 5120, 27648, 152064
+    rand = lambda *shape, scale=1.0: (torch.randn(*shape, device=DEV, generator=gen) * scale).to(torch.bfloat16)
+    if what == "down":
+        x, w = rand(T, I), rand(H, I, scale=I ** -0.5)
+        before = torch.randn(T, H, device=DEV, generator=gen)
+        out = before.clone()
+        ops.gemm(x, w, out, accumulate=True)
+        want = before + x.float() @ w.float().T
+        tol = 2e-3          # float32 sums of 27,648 products, in another order
+    elif what == "gate_up":
+        x, w = rand(T, H), rand(2 * I, H, scale=H ** -0.5)
+        out = torch.empty(T, I, dtype=torch.bfloat16, device=DEV)
+        ops.gate_up_silu(w, out, x=x)
+        gu = (x.float() @ w.float().T).to(torch.bfloat16).float()
+        want = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+        out, tol = out.float(), 2 ** -6
+    elif what == "qkv":
+        N = (40 + 2 * 8) * 128
+        x, w, b = rand(T, H), rand(N, H, scale=H ** -0.5), rand(N, scale=0.3)
+        out = torch.empty(T, N, dtype=torch.bfloat16, device=DEV)
+        ops.gemm(x, w, out, bias=b)
+        want = x.float() @ w.float().T + b.float()
+        out, tol = out.float(), 2 ** -7
+    else:
+        T = min(T, 64)          # logits are asked for at a few places
+        x, w = rand(T, H), rand(V, H, scale=H ** -0.5)
+        out = torch.empty(T, V, dtype=torch.float32, device=DEV)
+        ops.gemm(x, w, out)
+        want = x.float() @ w.float().T
+        tol = 2e-3
+    err = (out - want).abs().max().item()
+    assert err <= tol * (1 + want.abs().max().item()), f"{what} at {T} tokens: {err:.3e}"
+
+
+def test_variants_without_a_kernel_are_refused_by_the_library_itself():
+    """A rotation's pairing and a gate's activation are parameters of the C entry points; a value that no
+    kernel implements comes back as an error, whoever calls."""
+    from sprout_lm_amd import ops
+    lib = ops.library()
+    stream = torch.cuda.current_stream().cuda_stream
+    qkv = torch.zeros(2, 4 * 16, device=DEV)
+    pos = torch.zeros(2, dtype=torch.int32, device=DEV)
+    inv = torch.ones(8, device=DEV)
+    args = (stream, 0, qkv.data_ptr(), pos.data_ptr(), inv.data_ptr(), None, 16, None, None, None, 2, 4, 0, 16, 0, 0)
+    assert lib.sp_rope_cache(*args, 0) == 0
+    assert lib.sp_rope_cache(*args, 1) != 0 and b"pairing 1" in lib.sp_last_error()
+    gu = torch.zeros(2, 32, device=DEV)
+    out = torch.zeros(2, 16, device=DEV)
+    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 0) == 0
+    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 3) != 0 and b"activation 3" in lib.sp_last_error()
+    assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 0) == 1
+    assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 1) == 0
+    assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 2) == 0
+    assert not ops.fused_supported(ops.FUSED_SILU, 8, 9728, 896, variant="gelu")
+    with pytest.raises(ops.KernelError, match="activation 'relu'"):
+        ops.silu_mul(gu, out, activation="relu")
+    torch.cuda.synchronize()
+
+
 def test_sampling_greedy_ties_nonfinite_and_temperature():
     from sprout_lm_amd import ops
     V = 151936 // 8 + 13

@@ -25,8 +25,9 @@ def requests_for(name, lengths, seed=100):
     return {f"r{i}": H.random_tokens(vocab, n, seed + i) for i, n in enumerate(lengths)}
 
 
-def replay_in_process(folder, name, dtype, trace, max_tokens, page=None, num_blocks=None):
-    """Drive the engine's TraceSession directly; returns per step the logits rows (or None)."""
+def replay_in_process(folder, name, dtype, trace, max_tokens, page=None, num_blocks=None, reused=None):
+    """Drive the engine's TraceSession directly; returns per step the logits rows (or None).
+    `reused`: a dict that receives, per physical page that served more than one request, those requests."""
     from sprout_lm_amd.engine import ModelRunner
     from sprout_lm_amd.engine.trace import TraceSession
     page = page or H.PAGE_SIZE[name]
@@ -34,9 +35,19 @@ def replay_in_process(folder, name, dtype, trace, max_tokens, page=None, num_blo
                                      max_sequences=8)
     session = TraceSession(runner)
     out = []
+    owners: dict = {}                      # physical page -> requests that held it, in order
     for record in trace.steps:
         logits = session.run_step(record)
         out.append(None if logits is None or not logits.shape[0] else logits.cpu().numpy().copy())
+        holders = {}
+        for rid, seq in session.live.items():
+            for page_id in seq.blocks[0]:
+                assert holders.setdefault(page_id, rid) == rid, f"page {page_id} is held by two requests at once"
+                if rid not in owners.setdefault(page_id, []):
+                    owners[page_id].append(rid)
+    if reused is not None:
+        reused.update({p: r for p, r in owners.items() if len(r) > 1})
+        assert len(owners) <= runner.cache.num_blocks
     assert runner.cache.free_pages() == [runner.cache.num_blocks], "pages were lost"
     assert not session.live
     return out
@@ -57,7 +68,7 @@ def check(folder, dtype, requests, trace, results):
     return worst
 
 
-LENGTHS = {"A": [5, 17, 33, 70, 128, 64], "B": [1, 9, 40, 70, 97, 33, 2], "C": [48, 130, 65]}
+LENGTHS = {"A": [5, 17, 33, 70, 128, 64], "B": [1, 9, 40, 70, 97, 33, 2], "C": [48, 130, 65, 200, 90, 33]}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -76,7 +87,10 @@ def test_replay_family(folders, name, dtype, family):
         # the pool holds exactly four requests rounded up to 64 tokens: pages are used again
         trace = traces.mixed(requests, seed=7)
         pool = sum(sorted(-(-len(t) // 64) * 64 for t in requests.values())[-4:])
-    results = replay_in_process(folders[name], name, dtype, trace, pool)
+    reused = {}
+    results = replay_in_process(folders[name], name, dtype, trace, pool, reused=reused)
+    if family == "mixed":     # what the family is for: later requests compute in pages that earlier ones gave back
+        assert len(reused) >= 2, "no page of the pool served two requests"
     worst = check(folders[name], dtype, requests, trace, results)
     print(f"{family} {name} {dtype}: {len(trace.steps)} steps, worst error {worst:.3e}")
 
@@ -89,7 +103,9 @@ def test_replay_with_pages_of_odd_sizes(folders, name, dtype, page):
     requests = requests_for(name, LENGTHS[name], seed=300)
     trace = traces.mixed(requests, seed=11)
     pages = sum(sorted(-(-len(t) // page) for t in requests.values())[-4:])
-    results = replay_in_process(folders[name], name, dtype, trace, None, page=page, num_blocks=pages)
+    reused = {}
+    results = replay_in_process(folders[name], name, dtype, trace, None, page=page, num_blocks=pages, reused=reused)
+    assert len(reused) >= 2, "no page of the pool served two requests"
     check(folders[name], dtype, requests, trace, results)
 
 
