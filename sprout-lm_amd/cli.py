@@ -4,8 +4,9 @@
     python -m sprout_lm_amd generate MODEL_DIR --prompt-ids 1,2,3 [--max-new-tokens N] ...
     python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b | --config FILE  --out DIR [--seed N]
 
-`demo` follows the reference's src/demo.ts (three requests, one arriving late, a table of work per
-tick; --pressure shrinks the pool so that requests are preempted).  `generate` follows
+`demo` is the counterpart of the reference's src/demo.ts, with the reference's two options: a few requests on a
+tiny random model, told round by round (--json: the same as one JSON document; --pressure: a pool so small that
+requests are preempted and their cache is computed again).  `generate` follows
 scripts/smoke-cuda.ts: one prompt on a model folder, one JSON line per scheduling round and a final
 report; the reference's environment variables MAX_NEW_TOKENS, KV_TOKENS, MAX_SEQUENCES,
 PREFILL_CHUNK_SIZE and REPORT_PATH are honoured as defaults of the options of the same meaning.
@@ -124,48 +125,88 @@ def cmd_generate(args) -> int:
 
 
 def cmd_demo(args) -> int:
-    """Three requests on a tiny random model; the third shares a prefix and arrives late (src/demo.ts:6-40)."""
+    """A few rounds of the engine on a tiny random model, told round by round.
+
+    Four requests with random token ids: `long` (a prompt that needs several portions), `short`, `twin` (it
+    starts with the first 16 tokens of `long` and arrives a round later, so it finds two of its pages in the
+    cache) and `late`, which arrives while the others decode and samples with a temperature.  Every round prints the one batch that the
+    model ran: portions of prompts beside single decoded tokens, flat in one step; whether the step was replayed
+    from a recorded graph and in which bucket (sequences, context); whether the round after it was already on the
+    GPU when this one's tokens came back; and what the cache pool looks like.  --pressure makes the pool so small
+    that requests lose their pages to older ones and compute them again.
+    """
+    import random
+
     import torch
     from .engine.engine import Engine
     from .weights.random_init import write_model_folder
-    config = preset_config("tiny-a")
+    config = preset_config("tiny-b")
+    page, pages = 8, (9 if args.pressure else 24)
     with tempfile.TemporaryDirectory() as folder:
-        write_model_folder(folder, config, seed=1, dtype=torch.bfloat16, std=0.08)
-        engine = Engine.from_folder(folder, args.dtype, block_size=4, num_blocks=5 if args.pressure else 18,
-                                    max_sequences=3, max_batch_tokens=6, prefill_chunk_size=4, record_trace=True)
-    encode = lambda text: [ord(c) % config.vocab_size for c in text]
-    reports = []
-    if not args.json:
-        print("sprout-lm_amd demo · MI355X / random UNTRAINED Qwen2 weights")
-        print("Token ids show scheduling and numerical correctness, not language quality.\n")
-    engine.add("A", encode("shared: hi"), 7, ignore_eos=True)
-    engine.add("B", encode("other"), 4, ignore_eos=True)
-    iterations = 0
-    while engine.pending:
-        if iterations == 2:
-            engine.add("C", encode("shared: bye"), 3, ignore_eos=True)
-        iterations += 1
-        if iterations > 2000:
-            raise RuntimeError("Demo did not converge.")
+        write_model_folder(folder, config, seed=2, dtype=torch.bfloat16, std=0.08)
+        engine = Engine.from_folder(folder, args.dtype, block_size=page, num_blocks=pages, max_sequences=3,
+                                    max_batch_tokens=24, prefill_chunk_size=16, record_trace=True)
+    rng = random.Random(5)
+    ids = lambda n: [rng.randrange(config.vocab_size - 2) for _ in range(n)]
+    long_prompt = ids(40)
+    # before which round each request arrives: `twin` after `long` has computed (and offered) its first pages
+    arrivals = {0: [("long", long_prompt, 10, {}), ("short", ids(6), 12, {})],
+                1: [("twin", long_prompt[:16] + ids(5), 8, {})],
+                5: [("late", ids(11), 6, {"temperature": 0.8, "seed": 7})]}
+    say = (lambda *a: None) if args.json else print
+    say(f"sprout-lm_amd demo: {config.num_hidden_layers}-layer Qwen2 of random weights in {args.dtype} on "
+        f"{torch.cuda.get_device_name()}; {pages} pages of {page} tokens, 3 sequences, 24 tokens a step")
+    say("(token ids only: the weights are untrained, what is shown is the engine at work)\n")
+    from .engine.graphs import _bucket
+    rounds, round_no = [], 0
+    while engine.pending or any(r >= round_no for r in arrivals):
+        for name, prompt, new, sampling in arrivals.get(round_no, []):
+            engine.add(name, prompt, new, ignore_eos=True, **sampling)
+        round_no += 1
+        if round_no > 500:
+            raise RuntimeError("the demo's requests did not finish in 500 rounds")
         report = engine.step()
-        reports.append(report.to_dict())
-        if not args.json:
-            memory = report.memory
-            print(f"Tick {report.tick} | free pages {memory['free_pages']}/{memory['total_pages']} | cached {memory['cached_pages']}")
-            for w in report.work:
-                pages = " ".join(f"{i}→{p}" for i, p in enumerate(w["block_table"][0])) if w["block_table"] else ""
-                print(f"  {w['id']:>2} {w['phase']:<9} position {w['from']:>3} tokens {w['tokens']}  pages {pages}")
-            for event in report.events:
-                print(f"  {event['id']} {event['type']}: {event['detail']}")
-            print()
-    results = [engine.result(i) for i in "ABC"]
+        graphs = engine.model._graphs
+        replayed = report.replayed
+        bucket = None
+        if replayed:     # the recorded graph of this many sequences (rounded up to a power of two), last used first
+            bucket = next((k for k in reversed(list(graphs.graphs)) if k[0] == _bucket(len(report.work))), None)
+        record = {"round": round_no, "work": report.work, "events": report.events, "from_graph": replayed,
+                  "graph_bucket": bucket, "launched_ahead": report.launched_ahead,
+                  "next_round_already_launched": engine._ahead is not None,
+                  "free_pages": report.memory["free_pages"], "cached_pages": report.memory["cached_pages"]}
+        rounds.append(record)
+        if args.json:
+            continue
+        batch = " + ".join(f"{w['tokens']} of {w['id']} ({w['phase']} from {w['from']})" for w in report.work) or "nothing to run"
+        how = "launched kernel by kernel"
+        if replayed:
+            how = f"graph replay, bucket {bucket[0]} sequences x {bucket[1]} keys" if bucket else "graph replay"
+            how += " (launched during the round before)" if report.launched_ahead else ""
+        ahead = "; the next round is already on the GPU" if record["next_round_already_launched"] else ""
+        say(f"round {round_no:>2}: one batch of {sum(w['tokens'] for w in report.work)} tokens = {batch}")
+        say(f"          {how}{ahead}; pages free {record['free_pages']}/{pages}, kept for reuse {record['cached_pages']}")
+        for event in report.events:
+            if event["type"] != "token":
+                say(f"          {event['id']}: {event['type']} - {event['detail']}")
+        made = {e['id']: e['token'] for e in report.events if e['type'] == 'token'}
+        if made:
+            say("          new tokens: " + ", ".join(f"{k} -> {v}" for k, v in made.items()))
+    results = {name: engine.result(name) for name in ("long", "short", "twin", "late")}
+    stats = engine.stats()
+    replays = engine.model._graphs.replays if engine.model._graphs else 0
+    summary = {"mode": "pressure" if args.pressure else "roomy", "rounds": rounds, "results": results, "stats": stats,
+               "graphs_recorded": len(engine.model._graphs.graphs) if engine.model._graphs else 0, "graph_replays": replays}
     if args.json:
-        print(json.dumps({"mode": "pressure" if args.pressure else "normal", "reports": reports, "results": results}, indent=2))
+        print(json.dumps(summary, indent=2))
     else:
-        print("Results:")
-        for r in results:
-            print(f"  {r['id']}: {r['status']}, prefix tokens reused {r['prefix_hits']}, output {r['output']}")
-        print("Cached pages may remain after requests finish; their active_refs are zero.")
+        say("\nwhat came out:")
+        for name, r in results.items():
+            say(f"  {name:>5}: {r['status']} ({r['finish_reason']}), {r['prefix_hits']} prompt tokens found in the cache, "
+                f"preempted {r['preemptions']} times, output {r['output']}")
+        say(f"  {stats['preemptions']} preemptions, {stats['recomputed_tokens']} tokens computed again, "
+            f"{summary['graphs_recorded']} graphs recorded and replayed {replays} times in {round_no} rounds")
+    engine.close()
     return 0
 
 
@@ -174,9 +215,9 @@ def main(argv=None) -> int:
                                      formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = parser.add_subparsers(dest="command", required=True)
 
-    demo = sub.add_parser("demo", help="three requests on a tiny random model, tick by tick")
+    demo = sub.add_parser("demo", help="four requests on a tiny random model, round by round")
     demo.add_argument("--json", action="store_true")
-    demo.add_argument("--pressure", action="store_true", help="a pool of 5 pages: requests are preempted")
+    demo.add_argument("--pressure", action="store_true", help="a pool of 9 pages: requests are preempted")
     demo.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     demo.set_defaults(run=cmd_demo)
 

@@ -17,8 +17,11 @@ from .scheduler import Scheduler, Work
 class StepReport:
     """What one scheduling iteration did (reference: src/engine.ts:27-33, :189)."""
 
-    def __init__(self, tick, work, events, cache):
+    def __init__(self, tick, work, events, cache, replayed=False, launched_ahead=False):
         self.tick, self.work, self.events = tick, work, events
+        # beyond the reference's report: the step ran as a replay of a recorded graph; it had been launched
+        # before the step before it was read back
+        self.replayed, self.launched_ahead = replayed, launched_ahead
         self._cache = cache
         self._memory = None
 
@@ -29,7 +32,8 @@ class StepReport:
         return self._memory
 
     def to_dict(self) -> dict:
-        return {"tick": self.tick, "work": self.work, "events": self.events, "memory": self.memory}
+        return {"tick": self.tick, "work": self.work, "events": self.events, "memory": self.memory,
+                "replayed": self.replayed, "launched_ahead": self.launched_ahead}
 
 
 class Engine:
@@ -145,7 +149,8 @@ class Engine:
             sampled = {w.request.id: t for w, t in zip(sampling, tokens)}
             reports = [w.report() for w in work]
         events = self.scheduler.complete(work, sampled)
-        return StepReport(self.scheduler.tick, reports, events, self.cache)
+        return StepReport(self.scheduler.tick, reports, events, self.cache, replayed=pending is not None,
+                          launched_ahead=ahead is not None)
 
     @staticmethod
     def _discard(ahead) -> None:

@@ -22,6 +22,33 @@ from ..config.engine_options import EngineOptions
 from ..sampling.params import SamplingParams
 
 
+class RequestRefused(ValueError):
+    """A request that can never run: its id, its tokens or its length do not fit this engine."""
+
+
+@dataclass(frozen=True)
+class Limits:
+    """What a request is measured against when it arrives."""
+
+    vocab_size: int
+    max_context: int      # positions the model has
+    pool_tokens: int      # token slots of the whole cache pool
+
+
+@dataclass(frozen=True)
+class Event:
+    """Something that happened to a request in a scheduling round.  Reports and traces carry `to_dict()`."""
+
+    tick: int
+    id: str
+    kind: str             # queued | admitted | token | finished | cancelled | preempted
+    detail: str
+    extra: tuple = ()     # (key, value) pairs of the kind's own fields: token and index, finish_reason
+
+    def to_dict(self) -> dict:
+        return {"tick": self.tick, "id": self.id, "type": self.kind, "detail": self.detail, **dict(self.extra)}
+
+
 @dataclass
 class Request:
     id: str
@@ -35,6 +62,31 @@ class Request:
     prefix_hits: int = 0
     finish_reason: str | None = None   # eos | length
     preemptions: int = 0
+
+    @classmethod
+    def checked(cls, id, order: int, prompt, max_new_tokens, params: SamplingParams, limits: Limits, known_ids) -> "Request":
+        """A new request, or RequestRefused saying what is wrong with it.  What is checked is what the reference
+        checks when a request arrives (src/engine.ts:74-85): the id, the token ids, the number of new tokens, and
+        that the request could run at all: the last token it samples is never fed back, so it needs one cache slot
+        less than it has tokens."""
+        if not isinstance(id, str) or id == "" or id in known_ids:
+            raise RequestRefused(f"A request needs an id of its own: {id!r} is empty, no string, or already in use.")
+        tokens = list(prompt)
+        if not tokens:
+            raise RequestRefused(f"Request {id!r} brings no prompt: at least one token id in [0, {limits.vocab_size}) is needed.")
+        for place, token in enumerate(tokens):
+            if isinstance(token, bool) or not isinstance(token, int) or not 0 <= token < limits.vocab_size:
+                raise RequestRefused(f"Request {id!r}: prompt[{place}] = {token!r} is no token id in [0, {limits.vocab_size}).")
+        if isinstance(max_new_tokens, bool) or not isinstance(max_new_tokens, int) or max_new_tokens < 1:
+            raise RequestRefused(f"Request {id!r}: max_new_tokens must be a positive integer, got {max_new_tokens!r}.")
+        slots = len(tokens) + max_new_tokens - 1
+        if slots > limits.max_context:
+            raise RequestRefused(f"Request {id!r}: {len(tokens)} prompt tokens and {max_new_tokens} new ones need "
+                                 f"{slots} positions, the model has {limits.max_context}.")
+        if slots > limits.pool_tokens:
+            raise RequestRefused(f"Request {id!r}: {slots} cache slots are more than the whole pool holds "
+                                 f"({limits.pool_tokens} = num_blocks x block_size), even with nothing else running.")
+        return cls(id, order, tokens, max_new_tokens, params)
 
     def history(self) -> list:
         return self.prompt + self.output
@@ -73,67 +125,63 @@ class Scheduler:
         self.cache, self.options = cache, options
         self.vocab_size, self.max_context = vocab_size, max_context
         self.eos_token_ids = tuple(eos_token_ids)
+        self.limits = Limits(vocab_size, max_context, options.num_blocks * options.block_size)
         self.requests: dict[str, Request] = {}
         self.active: dict[str, Request] = {}
         self.waiting: list[str] = []
         self.trace: list[dict] = []
         self.tick = 0
-        self._next_order = 0
+        self._arrivals = 0
         self._step_events: list[dict] | None = None
         self.stats = {"preemptions": 0, "recomputed_tokens": 0, "prefix_hit_tokens": 0}
 
     # ------------------------------------------------------------------ requests
     def add(self, id: str, prompt, max_new_tokens: int, params: SamplingParams | None = None) -> None:
-        """Reference: Engine.add, src/engine.ts:74-93 (same checks, same order)."""
-        if not isinstance(id, str) or not id or id in self.requests:
-            raise ValueError("Request ID must be nonempty and unique.")
-        prompt = list(prompt)
-        if not prompt or any(isinstance(t, bool) or not isinstance(t, int) or t < 0 or t >= self.vocab_size for t in prompt):
-            raise ValueError("Prompt must contain valid token IDs.")
-        if isinstance(max_new_tokens, bool) or not isinstance(max_new_tokens, int) or max_new_tokens <= 0:
-            raise ValueError("max_new_tokens must be a positive integer.")
-        # the last sampled token is never fed back, so it needs no cache slot
-        slots = len(prompt) + max_new_tokens - 1
-        if slots > self.max_context:
-            raise ValueError("Request exceeds the model context limit.")
-        if slots > self.options.num_blocks * self.options.block_size:
-            raise ValueError("Request cannot fit alone in the KV pool. Increase num_blocks or shorten it.")
-        request = Request(id, self._next_order, prompt, max_new_tokens, params or SamplingParams())
-        self._next_order += 1
-        self.requests[id] = request
-        self.waiting.append(id)
-        self._emit("queued", request, f"{len(prompt)} prompt tokens")
+        """Take a request into the waiting line (first come, first admitted), or raise RequestRefused."""
+        request = Request.checked(id, self._arrivals, prompt, max_new_tokens, params or SamplingParams(), self.limits,
+                                  self.requests)
+        self._arrivals += 1
+        self.requests[request.id] = request
+        self.waiting.append(request.id)
+        self._note(request, "queued", f"waits with {len(request.prompt)} prompt tokens for up to {max_new_tokens} new ones")
 
     @property
     def pending(self) -> bool:
         return bool(self.active or self.waiting)
 
-    def forget(self, id: str) -> bool:
+    def _alive(self, id: str) -> Request | None:
+        """The request if it still waits or runs."""
         request = self.requests.get(id)
-        if request is None or request.status in ("waiting", "running"):
+        return request if request is not None and request.status in ("waiting", "running") else None
+
+    def forget(self, id: str) -> bool:
+        """Drop the record of a request that has ended; False for one that is unknown or still alive."""
+        if id not in self.requests or self._alive(id) is not None:
             return False
         del self.requests[id]
         return True
 
     def cancel(self, id: str) -> bool:
-        request = self.requests.get(id)
-        if request is None or request.status in ("finished", "cancelled"):
+        """End a waiting or running request now.  Its pages go back to the pool at once (pages it shares with
+        the prefix cache or with other requests stay with those); False if there was nothing to end."""
+        request = self._alive(id)
+        if request is None:
             return False
-        self._drop_cache(request)
-        request.status = "cancelled"
-        self.active.pop(id, None)
-        self.waiting = [w for w in self.waiting if w != id]
-        self._emit("cancelled", request, "Released live KV references")
+        held = sum(len(b) for b in request.seq.blocks) if request.seq else 0
+        self._leave(request, "cancelled")
+        self._note(request, "cancelled", f"stopped after {len(request.output)} tokens; {held} page references given back")
         return True
 
     def result(self, id: str) -> dict:
-        request = self.requests.get(id)
-        if request is None:
-            raise KeyError(f"Unknown request: {id}")
+        """Where a request stands (reference: Engine.result, src/engine.ts:111-124, plus `preemptions`)."""
+        if id not in self.requests:
+            raise KeyError(f"No request {id!r} is known to the engine (finished requests stay until `forget`).")
+        request = self.requests[id]
+        seq = request.seq
         return {"id": id, "status": request.status, "output": list(request.output),
                 "finish_reason": request.finish_reason,
-                "computed_tokens": request.seq.length if request.seq else 0,
-                "block_table": list(request.seq.blocks[0]) if request.seq and request.seq.blocks else [],
+                "computed_tokens": seq.length if seq else 0,
+                "block_table": list(seq.blocks[0]) if seq and seq.blocks else [],
                 "prefix_hits": request.prefix_hits, "preemptions": request.preemptions}
 
     # ------------------------------------------------------------------ one step
@@ -157,23 +205,23 @@ class Scheduler:
             remaining = total - start - (phase == "recompute")
             count = min(budget, 1 if phase == "decode" else self.options.prefill_chunk_size, remaining)
             multiple = self.options.step_token_multiple
+            closes_step = False
             if multiple > 1 and phase != "decode" and count < remaining:
                 # a portion that carries the step over a whole multiple is cut back to it and closes the step
                 # (a portion that ends its prompt is left alone: the request's first token is not held back)
                 used = sum(len(w.tokens) for w in planned.values())
                 aligned = (used + count) // multiple * multiple - used
                 if 0 < aligned < count:
-                    count = aligned
-                    budget = count
+                    count, closes_step = aligned, True
             if count <= 0:
                 continue
             ok, refund = self._reserve(request, start + count, planned)
             budget += refund
             if not ok:
-                continue
+                continue      # the step goes on with its whole budget: nothing was cut for a portion that is not in it
             tokens = request.history_slice(start, start + count)
             planned[request.id] = Work(request, phase, start, tokens, samples=start + count == total)
-            budget -= count
+            budget = 0 if closes_step else budget - count
         return [planned[r.id] for r in batch if r.id in planned]
 
     def plan_ahead(self, running: list[Work]) -> list[Work] | None:
@@ -229,16 +277,14 @@ class Scheduler:
             if isinstance(token, bool) or not isinstance(token, int) or token < 0 or token >= self.vocab_size:
                 raise RuntimeError("Runner returned invalid sampled token.")
             request.output.append(token)
-            self._emit("token", request, str(token), token=token, index=len(request.output) - 1)
+            self._note(request, "token", f"token {token}", token=token, index=len(request.output) - 1)
             stops = request.params.stop_token_ids if request.params.stop_token_ids is not None else self.eos_token_ids
             eos = token in stops and not request.params.ignore_eos
             if eos or len(request.output) == request.max_new_tokens:
                 request.finish_reason = "eos" if eos else "length"
-                request.status = "finished"
-                self._drop_cache(request)
-                del self.active[request.id]
-                self._emit("finished", request, f"{len(request.output)} output tokens",
-                           finish_reason=request.finish_reason)
+                self._leave(request, "finished")
+                self._note(request, "finished", f"{len(request.output)} tokens, ended by "
+                           + ("a stop token" if eos else "its length limit"), finish_reason=request.finish_reason)
         events, self._step_events = self._step_events or [], None
         return events
 
@@ -246,11 +292,8 @@ class Scheduler:
         """A step failed: every request ends and every page comes back (reference: src/service.ts:222-231)."""
         for request in list(self.requests.values()):
             if request.status in ("waiting", "running"):
-                self._drop_cache(request)
-                request.status = "cancelled"
-                self._emit("cancelled", request, f"engine_error: {reason}")
-        self.active.clear()
-        self.waiting.clear()
+                self._leave(request, "cancelled")
+                self._note(request, "cancelled", f"engine_error: {reason}")
         self.cache.clear_prefixes()
 
     # ------------------------------------------------------------------ internals
@@ -260,15 +303,22 @@ class Scheduler:
         return "recompute" if request.seq.length < len(request.prompt) + len(request.output) - 1 else "decode"
 
     def _admit(self) -> None:
-        while len(self.active) < self.options.max_sequences and self.waiting:
+        """Waiting requests start in arrival order while a sequence slot is free.  A request that was preempted
+        comes back with its output: whatever of its prompt still lies in cached pages is found again, the rest of
+        its history is computed again (reference: src/engine.ts:197-207)."""
+        while self.waiting and len(self.active) < self.options.max_sequences:
             request = self.requests[self.waiting.pop(0)]
-            history = request.history()
-            request.seq = self.cache.reuse_prefix(history) if self.options.prefix_caching else self.cache.create()
-            request.prefix_hits += request.seq.length
-            self.stats["prefix_hit_tokens"] += request.seq.length
+            if self.options.prefix_caching:
+                request.seq = self.cache.reuse_prefix(request.history())
+            else:
+                request.seq = self.cache.create()
+            found = request.seq.length
+            request.prefix_hits += found
+            self.stats["prefix_hit_tokens"] += found
             request.status = "running"
             self.active[request.id] = request
-            self._emit("admitted", request, f"Reused {request.seq.length} prefix tokens; pages {request.seq.blocks}")
+            self._note(request, "admitted", f"{found} of {request.history_length()} tokens found in cached pages "
+                       f"{[list(b) for b in request.seq.blocks]}" if found else f"starts with an empty cache")
 
     def _reserve(self, request: Request, new_length: int, planned: dict) -> tuple[bool, int]:
         """Pages for `request` up to `new_length`; preempts younger requests, else the request itself.
@@ -291,21 +341,26 @@ class Scheduler:
         return True, refund
 
     def _preempt(self, request: Request) -> None:
-        self._drop_cache(request)
-        request.status = "waiting"
+        """Back to the end of the waiting line with nothing but its tokens (src/engine.ts:224-231)."""
+        self._leave(request, "waiting")
         request.preemptions += 1
         self.stats["preemptions"] += 1
-        del self.active[request.id]
         self.waiting.append(request.id)
-        self._emit("preempted", request, "Keep output tokens; rebuild missing KV after readmission")
+        self._note(request, "preempted", f"pages given up for an older request; its {len(request.output)} tokens are "
+                   f"kept and the cache is computed again after readmission")
 
-    def _drop_cache(self, request: Request) -> None:
+    def _leave(self, request: Request, status: str) -> None:
+        """The request stops running or waiting: its cache goes back to the pool, the books forget it."""
         if request.seq is not None:
             request.seq.release()
             request.seq = None
+        request.status = status
+        self.active.pop(request.id, None)
+        if request.id in self.waiting:
+            self.waiting.remove(request.id)
 
-    def _emit(self, type: str, request: Request, detail: str, **extra) -> None:
-        event = {"tick": self.tick, "id": request.id, "type": type, "detail": detail, **extra}
+    def _note(self, request: Request, kind: str, detail: str, **extra) -> None:
+        event = Event(self.tick, request.id, kind, detail, tuple(extra.items())).to_dict()
         if self.options.record_trace:
             self.trace.append(event)
         if self._step_events is not None:

@@ -132,12 +132,27 @@ def test_command_line_generate_and_demo(folders, tmp_path):
     assert final["phase"] == "finished" and len(final["output"]) == 5
     assert final["output"] == plain_greedy(folders["A"], "float32", [3, 1, 4, 1, 5, 9, 2, 6], 5)[0]
     assert json.load(open(report))["output"] == final["output"]
-    demo = subprocess.run([sys.executable, "-m", "sprout_lm_amd", "demo", "--json", "--pressure"], cwd=ROOT,
-                          capture_output=True, text=True, timeout=120)
-    assert demo.returncode == 0, demo.stderr
-    shown = json.loads(demo.stdout)
-    assert shown["mode"] == "pressure" and [r["status"] for r in shown["results"]] == ["finished"] * 3
-    assert [len(r["output"]) for r in shown["results"]] == [7, 4, 3]
+    shown = {}
+    for mode in ("--pressure", None):
+        demo = subprocess.run([sys.executable, "-m", "sprout_lm_amd", "demo", "--json"] + ([mode] if mode else []), cwd=ROOT,
+                              capture_output=True, text=True, timeout=120)
+        assert demo.returncode == 0, demo.stderr
+        shown[mode] = json.loads(demo.stdout)
+        results = shown[mode]["results"]
+        assert [results[k]["status"] for k in ("long", "short", "twin", "late")] == ["finished"] * 4
+        assert [len(results[k]["output"]) for k in ("long", "short", "twin", "late")] == [10, 12, 8, 6]
+    roomy, tight = shown[None], shown["--pressure"]
+    assert tight["mode"] == "pressure" and tight["stats"]["preemptions"] > 0 and tight["stats"]["recomputed_tokens"] > 0
+    assert roomy["stats"]["preemptions"] == 0 and roomy["results"]["twin"]["prefix_hits"] == 16
+    # what the demo is there to show: a round whose one batch mixes a portion of a prompt with decoded tokens,
+    # rounds replayed from a recorded graph, and rounds whose successor was launched before they were read back
+    assert any({w["phase"] for w in r["work"]} >= {"prefill", "decode"} for r in roomy["rounds"])
+    assert roomy["graph_replays"] > 0 and any(r["next_round_already_launched"] for r in roomy["rounds"])
+    # scheduling changes nothing of what the greedy requests generate
+    for k in ("long", "short", "twin"):
+        assert tight["results"][k]["output"] == roomy["results"][k]["output"]
+    text = subprocess.run([sys.executable, "-m", "sprout_lm_amd", "demo"], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert text.returncode == 0 and "graph replay, bucket" in text.stdout and "what came out:" in text.stdout
 
 
 def test_first_tokens_and_long_decoding(folders):

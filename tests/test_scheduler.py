@@ -184,17 +184,17 @@ def test_invalid_inputs_and_requests_that_cannot_fit():
     with pytest.raises(Exception, match="positive integer"):
         make(max_batch_tokens=0)
     engine = make(block_size=2, num_blocks=1, max_sequences=1)
-    for bad, pattern in (([], "valid token"), ([-1], "valid token"), ([50], "valid token")):
+    for bad, pattern in (([], "brings no prompt"), ([-1], r"prompt\[0\] = -1 is no token id"), ([3, 50], r"prompt\[1\] = 50 is no token id")):
         with pytest.raises(ValueError, match=pattern):
             engine.add("x", bad, 1)
     with pytest.raises(ValueError, match="positive integer"):
         engine.add("x", [1], 0)
-    with pytest.raises(ValueError, match="cannot fit"):
+    with pytest.raises(ValueError, match="more than the whole pool holds"):
         engine.add("x", [1, 2], 2)
-    with pytest.raises(ValueError, match="context limit"):
+    with pytest.raises(ValueError, match="the model has 64"):
         make(num_blocks=64).add("x", [1], 65)
     engine.add("x", [1, 2], 1)
-    with pytest.raises(ValueError, match="unique"):
+    with pytest.raises(ValueError, match="id of its own"):
         engine.add("x", [1], 1)
     drain(engine)
 
