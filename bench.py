@@ -6,8 +6,10 @@
 Default: Qwen2.5-0.5B layer sizes with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
-Beside the contract's fields the line holds the prefill of 2,048 tokens, the roofline of the decode
-step, decoding at batch 1 and 64, `step_ms` (median, 95th percentile and maximum of the timed steps as the
+Beside the contract's fields the line holds the prefill of 2,048 tokens (the median of its repeats), the
+roofline of the decode step, `points`: decoding at batch 1 and 64, and the same decode step and prefill at
+Qwen2.5-7B sizes with all 28 layers, each with its fraction of the published peak (`7b_...`), `measured`: what
+this GPU gave a kernel that only reads and one that only multiplies, just before the run, `step_ms` (median, 95th percentile and maximum of the timed steps as the
 host sees them, and `host`: the part of a step that the host spends planning and launching, which the
 look-ahead hides behind the GPU's work), `prefill_in_portions` (the same prompt prefilled 256 and 512 tokens a step), `mixed` (the batch decoding while another prompt is prefilled 256
 tokens a step) and, with --pressure SHARE, a run in a pool too small for its requests (preemptions,
@@ -172,7 +174,7 @@ def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
     if chunk:
         engine = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk))
     rng = random.Random(1)
-    best = None
+    times = []
     for r in range(repeats + 1):
         prompt = [rng.randrange(cfg.vocab_size) for _ in range(tokens)]
         engine.add(f"p{r}", prompt, 1, ignore_eos=True)
@@ -183,9 +185,34 @@ def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
         engine.forget(f"p{r}")
-        if r > 0:
-            best = elapsed if best is None else min(best, elapsed)
-    return best
+        if r > 0:      # the first prompt warms up
+            times.append(elapsed)
+    return sorted(times)[len(times) // 2]      # the median, as for the decode steps
+
+
+def second_model_points(preset, dtype, element, batch, context, prefill_tokens, steps, dtype_name) -> dict:
+    """Decode tokens a second and prefill tokens a second of another size of the model, every layer of it, with
+    their fractions of the published peaks: flat numbers for `points`, named by the size."""
+    import gc
+    import torch
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.registry import config_from_dict
+    gc.collect()
+    torch.cuda.empty_cache()
+    cfg = config_from_dict(dict(PRESETS[preset]))
+    tag = preset.split("-")[-1]
+    engine = make_engine(cfg, dtype, batch, context, prefill_tokens)
+    parts = engine.model.parts
+    step_s, _ = measure_decode(engine, cfg, batch, context, steps, 3)
+    prefill_s = measure_prefill(engine, cfg, prefill_tokens, repeats=3)
+    engine.close()
+    read = decode_step_bytes(parts, batch, context, element)
+    return {f"{tag}_layers": cfg.num_hidden_layers,
+            f"{tag}_decode_b{batch}": round(batch / step_s, 1), f"{tag}_decode_b{batch}_ms": round(step_s * 1000, 4),
+            f"{tag}_decode_b{batch}_hbm_frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 5),
+            f"{tag}_prefill_{prefill_tokens}": round(prefill_tokens / prefill_s, 1),
+            f"{tag}_prefill_{prefill_tokens}_ms": round(prefill_s * 1000, 3),
+            f"{tag}_prefill_{prefill_tokens}_frac": round(prefill_flops(parts, prefill_tokens) / prefill_s / MFMA_PEAK[dtype_name], 5)}
 
 
 def main() -> int:
@@ -202,6 +229,8 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--mixed-chunk", type=int, default=256,
                         help="also time the batch decoding beside a prompt prefilled this many tokens a step (0: skip)")
+    parser.add_argument("--second-preset", default="qwen2.5-7b",
+                        help="sizes of the second model whose decode step and prefill go into `points` ('' or 'none': skip)")
     parser.add_argument("--pressure", type=float, default=0.0, metavar="SHARE",
                         help="also run the batch from 512-token prompts in a pool of this share of the pages it needs")
     args = parser.parse_args()
@@ -218,6 +247,9 @@ def main() -> int:
     cfg = config_from_dict(raw)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     element = 2 if args.dtype == "bf16" else 4
+
+    from sprout_lm_amd import ops
+    measured = ops.probe_machine()
 
     biggest = max(args.batch, 1 if args.no_points else 64)
     engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
@@ -239,9 +271,12 @@ def main() -> int:
     portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 2, c), 1)
                 for c in (256, 512) if c < args.prefill_tokens and not args.no_points}
     engine.close()
+    del engine
+    if not args.no_points and args.second_preset not in ("", "none", args.preset):
+        points.update(second_model_points(args.second_preset, dtype, element, args.batch, args.context, args.prefill_tokens,
+                                          min(args.steps, 24), args.dtype))
     pressure = None
     if args.pressure:
-        del engine
         pressure = measure_pressure(cfg, dtype, args.batch, 512, 256, args.pressure)
 
     read = decode_step_bytes(parts, args.batch, args.context, element)
@@ -263,9 +298,11 @@ def main() -> int:
         "prefill": {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens,
                     "ms": round(prefill_s * 1000, 3), "frac": round(flops / prefill_s / MFMA_PEAK[args.dtype], 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 5)},
-        "points": points, "step_ms": spread,
+                     "frac": round(achieved / HBM_PEAK_GBS, 5),
+                     "frac_of_measured": round(achieved / measured["hbm_read_gbs"], 5)},
+        "points": points, "measured": measured, "step_ms": spread,
     }
+    line["prefill"]["frac_of_measured"] = round(flops / prefill_s / (measured["mfma_bf16_tflops"] * 1e12), 5) if args.dtype == "bf16" else None
     if portions:
         line["prefill_in_portions"] = portions
     if mixed:

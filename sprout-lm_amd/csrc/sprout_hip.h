@@ -124,4 +124,10 @@ int sp_sample_workspace_floats(int R, int V);
 int sp_sample_static(void* stream, const float* logits, const float* temperature, const int64_t* seed,
                      const int32_t* counter, int32_t* out, int R, int V);
 int sp_sample_static_max_floats();
+
+// Probes for the benchmark's report, not used by the engine: a kernel that only reads `bytes` of `data` (16-byte
+// loads from `blocks` blocks of 256 threads), and one that only multiplies on the matrix cores (`blocks` blocks of four waves,
+// `iterations` x 4 independent 32x32x16 bfloat16 products a wave; *flops receives the operations of one launch).
+int sp_probe_read(void* stream, const void* data, int64_t bytes, int blocks, float* sink);
+int sp_probe_mfma(void* stream, int blocks, int iterations, float* sink, double* flops);
 }

@@ -441,3 +441,28 @@ def sample(logits: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, tem
             raise KernelError("sample: temperature must be float32 and seed int64, one per row")
     check(library().sp_sample(_stream(), logits.data_ptr(), _ptr(temperature), _ptr(seed), _ptr(counter), out.data_ptr(),
                               workspace.data_ptr(), R, V))
+
+
+def probe_machine(device=None, megabytes: int = 4096, repeats: int = 5) -> dict:
+    """What this GPU gives a kernel that only reads memory (GB/s) and one that only multiplies bfloat16 on the
+    matrix cores (TFLOP/s): the best of a few runs of the library's two probe kernels, for reports that set a
+    measured rate beside the published peak."""
+    import ctypes
+    lib = library()
+    device = device or torch.device("cuda", torch.cuda.current_device())
+    data = torch.zeros(megabytes << 20, dtype=torch.uint8, device=device)
+    sink = torch.zeros(4, dtype=torch.float32, device=device)
+    flops = ctypes.c_double()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_read = best_mfma = float("inf")
+    for _ in range(repeats + 1):       # the first run warms up
+        for blocks in (1024, 2048, 4096, 8192):     # how many blocks read fastest differs a little from box to box
+            start.record()
+            check(lib.sp_probe_read(_stream(), data.data_ptr(), data.numel(), blocks, sink.data_ptr()))
+            stop.record(); stop.synchronize()
+            best_read = min(best_read, start.elapsed_time(stop))
+        start.record()
+        check(lib.sp_probe_mfma(_stream(), 256 * 8, 20000, sink.data_ptr(), ctypes.byref(flops)))
+        stop.record(); stop.synchronize()
+        best_mfma = min(best_mfma, start.elapsed_time(stop))
+    return {"hbm_read_gbs": round(data.numel() / best_read / 1e6, 1), "mfma_bf16_tflops": round(flops.value / best_mfma / 1e9, 1)}

@@ -43,6 +43,8 @@ def _declare(lib):
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
         "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],
+        "sp_probe_mfma": [c_void, c_int, c_int, c_void, ctypes.POINTER(ctypes.c_double)],
     }
     lib.sp_attention_workspace_floats.argtypes = [c_int] * 10
     lib.sp_attention_workspace_floats.restype = c_i64
