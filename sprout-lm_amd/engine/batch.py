@@ -112,13 +112,34 @@ class DescriptorStager:
         return [self._dev[i][off:off + n].view(a.shape) for a, off, n in zip(arrays, offsets, sizes)]
 
 
-def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, workspace: Workspace, act_dtype,
-                  attention_kind: int = 0) -> StepContext:
-    """Lay the entries out flat and stage every array the kernels need.
+@dataclass
+class StepArrays:
+    """A step's integer arrays on the host, in the order in which they are staged, and what the step's kernels
+    need to know of them.  One builder serves the eager step and the recorded ones."""
+
+    names: list            # one name per array, in staging order
+    arrays: list           # numpy int32 arrays
+    lists: dict            # attention work lists by name (also part of `arrays`)
+    n_tokens: int
+    n_seqs: int
+    n_logits: int
+    max_q_len: int
+    max_decode_ctx: int
+    max_ctx: int
+    mean_walk: int
+    host: dict
+
+    def named(self, name: str):
+        return self.arrays[self.names.index(name)]
+
+
+def step_arrays(entries: list[StepEntry], cache, table_width: int | None = None) -> StepArrays:
+    """Lay the entries out flat: token ids, positions, per-sequence start / length / context, the places of
+    wanted logits, state slots, the attention work lists, and per cache group the block tables (`table_width`
+    entries a row, by default as many as the longest table) and the cache slot of every token.
 
     Each entry's sequence must already hold pages for its new tokens (CacheManager.reserve).
     """
-    ctx = StepContext(workspace, act_dtype, attention_kind)
     bs = cache.block_size
     q_lens = [len(e.tokens) for e in entries]
     starts = np.zeros(len(entries), dtype=np.int32)
@@ -135,37 +156,54 @@ def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, wor
     logit_rows = np.asarray(rows, dtype=np.int32)
     state_slots = np.asarray([e.seq.state_slot for e in entries], dtype=np.int32)
 
+    names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots", "seq_of_token"]
     arrays = [token_ids, positions, starts, q_len, ctx_len, logit_rows, state_slots, seq_of_token]
     lists = ops.attention_lists(q_lens)
-    list_names = sorted(lists)
-    arrays += [lists[name] for name in list_names]
+    for name in sorted(lists):
+        names.append(name)
+        arrays.append(lists[name])
     for gi, group in enumerate(cache.groups):
-        width = max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
+        width = table_width or max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
         tables = np.full((len(entries), width), -1, dtype=np.int32)
         slots = np.full(T, -1, dtype=np.int32)
         for s, e in enumerate(entries):
-            blocks = e.seq.blocks[gi]
+            blocks = e.seq.blocks[gi][:width]
             tables[s, :len(blocks)] = blocks
             if q_lens[s]:
                 pos = np.arange(first_pos[s], ctx_len[s])
-                pages = np.asarray(blocks, dtype=np.int64)[pos // bs]
+                pages = np.asarray(e.seq.blocks[gi], dtype=np.int64)[pos // bs]
                 slots[starts[s]:starts[s] + q_lens[s]] = pages * bs + pos % bs
+        names += [f"tables{gi}", f"slots{gi}"]
         arrays += [tables, slots]
-
-    dev = stager.upload(arrays)
-    (ctx.token_ids, ctx.positions, ctx.q_start, ctx.q_len, ctx.ctx_len, ctx.logit_rows, ctx.state_slots,
-     ctx.seq_of_token) = dev[:8]
-    on_device = {name: (d, len(lists[name])) for name, d in zip(list_names, dev[8:8 + len(list_names)])}
     decode_ctx = [int(c) for c, q in zip(ctx_len, q_lens) if q == 1]
-    ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, len(entries), on_device,
-                                       max(decode_ctx, default=0), max((int(c) for c in ctx_len), default=0),
-                                       ops.mean_tile_walk(q_lens, ctx_len))
-    rest = dev[8 + len(list_names):]
-    ctx.group_tables = rest[0::2]
-    ctx.group_slots = rest[1::2]
-    ctx.n_tokens, ctx.n_seqs, ctx.n_logits = T, len(entries), len(rows)
-    ctx.max_q_len = max(q_lens, default=0)
-    ctx.host = {"q_start": starts, "q_len": q_len, "ctx_len": ctx_len, "positions": positions,
-                "token_ids": token_ids, "state_slots": state_slots, "seq_of_token": seq_of_token,
-                "first_pos": first_pos}
+    host = {"q_start": starts, "q_len": q_len, "ctx_len": ctx_len, "positions": positions, "token_ids": token_ids,
+            "state_slots": state_slots, "seq_of_token": seq_of_token, "first_pos": first_pos}
+    return StepArrays(names, arrays, lists, T, len(entries), len(rows), max(q_lens, default=0), max(decode_ctx, default=0),
+                      max((int(c) for c in ctx_len), default=0), ops.mean_tile_walk(q_lens, ctx_len), host)
+
+
+def context_from(step: StepArrays, dev: list, n_groups: int, workspace: Workspace, act_dtype, attention_kind: int = 0,
+                 max_decode_ctx: int | None = None, max_ctx: int | None = None) -> StepContext:
+    """The step's context over the device copies `dev` of `step.arrays` (same order)."""
+    ctx = StepContext(workspace, act_dtype, attention_kind)
+    by_name = dict(zip(step.names, dev))
+    ctx.token_ids, ctx.positions, ctx.q_start = by_name["token_ids"], by_name["positions"], by_name["q_start"]
+    ctx.q_len, ctx.ctx_len, ctx.logit_rows = by_name["q_len"], by_name["ctx_len"], by_name["logit_rows"]
+    ctx.state_slots, ctx.seq_of_token = by_name["state_slots"], by_name["seq_of_token"]
+    on_device = {name: (by_name[name], len(step.lists[name])) for name in step.lists}
+    ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, step.n_seqs, on_device,
+                                       step.max_decode_ctx if max_decode_ctx is None else max_decode_ctx,
+                                       step.max_ctx if max_ctx is None else max_ctx, step.mean_walk)
+    ctx.group_tables = [by_name[f"tables{g}"] for g in range(n_groups)]
+    ctx.group_slots = [by_name[f"slots{g}"] for g in range(n_groups)]
+    ctx.n_tokens, ctx.n_seqs, ctx.n_logits = step.n_tokens, step.n_seqs, step.n_logits
+    ctx.max_q_len = step.max_q_len
+    ctx.host = step.host
     return ctx
+
+
+def build_context(entries: list[StepEntry], cache, stager: DescriptorStager, workspace: Workspace, act_dtype,
+                  attention_kind: int = 0) -> StepContext:
+    """Lay the entries out flat and stage every array the kernels need, in one copy to the device."""
+    step = step_arrays(entries, cache)
+    return context_from(step, stager.upload(step.arrays), len(cache.groups), workspace, act_dtype, attention_kind)

@@ -1,4 +1,4 @@
-"""Decode steps as HIP graphs.
+"""Steps as HIP graphs.
 
 A step in which every request brings exactly one token launches a long chain of small kernels; the
 host cannot issue them as fast as the GPU runs them.  Such steps are recorded once per batch shape
@@ -9,6 +9,13 @@ descriptor upload, one graph launch and one small download make a step.
 Shapes are bucketed: the number of sequences to a power of two (missing ones are filled with
 one-token dummies that write no cache), the block-table width and the key splits of attention to a
 power-of-two context.  Nothing in a graph depends on the values of a step.
+
+Steps that bring portions of prompts are recorded as well once their shape comes a second time (the same
+numbers of tokens and of wanted places request by request, the longest context in the same bucket): a long
+prompt fed in equal portions, or a batch that decodes beside such a portion, repeats its shape step after step,
+and at small model sizes the host needs as long to issue such a step's two hundred launches as the GPU to run
+them.  These graphs hold no padding and no sampling; their descriptors come from the same builder as an eager
+step's (`batch.step_arrays`).
 """
 from __future__ import annotations
 
@@ -19,7 +26,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from .batch import CacheSlotView, StepContext, Workspace
+from .batch import CacheSlotView, StepContext, Workspace, context_from, step_arrays
 
 
 def _bucket(n: int, floor: int = 1) -> int:
@@ -168,34 +175,128 @@ class _DecodeGraph:
         ops.sample(self.logits, self.sampled, self.sample_ws, self.temperature, self.seed, self.counter)
 
     def _record(self) -> None:
-        # once eagerly, so that every workspace buffer exists before anything is recorded
-        self._body()
-        torch.cuda.current_stream().synchronize()
-        self.ctx.workspace.frozen = True
-        graph = torch.cuda.CUDAGraph()
-        # No garbage collection while the stream is capturing: a dead cycle that holds GPU objects (an older
-        # engine's graphs, events, pinned buffers) would be destroyed in the middle of the capture, and what
-        # their destructors call is not allowed then (the process aborts).  Collect first, then hold it off.
-        gc.collect()
-        collecting = gc.isenabled()
-        gc.disable()
-        try:
-            with torch.cuda.graph(graph):
-                self._body()
-        finally:
-            if collecting:
-                gc.enable()
-            self.ctx.workspace.frozen = False
-        self.graph = graph
-        # the eager run above already produced this step's results; replaying would only repeat it
+        _record(self)     # its eager run already produced this step's results
+
+
+class _PortionGraph:
+    """Static buffers and the recorded graph of one step shape with portions of prompts in it."""
+
+    def __init__(self, runner, first, ctx_bucket: int):
+        self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
+        cache = runner.cache
+        self.table_width = -(-ctx_bucket // cache.block_size)
+        self.sizes = [a.size for a in first.arrays]
+        self.offsets, total = [], 0
+        for n in self.sizes:
+            self.offsets.append(total)
+            total += (n + 3) // 4 * 4          # every array 16-byte aligned
+        self.host = torch.zeros(max(total, 4), dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(max(total, 4), dtype=torch.int32, device=runner.device)
+        views = [self.dev[o:o + n].view(a.shape) for o, n, a in zip(self.offsets, self.sizes, first.arrays)]
+        # buffers of its own: a graph holds their addresses.  The longest context is known to the kernels as its
+        # bucket only (how a long walk is shared out follows it), and the step has no values on the host.
+        self.ctx = context_from(first, views, len(cache.groups), Workspace(runner.device), runner.dtype,
+                                runner.attention_kind, max_decode_ctx=ctx_bucket, max_ctx=ctx_bucket)
+        self.ctx.host = {}
+        self.copied = None
+        self.graph = None
+        self.logits = None
+
+    def fill(self, step) -> None:
+        if [a.size for a in step.arrays] != self.sizes:
+            raise RuntimeError("A recorded step was given arrays of another shape than it was recorded with.")
+        if self.copied is not None:
+            self.copied.synchronize()      # the last launch's upload may still be reading the staging buffer
+        for a, o, n in zip(step.arrays, self.offsets, self.sizes):
+            self.host_np[o:o + n] = a.reshape(-1)
+
+    def launch(self) -> None:
+        self.dev.copy_(self.host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+        if self.graph is None:
+            _record(self)
+        else:
+            self.graph.replay()
+
+    def _body(self):
+        self.ctx.shared.clear()            # see _DecodeGraph._body
+        self.logits = self.runner.forward(self.ctx)
+
+
+def _record(state) -> None:
+    """Run `state._body` once eagerly (every workspace buffer then exists, and this step's results are there),
+    then record it.
+
+    No garbage collection while the stream is capturing: a dead cycle that holds GPU objects (an older engine's
+    graphs, events, pinned buffers) would be destroyed in the middle of the capture, and what their destructors
+    call is not allowed then (the process aborts).  Collect first, then hold it off."""
+    state._body()
+    torch.cuda.current_stream().synchronize()
+    state.ctx.workspace.frozen = True
+    graph = torch.cuda.CUDAGraph()
+    gc.collect()
+    collecting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            state._body()
+    finally:
+        if collecting:
+            gc.enable()
+        state.ctx.workspace.frozen = False
+    state.graph = graph
 
 
 class DecodeGraphs:
     def __init__(self, runner, max_graphs: int = 32):
         self.runner = weakref.proxy(runner)
-        self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self.graphs: dict[tuple, object] = {}     # decode steps: (sequences, context bucket); others: (shape, bucket)
         self.max_graphs = max_graphs
         self.replays = 0
+        self.portion_replays = 0
+        self._sightings: dict[tuple, int] = {}
+
+    def _context_bucket(self, longest: int) -> int:
+        return min(_bucket(longest, 256), -(-self.runner.max_positions // 256) * 256)
+
+    def _make_room(self) -> None:
+        if len(self.graphs) >= self.max_graphs:
+            # the least recently used graph goes; a step launched ahead may still be running from it
+            torch.cuda.current_stream().synchronize()
+            self.graphs.pop(next(iter(self.graphs)))
+
+    def portion_step(self, entries, record_at: int = 2):
+        """Run a step that is not one token a request from a recorded graph, if its shape has been seen
+        `record_at` times (the step that reaches the count is the one recorded).  Returns the float32 logits
+        at the wanted places (the graph's own buffer: valid until the same shape runs again), or None if the step
+        is not taken this way: then nothing was launched.  The sequences' lengths are advanced."""
+        runner = self.runner
+        if not runner.parts.graph_safe_portions or not entries:
+            return None
+        bucket = self._context_bucket(max(e.seq.length + len(e.tokens) for e in entries))
+        key = (tuple((len(e.tokens), len(e.want)) for e in entries), bucket)
+        state = self.graphs.pop(key, None)
+        if state is None:
+            seen = self._sightings.get(key, 0) + 1
+            if len(self._sightings) > 4096:
+                self._sightings.clear()
+            self._sightings[key] = seen
+            if seen < record_at:
+                return None
+        step = step_arrays(entries, runner.cache, table_width=-(-bucket // runner.cache.block_size))
+        if state is None:
+            self._make_room()
+            state = _PortionGraph(runner, step, bucket)
+        self.graphs[key] = state
+        state.fill(step)
+        state.launch()
+        self.portion_replays += 1
+        for e in entries:
+            runner.cache.commit(e.seq, e.seq.length + len(e.tokens))
+        return state.logits
 
     def usable(self, entries) -> bool:
         runner = self.runner
@@ -215,14 +316,11 @@ class DecodeGraphs:
         n = len(entries)
         S = _bucket(n)
         longest = max(e.seq.length for e in entries) + 1
-        ctx_bucket = min(_bucket(longest, 256), -(-runner.max_positions // 256) * 256)
+        ctx_bucket = self._context_bucket(longest)
         key = (S, ctx_bucket)
         state = self.graphs.pop(key, None)
         if state is None:
-            if len(self.graphs) >= self.max_graphs:
-                # the least recently used graph goes; a step launched ahead may still be running from it
-                torch.cuda.current_stream().synchronize()
-                self.graphs.pop(next(iter(self.graphs)))
+            self._make_room()
             state = _DecodeGraph(runner, S, ctx_bucket)
         self.graphs[key] = state          # most recently used last
         previous, sources = (None, None) if feed is None else (feed[0].sampled, feed[1])

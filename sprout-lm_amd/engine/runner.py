@@ -64,6 +64,7 @@ class ModelRunner:
         self.attention_kind = 1 if dtype == torch.float32 else 0
         self.vocab_size, self.hidden_size, self.max_positions = plan.vocab_size, plan.hidden_size, plan.max_positions
         self.use_graphs = use_graphs
+        self.record_portions = True      # steps with portions of prompts are recorded too, once their shape recurs
         self.load_notes: list[str] = []    # what the loader saw and left alone (tensors nobody asked for)
         self._graphs = None
         self._sampler = None
@@ -188,7 +189,8 @@ class ModelRunner:
     def step_and_sample(self, entries: list[StepEntry], params, counters) -> list[int]:
         """One step plus sampling at every wanted place; returns the sampled token ids on the host.
 
-        Steps in which every request brings one token are replayed from a recorded HIP graph.
+        Steps in which every request brings one token are replayed from a recorded HIP graph; so are other
+        steps whose shape comes again and again (`step_recorded`).
         """
         from ..sampling.sampler import Sampler
         pending = self.launch_decode(entries, params, counters)
@@ -196,7 +198,24 @@ class ModelRunner:
             return self.finish_decode(pending)
         if self._sampler is None:
             self._sampler = Sampler(self.device, self.vocab_size)
-        return self._sampler.sample(self.step(entries), params, counters)
+        logits = self.step_recorded(entries)
+        if logits is None:
+            logits = self.step(entries)
+        return self._sampler.sample(logits, params, counters)
+
+    def step_recorded(self, entries: list[StepEntry], record_at: int = 2):
+        """`step` from a recorded graph of the step's shape, where there is one or the shape has now come
+        `record_at` times; None otherwise (nothing has been run then).  The logits lie in the graph's own buffer
+        and are overwritten when the same shape runs again."""
+        if not self.use_graphs or not self.record_portions:
+            return None
+        if self._graphs is None:
+            from .graphs import DecodeGraphs
+            self._graphs = DecodeGraphs(self)
+        if not self.parts.graph_safe_portions:
+            return None
+        self.validate(entries)
+        return self._graphs.portion_step(entries, record_at)
 
     def launch_decode(self, entries: list[StepEntry], params, counters, feed=None):
         """Start a step in which every request brings one token, without waiting for its result.

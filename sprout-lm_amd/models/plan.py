@@ -106,6 +106,8 @@ class ModelParts:
         every = [part for _, part in self._named] + list(self.blocks)
         every += [getattr(b.mixer, "position", None) for b in self.blocks if hasattr(b, "mixer")]
         self.graph_safe = all(getattr(part, "graph_safe", False) for part in every if part is not None)
+        self.graph_safe_portions = self.graph_safe and all(getattr(part, "graph_safe_portions", False)
+                                                           for part in every if part is not None)
 
     # ------------------------------------------------------------------ what a step costs, summed over the parts
     def _calls(self):

@@ -28,6 +28,8 @@ class Attention(Mixer):
 
     graph_safe = True
 
+    graph_safe_portions = True
+
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
                  out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None):
         try:      # sizes no kernel takes are refused when the part is built, not at the first step

@@ -49,6 +49,8 @@ class Part:
     # host-side decisions from the step's values, no allocation): such a part may be recorded into
     # a HIP graph and replayed with new values in the same buffers.
     graph_safe = False
+    # True if that holds for every step, also one with portions of prompts in it (then `ctx.host` is empty).
+    graph_safe_portions = False
 
     def tensors(self) -> dict[str, TensorSpec]:
         """Local tensor name -> what is expected of it."""

@@ -10,6 +10,8 @@ class PreNormBlock(Block):
 
     graph_safe = True
 
+    graph_safe_portions = True
+
     def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 

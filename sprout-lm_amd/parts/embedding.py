@@ -9,6 +9,7 @@ from .base import Part, register_part
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
     graph_safe = True
+    graph_safe_portions = True
 
     def __init__(self, vocab: int, hidden: int):
         self.vocab, self.hidden = vocab, hidden
@@ -28,6 +29,8 @@ class LinearHead(Part):
     """logits = W . x in float32.  With `tied`, W is the embedding table and the head has no tensor."""
 
     graph_safe = True
+
+    graph_safe_portions = True
 
     def __init__(self, vocab: int, hidden: int, tied: bool):
         self.vocab, self.hidden, self.tied = vocab, hidden, tied

@@ -15,6 +15,8 @@ class GatedMLP(FeedForward):
 
     graph_safe = True
 
+    graph_safe_portions = True
+
     def __init__(self, hidden: int, inner: int, activation: str = "silu"):
         if activation not in ops.GATE_ACTIVATIONS:     # refused when the part is built, not at the first step
             raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; "

@@ -12,6 +12,8 @@ class RMSNorm(Norm):
 
     graph_safe = True
 
+    graph_safe_portions = True
+
     def __init__(self, size: int, eps: float):
         self.size, self.eps = size, eps
 

@@ -18,6 +18,8 @@ class NeoxRotary(PositionEncoding):
     """
 
     graph_safe = True
+
+    graph_safe_portions = True
     pairing = "halves"      # which dimensions turn together, as the kernels name it (ops.ROTARY_PAIRINGS)
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
@@ -57,6 +59,8 @@ class NoPosition(PositionEncoding):
     pairing = "halves"      # nothing turns; the kernels are asked for the pairing they have
 
     graph_safe = True
+
+    graph_safe_portions = True
 
     def __init__(self, head_dim: int = 0):
         self.head_dim = head_dim

@@ -1,4 +1,4 @@
-"""Decode steps replayed from recorded HIP graphs, compared by their logits with the plain implementation.
+"""Steps replayed from recorded HIP graphs, compared by their logits with the plain implementation.
 
 Generation runs every step of single tokens through `ModelRunner.launch_decode`; the other logits tests step
 eagerly.  Here the recorded path itself is held to the plain side: its own descriptor builder, padded rows,
@@ -115,3 +115,97 @@ def test_recorded_steps_at_real_layer_sizes_match_plain(tmp_path):
         s.release()
     assert runner.cache.free_pages() == [64]
     print(f"recorded steps at real layer sizes: worst {worst:.2f} of the bound")
+
+
+def fed_step(runner, seqs, tokens, fed, takes, folder, dtype, label, recorded=True):
+    """One step in which request r brings its next `takes[r]` tokens and wants the logits of the last of them,
+    through `step_recorded` (eagerly where that declines); every wanted row against the plain side.
+    Returns (whether the step ran from a graph, worst error as a fraction of the bound)."""
+    from sprout_lm_amd.engine import StepEntry
+    entries = []
+    for r, n in takes.items():
+        assert runner.cache.reserve(seqs[r], fed[r] + n)
+        entries.append(StepEntry(seqs[r], tokens[r][fed[r]:fed[r] + n], [n - 1]))
+    logits = runner.step_recorded(entries) if recorded else None
+    from_graph = logits is not None
+    if logits is None:
+        logits = runner.step(entries)
+    got = logits.cpu().numpy()
+    worst = 0.0
+    for i, (r, n) in enumerate(takes.items()):
+        fed[r] += n
+        want = H.plain_logits(folder, dtype, tokens[r][:fed[r]], rows=[fed[r] - 1])[0]
+        err = float(np.abs(got[i] - want).max()) / H.tolerance(dtype, want)
+        worst = max(worst, err)
+        assert err <= 1.0, f"{label}: request {r} up to position {fed[r] - 1}: {err:.2f} of the bound"
+    return from_graph, worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_recorded_portions_match_plain(tmp_path, name, dtype):
+    """Steps with portions of prompts are recorded when their shape comes a second time.  A prompt in equal
+    portions (the last one shorter: another shape), then two requests that decode beside the portions of a
+    third, which computes in the pages the first gave back; every step's wanted logits against the plain side,
+    replay after replay, with eager steps of other shapes between them."""
+    from sprout_lm_amd.engine import ModelRunner
+    folder = H.make_model_folder(str(tmp_path), name)
+    page = H.PAGE_SIZE[name]
+    vocab = H.CONFIGS[name]["vocab_size"]
+    tokens = {r: H.random_tokens(vocab, n, 500 + i) for i, (r, n) in enumerate(dict(a=127, b=40, c=47, d=118).items())}
+    runner = ModelRunner.from_folder(folder, dtype, block_size=page, num_blocks=-(-127 // page) + 2 * -(-64 // page),
+                                     max_sequences=4)
+    seqs = {r: runner.cache.create() for r in "abc"}
+    fed = dict.fromkeys("abcd", 0)
+    ran, worst = [], 0.0
+    for n in [24] * 5 + [7]:
+        g, w = fed_step(runner, seqs, tokens, fed, {"a": n}, folder, dtype, "one prompt in portions")
+        ran.append(g)
+        worst = max(worst, w)
+    assert ran == [False, True, True, True, True, False]         # recorded at the second sighting
+    held = set(seqs["a"].blocks[0])
+    seqs.pop("a").release()
+    for r, n in (("b", 30), ("c", 41)):                           # two prompts, eagerly
+        _, w = fed_step(runner, seqs, tokens, fed, {r: n}, folder, dtype, "whole prompt", recorded=False)
+        worst = max(worst, w)
+    seqs["d"] = runner.cache.create()
+    ran = []
+    for i in range(6):
+        g, w = fed_step(runner, seqs, tokens, fed, {"b": 1, "d": 18, "c": 1}, folder, dtype, "decode beside a portion")
+        ran.append(g)
+        worst = max(worst, w)
+        if i == 2:      # an eager step of another shape between replays, through the shared step context
+            _, w = fed_step(runner, seqs, tokens, fed, {"d": 2}, folder, dtype, "two tokens", recorded=False)
+            worst = max(worst, w)
+    assert ran == [False] + [True] * 5
+    assert held & set(seqs["d"].blocks[0]), "the late request got none of the pages that the first gave back"
+    assert runner._graphs.portion_replays == 9
+    for s in seqs.values():
+        s.release()
+    assert runner.cache.free_pages() == [runner.cache.num_blocks]
+    print(f"recorded portions {name} {dtype}: worst {worst:.2f} of the bound")
+
+
+def test_recorded_portions_at_real_layer_sizes_cross_a_context_bucket(tmp_path):
+    """Two layers with the sizes of Qwen2.5-0.5B, a prompt of 512 tokens in portions of 64: the tiled products
+    and the attention over tiles of queries, recorded.  The longest context a graph was recorded for is part of
+    its key (256 keys, then 512): the step that first passes 256 keys runs eagerly and the next one is recorded
+    anew."""
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.engine import ModelRunner
+    from sprout_lm_amd.weights import write_model_folder
+    raw = dict(PRESETS["qwen2.5-0.5b"], num_hidden_layers=2)
+    folder = str(tmp_path / "half_b")
+    write_model_folder(folder, S.config_from_dict(raw), seed=9, dtype=torch.bfloat16, std=0.02)
+    tokens = {"a": H.random_tokens(raw["vocab_size"], 512, 77)}
+    runner = ModelRunner.from_folder(folder, "bfloat16", block_size=16, num_blocks=40, max_sequences=2)
+    seqs, fed = {"a": runner.cache.create()}, {"a": 0}
+    ran, worst = [], 0.0
+    for _ in range(8):
+        g, w = fed_step(runner, seqs, tokens, fed, {"a": 64}, folder, "bfloat16", "portions of 64")
+        ran.append(g)
+        worst = max(worst, w)
+    assert ran == [False, True, True, True, False, True, True, True]
+    assert set(runner._graphs.graphs) == {(((64, 1),), 256), (((64, 1),), 512)}
+    print(f"recorded portions at real layer sizes: worst {worst:.2f} of the bound")
