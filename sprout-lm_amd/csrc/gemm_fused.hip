@@ -167,6 +167,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   float* squares = reinterpret_cast<float*>(lds + 4 * NT * TN * 64);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for the whole wave: a scalar
   const int lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int t0 = blockIdx.z * (16 * TN);   // the block's first token: tiles of tokens lie along z
   const int k_begin = blockIdx.y * a.k_per_split;
   const int k_end = min(a.K, k_begin + a.k_per_split);
   const int steps = (k_end - k_begin + 63) / 64;
@@ -175,12 +176,12 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   const uint16_t* wrow[NT];
 #pragma unroll
   for (int i = 0; i < NT; ++i) wrow[i] = a.w + size_t(weight_row<EPI, NT>(a, blockIdx.x, i, lr)) * a.K + k_begin + 16 * lj;
-  const float* norm_row = NORM ? a.residual + size_t(min(lr, a.T - 1)) * a.K + k_begin + 16 * lj : nullptr;
+  const float* norm_row = NORM ? a.residual + size_t(min(t0 + lr, a.T - 1)) * a.K + k_begin + 16 * lj : nullptr;
   const char* norm_w0 = NORM ? reinterpret_cast<const char*>(a.norm_w) + size_t(k_begin + 16 * lj) * (a.norm_w_bf16 ? 2 : 4) : nullptr;
   const uint16_t* xrow[TN];
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn)   // rows past T repeat the last one: their sums are not used
-    xrow[tn] = NORM ? nullptr : a.x + size_t(min(tn * 16 + lr, a.T - 1)) * a.K + k_begin + 16 * lj;
+    xrow[tn] = NORM ? nullptr : a.x + size_t(min(t0 + tn * 16 + lr, a.T - 1)) * a.K + k_begin + 16 * lj;
 
   // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
   // of this wave together (steps s0, s0 + 4, ...).
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     if (rope_dim < a.rotary_dim / 2) frequency = a.inv_freq[rope_dim];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
-      const int t = min(tn * 16 + et, a.T - 1);
+      const int t = min(t0 + tn * 16 + et, a.T - 1);
       position_of[tn] = a.positions[t];
       slot_of[tn] = a.slot_mapping[t];
     }
@@ -332,7 +333,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
                               : 1.f;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
-    const int t = tn * 16 + et;
+    const int t = t0 + tn * 16 + et;
     if (EPI == kEpiSilu) {
       const int r = a.rows_per_block;
 #pragma unroll
@@ -415,10 +416,11 @@ static size_t fused_lds_bytes(int TN, bool norm, int NT = 2) {
 template <int TN, int EPI, bool NORM, int NT = 2>
 static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
   const size_t lds = fused_lds_bytes(TN, NORM, NT);     // at most 48 KB (four token tiles of three tiles)
+  const dim3 grid(blocks, splits, (a.T + 16 * TN - 1) / (16 * TN));   // z: the tokens in tiles of 16 TN
   if (a.K % 64 == 0 && a.k_per_split % 64 == 0)
-    gemm_fused_kernel<TN, EPI, NORM, NT, true><<<dim3(blocks, splits), 256, lds, s>>>(a);
+    gemm_fused_kernel<TN, EPI, NORM, NT, true><<<grid, 256, lds, s>>>(a);
   else
-    gemm_fused_kernel<TN, EPI, NORM, NT, false><<<dim3(blocks, splits), 256, lds, s>>>(a);
+    gemm_fused_kernel<TN, EPI, NORM, NT, false><<<grid, 256, lds, s>>>(a);
   return check_launch("sp_gemm_fused");
 }
 
@@ -427,15 +429,21 @@ static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int split
 // (28 heads of 128 at a width of 3,584, 64 tokens: 36 us against about 20).  Head sizes that 32 does not divide
 // have no other way.
 static bool rope_one_tile(int T, int hd) { return T <= 16 || hd % 32 != 0; }
+// With the norm prologue a block takes 16 tokens whatever their number (further tiles of tokens are further
+// blocks, each normalising its own rows): one gathered tile a block as long as all the blocks find a CU of
+// their own, two tiles (half the blocks) beyond that, where a CU would have to pull for two blocks.
+static bool rope_one_tile_normed(int T, int N, int hd) {
+  return hd % 32 != 0 || (N / 16) * ((T + 15) / 16) <= 256;
+}
 
 template <int EPI, bool NORM>
 static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
   if constexpr (EPI == kEpiSilu) {   // up to 16 tokens: a block may own up to 24 inner columns (three tiles)
     if (a.rows_per_block > 16) return launch_fused<1, EPI, NORM, 3>(s, a, blocks, splits);
   }
-  if constexpr (NORM) {   // one tile of up to 16 tokens (fused_shape_ok)
+  if constexpr (NORM) {   // tiles of 16 tokens, each a block of its own
     if constexpr (EPI == kEpiRope) {
-      if (rope_one_tile(a.T, a.hd)) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);
+      if (rope_one_tile_normed(a.T, a.N, a.hd)) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);
     }
     return launch_fused<1, EPI, true>(s, a, blocks, splits);
   } else {
@@ -458,13 +466,14 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
 // columns: 256 blocks of 19 instead of 304 of 16, of which 48 CUs held two.  More than 16 columns (three tiles)
 // only with up to 16 tokens.
 static int silu_rows_per_block(int T, int I, int K, bool norm) {
-  const int most = T <= 16 ? 24 : 16;
+  const int most = (T <= 16 || norm) ? 24 : 16;
+  const int token_tiles = norm ? (T + 15) / 16 : 1;
   int best_rows = 16;
   double best = 1e30;
   for (int r = 4; r <= most; ++r) {
     const int blocks = (I + r - 1) / r;
     const double bytes = 4.0 * r * K + (norm ? 4.0 * min(T, 16) * K + 2.0 * K : 2.0 * T * K);
-    const double cost = double((blocks + 255) / 256) * bytes;
+    const double cost = double((blocks * token_tiles + 255) / 256) * bytes;
     if (cost <= best) { best = cost; best_rows = r; }
   }
   return best_rows;
@@ -475,11 +484,10 @@ static int fused_norm(hipStream_t s, const FusedArgs& a, bool norm, int blocks, 
   return norm ? fused_tokens<EPI, true>(s, a, blocks, splits) : fused_tokens<EPI, false>(s, a, blocks, splits);
 }
 
-// Whether the fused kernels take this shape.  K in 16-byte rows, T <= 64; the norm prologue takes up to
-// 16 tokens (one tile).
+// Whether the fused kernels take this shape: K in 16-byte rows, T <= 64.
 static bool fused_shape_ok(int T, int K, bool norm) {
-  if (T < 1 || T > 64 || K % 8) return false;
-  return !(norm && T > 16);
+  (void)norm;
+  return T >= 1 && T <= 64 && K % 8 == 0;
 }
 
 }  // namespace sprout
@@ -509,13 +517,15 @@ extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rot
   return kind == kEpiStore || kind == kEpiAccumulate || kind == kEpiStoreF32;
 }
 
-// Whether the norm prologue is faster than a norm kernel of its own before the product.  Every block
-// normalises all the rows by itself and keeps them in LDS, which costs more the wider the rows are:
+// Whether the norm prologue is faster than a norm kernel of its own before the product.  Every block reads
+// its 16 tokens' rows of the float32 residual beside its weight rows, which costs more the wider the rows are:
 // measured at 8 tokens, QKV product with prologue against norm kernel + product: 7.0 against 7.9 us at a
-// width of 896, 11.6 against 9.4 at 1536, 22.2 against 16.2 at 3584; the gated product alike.
+// width of 896, 11.6 against 9.4 at 1536, 22.2 against 16.2 at 3584; the gated product alike.  With more than
+// 16 tokens every tile of tokens reads the weights again: that pays while all the blocks run at once (1,152 rows
+// x 896 at 64 tokens: 8.6 us against 8.7 + 2.4 for the norm), not beyond (9,728 x 896: 21.2 against 8.5 + 2.4).
 extern "C" int sp_fused_norm_pays(int T, int N, int K) {
-  (void)N;
-  return fused_shape_ok(T, K, true) && K <= 1024;
+  if (!fused_shape_ok(T, K, true) || K > 1024) return 0;
+  return T <= 16 || (N / 16) * ((T + 15) / 16) <= 512;
 }
 
 namespace sprout {
@@ -585,7 +595,8 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.page_shift = -1;
   if (page_size > 0 && (page_size & (page_size - 1)) == 0)
     for (a.page_shift = 0; (1 << a.page_shift) < page_size;) ++a.page_shift;
-  const int blocks = (nq + 2 * nkv) * (hd / (rope_one_tile(T, hd) ? 16 : 32));
+  const bool one_tile = residual ? rope_one_tile_normed(T, N, hd) : rope_one_tile(T, hd);
+  const int blocks = (nq + 2 * nkv) * (hd / (one_tile ? 16 : 32));
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
 

@@ -93,7 +93,7 @@ class Attention(Mixer):
         T = residual.shape[0]
         if not self.fuse_input_norm:
             return False
-        if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, cache, True):
+        if ctx.act_dtype != torch.bfloat16 or T > 64 or not isinstance(norm, RMSNorm) or not self._fused(T, cache, True):
             return False
         if not ops.fused_norm_pays(T, self.w_qkv.shape[0], self.hidden):
             return False

@@ -46,7 +46,7 @@ class GatedMLP(FeedForward):
         T = residual.shape[0]
         if not self.fuse_input_norm:
             return False
-        if ctx.act_dtype != torch.bfloat16 or T > 16 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
+        if ctx.act_dtype != torch.bfloat16 or T > 64 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
             return False
         if not ops.fused_norm_pays(T, 2 * self.inner, self.hidden):
             return False
