@@ -165,7 +165,7 @@ def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
             "steps": ticks, "seconds": round(elapsed, 3), "net_value": round(made / elapsed, 1)}
 
 
-def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
+def measure_prefill(engine, cfg, tokens, repeats=5, chunk=None):
     """Seconds from a prompt's arrival to its first token; `chunk`: the prompt goes in portions of that size."""
     import random
     from dataclasses import replace
@@ -175,7 +175,10 @@ def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
         engine = Engine(engine.model, replace(engine.options, prefill_chunk_size=chunk))
     rng = random.Random(1)
     times = []
-    for r in range(repeats + 1):
+    # Two prompts warm up: the engine records a step's shape as a graph when it comes a second time, as the
+    # portions of equal-sized prompts do in service; the timed prompts run as every later one would.
+    warm = 2
+    for r in range(repeats + warm):
         prompt = [rng.randrange(cfg.vocab_size) for _ in range(tokens)]
         engine.add(f"p{r}", prompt, 1, ignore_eos=True)
         torch.cuda.synchronize()
@@ -185,7 +188,7 @@ def measure_prefill(engine, cfg, tokens, repeats=3, chunk=None):
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
         engine.forget(f"p{r}")
-        if r > 0:      # the first prompt warms up
+        if r >= warm:
             times.append(elapsed)
     return sorted(times)[len(times) // 2]      # the median, as for the decode steps
 
@@ -268,7 +271,7 @@ def main() -> int:
     mixed_aligned = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2,
                                   multiple=args.mixed_chunk) if args.mixed_chunk and args.batch < args.mixed_chunk else None
     prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
-    portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 2, c), 1)
+    portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 3, c), 1)
                 for c in (256, 512) if c < args.prefill_tokens and not args.no_points}
     engine.close()
     del engine
