@@ -62,7 +62,9 @@ class SequenceCache:
 
 @dataclass
 class _PrefixEntry:
-    pages: list[int]
+    """One full page of a prefix, in every group: the page's id, or None where a windowed group has given its
+    page back (the entry then still links the chain, and serves requests whose window lies behind it)."""
+    pages: list
     last_used: int
 
 
@@ -94,10 +96,9 @@ class CacheManager:
                 g = len(groups) - 1
             groups[g].slots.append(slot)
             self.slot_location.append((kind, g, len(groups[g].slots) - 1))
-        # Pages may be shared between requests only if every key of the prefix stays in the cache and
-        # no other per-request state would have to be rebuilt.
-        self.prefix_caching = bool(prefix_caching and self.groups and not self.state_groups
-                                   and all(g.spec.window is None for g in self.groups))
+        # Pages may be shared between requests unless per-request state would have to be rebuilt with them: a
+        # state is no function of pages.  A group with a window shares the pages its window still covers.
+        self.prefix_caching = bool(prefix_caching and self.groups and not self.state_groups)
         self._prefixes: dict[bytes, _PrefixEntry] = {}
         self._clock = 0
         self.evictions = 0
@@ -163,23 +164,43 @@ class CacheManager:
         if not self.prefix_caching:
             return seq
         bs, key = self.block_size, b""
+        keys, entries = [], []
         end = bs
         while end < len(tokens):
             key = self._chain(key, tokens[end - bs:end])
             entry = self._prefixes.get(key)
             if entry is None:
                 break
-            self._clock += 1
-            entry.last_used = self._clock
-            for g, page in zip(self.groups, entry.pages):
-                g.pool.retain(page)
-            for gi, (blocks, page) in enumerate(zip(seq.blocks, entry.pages)):
-                blocks.append(page)
-                seq.table_versions[gi] += 1
-            seq.prefix_keys.append(key)
-            seq.length = end
+            keys.append(key)
+            entries.append(entry)
             end += bs
+        # The request computes position n * bs next and reads, in a group with a window, the keys from
+        # n * bs - window + 1 on: the longest run of pages whose entries still hold those.
+        n = len(entries)
+        while n > 0 and not all(entries[i].pages[gi] is not None
+                                for gi, g in enumerate(self.groups) if g.spec.window is not None
+                                for i in range(self._first_needed(g, n * bs) // bs, n)):
+            n -= 1
+        for i in range(n):
+            self._clock += 1
+            entries[i].last_used = self._clock
+        for gi, g in enumerate(self.groups):
+            first = 0 if g.spec.window is None else self._first_needed(g, n * bs) // bs
+            for i in range(n):
+                page = entries[i].pages[gi] if i >= first else FREED
+                if page != FREED:
+                    g.pool.retain(page)
+                seq.blocks[gi].append(page)
+            if n:
+                seq.table_versions[gi] += 1
+        seq.prefix_keys = keys[:n]
+        seq.length = n * bs
         return seq
+
+    @staticmethod
+    def _first_needed(group, length: int) -> int:
+        """The oldest key that the token at position `length` reads in `group`."""
+        return 0 if group.spec.window is None else max(0, length - group.spec.window + 1)
 
     def publish(self, tokens, seq: SequenceCache, length: int | None = None) -> None:
         """Offer the full page of `seq` that ends at `length` (default: its computed length) for reuse.
@@ -201,24 +222,40 @@ class CacheManager:
         key = seq.prefix_keys[n_pages - 1]
         if key in self._prefixes:
             return
-        pages = [blocks[n_pages - 1] for blocks in seq.blocks]
+        # (a window may already have passed the page, when a long portion was computed in one step)
+        pages = [None if blocks[n_pages - 1] == FREED else blocks[n_pages - 1] for blocks in seq.blocks]
         for g, page in zip(self.groups, pages):
-            g.pool.retain(page)   # the cache's own reference, beside the live requests'
+            if page is not None:
+                g.pool.retain(page)   # the cache's own reference, beside the live requests'
         self._clock += 1
         self._prefixes[key] = _PrefixEntry(pages, self._clock)
 
-    def _evict_one(self) -> bool:
-        """Drop the least recently used prefix entry that only the cache still holds."""
+    def _evict_one(self, group: int | None = None) -> bool:
+        """Make a page free: drop the least recently used prefix entry that only the cache still holds.  For a
+        group with a window (`group`) a lesser step comes first: the least recently used entry gives back its
+        page of that group alone, if nobody else holds it, and stays as a link of its chain."""
+        if group is not None and self.groups[group].spec.window is not None:
+            pool, best = self.groups[group].pool, None
+            for entry in self._prefixes.values():
+                page = entry.pages[group]
+                if page is not None and pool.refs[page] == 1 and (best is None or entry.last_used < best.last_used):
+                    best = entry
+            if best is not None:
+                pool.release(best.pages[group])
+                best.pages[group] = None
+                self.evictions += 1
+                return True
         best_key, best = None, None
         for key, entry in self._prefixes.items():
-            if all(g.pool.refs[p] == 1 for g, p in zip(self.groups, entry.pages)):
+            if all(p is None or g.pool.refs[p] == 1 for g, p in zip(self.groups, entry.pages)):
                 if best is None or entry.last_used < best.last_used:
                     best_key, best = key, entry
         if best is None:
             return False
         del self._prefixes[best_key]
         for g, page in zip(self.groups, best.pages):
-            g.pool.release(page)
+            if page is not None:
+                g.pool.release(page)
         self.evictions += 1
         return True
 
@@ -240,7 +277,7 @@ class CacheManager:
         for gi, (g, count) in enumerate(zip(self.groups, self.pages_needed(seq, new_length))):
             for _ in range(count):
                 page = g.pool.allocate()
-                while page is None and self._evict_one():
+                while page is None and self._evict_one(gi):
                     page = g.pool.allocate()
                 if page is None:
                     for gj, p in reversed(taken):
@@ -263,8 +300,7 @@ class CacheManager:
             if g.spec.window is None:
                 continue
             # the next token (position new_length) reads keys >= new_length - window + 1
-            first_needed = max(0, new_length - g.spec.window + 1)
-            for i in range(first_needed // self.block_size):
+            for i in range(self._first_needed(g, new_length) // self.block_size):
                 if blocks[i] != FREED:
                     g.pool.release(blocks[i])
                     blocks[i] = FREED
@@ -285,7 +321,8 @@ class CacheManager:
     def clear_prefixes(self) -> None:
         for entry in self._prefixes.values():
             for g, page in zip(self.groups, entry.pages):
-                g.pool.release(page)
+                if page is not None:
+                    g.pool.release(page)
         self._prefixes.clear()
 
     # ------------------------------------------------------------------ reports
@@ -296,7 +333,7 @@ class CacheManager:
         """Reference: src/kv-cache.ts:162-171, one record per group."""
         groups = []
         for gi, g in enumerate(self.groups):
-            cached = {e.pages[gi] for e in self._prefixes.values()}
+            cached = {e.pages[gi] for e in self._prefixes.values() if e.pages[gi] is not None}
             groups.append({
                 "window": g.spec.window, "slots": list(g.slots), "total_pages": g.pool.num_pages,
                 "free_pages": g.pool.num_free, "cached_pages": len(cached),

@@ -21,7 +21,8 @@ def invariants(cache: CacheManager):
                 if page != FREED:
                     held[page] = held.get(page, 0) + 1
         for entry in cache._prefixes.values():
-            held[entry.pages[gi]] = held.get(entry.pages[gi], 0) + 1
+            if entry.pages[gi] is not None:
+                held[entry.pages[gi]] = held.get(entry.pages[gi], 0) + 1
         free = list(g.pool._free)
         assert len(free) == len(set(free)), "a page is on the free list twice"
         for page in range(g.pool.num_pages):
@@ -58,8 +59,7 @@ def test_reserve_is_all_or_nothing_over_groups():
 
 
 def test_window_gives_pages_back_as_it_passes_them():
-    cache = CacheManager([WINDOWED], block_size=4, num_blocks=5, max_sequences=1, prefix_caching=True)
-    assert not cache.prefix_caching      # a window cannot share prefixes
+    cache = CacheManager([WINDOWED], block_size=4, num_blocks=5, max_sequences=1, prefix_caching=False)
     seq = cache.create()
     for length in range(1, 41):
         assert cache.reserve(seq, length), f"window of 10 must fit 5 pages of 4 at length {length}"
@@ -113,6 +113,92 @@ def test_prefix_reuse_leaves_the_last_token_to_compute():
     assert cache.free_pages() == [8]
 
 
+def feed(cache, seq, tokens, portion):
+    """Compute `tokens` in portions, publishing every full page as the scheduler does after a step."""
+    bs = cache.block_size
+    while seq.length < len(tokens):
+        old, new = seq.length, min(len(tokens), seq.length + portion)
+        assert cache.reserve(seq, new)
+        cache.commit(seq, new)
+        for boundary in range((old // bs + 1) * bs, new + 1, bs):
+            cache.publish(tokens, seq, boundary)
+
+
+def test_a_windowed_group_shares_the_pages_its_window_still_covers():
+    """A group with a window of 10 beside one that keeps every key, pages of 4.  A second request with the same
+    first 21 tokens takes over five pages: all five in the full group; in the windowed group those from key
+    20 - 10 + 1 = 11 on (pages 2..4), the earlier places of its table marked as given back."""
+    cache = CacheManager([FULL, WINDOWED], block_size=4, num_blocks=12, max_sequences=3)
+    assert cache.prefix_caching
+    tokens = list(range(100, 123))                            # 23 tokens: five full pages and three more
+    a = cache.create()
+    feed(cache, a, tokens, portion=3)                         # portions shorter than the window: every page is live when offered
+    assert a.blocks[1][:3] == [FREED] * 3                     # a's own window (from key 14) has passed pages 0..2
+    b = cache.reuse_prefix(tokens[:21] + [7, 7])
+    assert b.length == 20 and b.blocks[0] == a.blocks[0][:5]
+    assert b.blocks[1][:2] == [FREED, FREED] and all(p != FREED for p in b.blocks[1][2:5])
+    assert b.blocks[1][3:5] == a.blocks[1][3:5]               # the very pages a wrote
+    invariants(cache)
+    # b goes on: its window passes pages like anyone's, the cache keeps its own reference
+    feed(cache, b, tokens[:21] + [7, 7], portion=2)
+    assert b.length == 23 and b.blocks[1][2] == FREED
+    invariants(cache)
+    a.release(); b.release()
+    assert cache.free_pages()[0] == 12 - 5                    # the five shared pages stay cached
+    cache.clear_prefixes()
+    assert cache.free_pages() == [12, 12]
+
+
+def test_a_long_portion_offers_what_its_window_has_left_and_reuse_stops_where_keys_are_missing():
+    """Computed in one step, a prompt of 24 tokens has given back the windowed pages before key 15 when its pages
+    are offered: the entries of pages 0..2 hold no page of that group.  A request that shares 8 tokens would
+    read keys from 8 - 10 + 1 < 0 on, which nobody holds: it shares nothing.  One that shares all 24 shares
+    five pages (one token is left to compute) and reads keys from 11 on: page 2 is missing, so it steps back
+    until its window is whole, which it never is here: nothing either.  After the same prompt came in short
+    portions, both share."""
+    cache = CacheManager([FULL, WINDOWED], block_size=4, num_blocks=16, max_sequences=4)
+    tokens = list(range(24))
+    a = cache.create()
+    feed(cache, a, tokens, portion=24)
+    assert [e.pages[1] is None for e in sorted(cache._prefixes.values(), key=lambda e: e.last_used)] == [True] * 3 + [False] * 3
+    assert cache.reuse_prefix(tokens[:8] + [99]).length == 0
+    assert cache.reuse_prefix(tokens).length == 0
+    invariants(cache)
+    for seq in list(cache.live):
+        seq.release()
+    cache.clear_prefixes()
+    a = cache.create()
+    feed(cache, a, tokens, portion=4)
+    assert cache.reuse_prefix(tokens[:8] + [99]).length == 8 and cache.reuse_prefix(tokens).length == 20
+    invariants(cache)
+
+
+def test_a_short_windowed_pool_takes_cached_pages_back_one_at_a_time():
+    """When a windowed group's pool is empty, the least recently used entry gives back that group's page alone
+    and stays a link of its chain; a request whose window would need the missing page shares less."""
+    cache = CacheManager([WINDOWED], block_size=4, num_blocks=6, max_sequences=3)
+    tokens = list(range(16))
+    a = cache.create()
+    feed(cache, a, tokens, portion=4)
+    a.release()                                               # four pages cached
+    assert cache.free_pages() == [2]
+    b = cache.create()
+    assert cache.reserve(b, 12)                               # three pages: one more than are free
+    assert cache.evictions == 1 and len(cache._prefixes) == 4
+    first = min(cache._prefixes.values(), key=lambda e: e.last_used)
+    assert first.pages == [None]                              # the oldest entry gave its page back and stays
+    invariants(cache)
+    c = cache.reuse_prefix(tokens)     # three pages offered; a window of 10 at key 12 begins at key 3, in page 0
+    assert c.length == 0
+    d = cache.reuse_prefix(tokens + [1] * 8)   # four pages: at key 16 the window begins at key 7, in page 1
+    assert d.length == 16 and d.blocks[0][0] == FREED and FREED not in d.blocks[0][1:]
+    invariants(cache)
+    for seq in (b, c, d):
+        seq.release()
+    cache.clear_prefixes()
+    assert cache.free_pages() == [6]
+
+
 def test_lru_eviction_takes_only_pages_no_request_uses():
     cache = CacheManager([FULL], block_size=2, num_blocks=3, max_sequences=4)
     a = cache.create()
@@ -143,10 +229,10 @@ def test_state_slots_are_per_request_and_come_back():
     assert cache.create().state_slot == a.state_slot
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(12))
 def test_random_orders_never_lose_or_double_a_page(seed):
     rng = random.Random(seed)
-    specs = [FULL, WINDOWED] if seed % 2 else [FULL]
+    specs = [[FULL], [FULL, WINDOWED], [WINDOWED], [PagedKVSpec(1, 8, window=5), FULL, WINDOWED]][seed % 4]
     cache = CacheManager(specs, block_size=4, num_blocks=12, max_sequences=5, prefix_caching=True)
     live = []
     prompts = [[rng.randrange(3) for _ in range(rng.randrange(1, 30))] for _ in range(8)]

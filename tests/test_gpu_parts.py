@@ -634,3 +634,139 @@ def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path, dtype):
     for s in seqs.values():
         s.release()
     assert runner.cache.free_pages() == [24]             # both layers have the same needs: one group of pages
+
+
+def register_windowed_toy():
+    """Two layers of the engine's own parts, the second with a window: two cache groups and no state."""
+    from dataclasses import dataclass
+    from typing import ClassVar
+
+    import sprout_lm_amd as S
+    from sprout_lm_amd.config.base import ModelConfig
+    from sprout_lm_amd.models.plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+    from sprout_lm_amd.registry import registered_architectures
+
+    if "ToyWindowForCausalLM" in registered_architectures():
+        return
+
+    @dataclass(frozen=True)
+    class WindowConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyWindowForCausalLM"
+        model_types: ClassVar[tuple] = ("toy_window",)
+        hidden: int = 0
+        inner: int = 0
+        vocab: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        window: int = 0
+        eps: float = 0.0
+        theta: float = 0.0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "window", "eps", "theta")})
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "model_type": "toy_window", "hidden": self.hidden,
+                    "inner": self.inner, "vocab": self.vocab, "heads": self.heads, "kv_heads": self.kv_heads,
+                    "window": self.window, "eps": self.eps, "theta": self.theta}
+
+    def build(cfg):
+        hd = cfg.hidden // cfg.heads
+        norm = lambda prefix: PartPlan("norm", "rmsnorm", {"size": cfg.hidden, "eps": cfg.eps}, prefix)
+        attention = lambda prefix, **extra: PartPlan("mixer", "attention", {
+            "hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.kv_heads, "head_dim": hd,
+            "position": PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": cfg.theta}), **extra}, prefix)
+        mlp = lambda prefix: PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner}, prefix)
+        mixers = [attention("l0.attn."), attention("l1.attn.", window=cfg.window)]
+        layers = [LayerPlan("pre_norm", {"mixer_norm": norm(f"l{i}.n1."), "mixer": m, "ffn_norm": norm(f"l{i}.n2."),
+                                         "ffn": mlp(f"l{i}.mlp.")}) for i, m in enumerate(mixers)]
+        return ModelPlan("ToyWindowForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
+                         PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.hidden}, "embed."),
+                         layers, [LayerCall(0, 0), LayerCall(1, 1)], norm("final."),
+                         PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.hidden, "tied": True}, "head."))
+
+    S.register_architecture("ToyWindowForCausalLM", WindowConfig, build, model_types=("toy_window",))
+
+
+WINDOWED = dict(model_type="toy_window", hidden=64, inner=96, vocab=89, heads=4, kv_heads=2, window=10, eps=1e-6, theta=1e4)
+
+
+def plain_windowed_logits(w, tokens, store):
+    c = WINDOWED
+    hd = c["hidden"] // c["heads"]
+    pos = np.arange(len(tokens))
+    x = P.f32(w["embed.weight"][np.asarray(tokens)])
+    for i, window in enumerate([None, c["window"]]):
+        p = f"l{i}.attn."
+        n = store(P.rms_norm(x, w[f"l{i}.n1.weight"], c["eps"]))
+        q = store(P.rope_neox(store(P.linear(n, w[p + "q_proj.weight"], w[p + "q_proj.bias"])), pos, hd, c["theta"]))
+        k = store(P.rope_neox(store(P.linear(n, w[p + "k_proj.weight"], w[p + "k_proj.bias"])), pos, hd, c["theta"]))
+        v = store(P.linear(n, w[p + "v_proj.weight"], w[p + "v_proj.bias"]))
+        a = store(P.causal_gqa_attention(q, k, v, c["heads"], c["kv_heads"], hd, window=window))
+        x = P.f32(x + P.linear(a, w[p + "o_proj.weight"]))
+        n = store(P.rms_norm(x, w[f"l{i}.n2.weight"], c["eps"]))
+        gate, up = store(P.linear(n, w[f"l{i}.mlp.gate_proj.weight"])), store(P.linear(n, w[f"l{i}.mlp.up_proj.weight"]))
+        x = P.f32(x + P.linear(store(P.swiglu(gate, up)), w[f"l{i}.mlp.down_proj.weight"]))
+    return P.linear(store(P.rms_norm(x, w["final.weight"], c["eps"])), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype):
+    """A model with a layer that keeps every key and one with a window of 10 (pages of 4): a second request takes
+    over the pages of a shared prefix in both cache groups, in the windowed one only those its window still covers
+    (the earlier places of its block table say `given back`), and computes on from there; a third one after the
+    first two have ended finds the pages in the cache alone.  Every logit row of the later requests against the
+    plain implementation, which knows no cache."""
+    register_windowed_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cache import FREED
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    folder = str(tmp_path / "windowed")
+    write_model_folder(folder, S.config_from_dict(WINDOWED), seed=17, dtype=torch.bfloat16, std=0.15)
+    runner = ModelRunner.from_folder(folder, dtype, block_size=4, num_blocks=40, max_sequences=3, prefix_caching=True)
+    cache = runner.cache
+    assert cache.prefix_caching and [g.spec.window for g in cache.groups] == [None, 10]
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    store = P.bf16_round if dtype == "bfloat16" else P.f32
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    shared = H.random_tokens(89, 30, 5)
+    requests = {"a": shared + H.random_tokens(89, 9, 6), "b": shared[:26] + H.random_tokens(89, 15, 7),
+                "c": shared[:22] + H.random_tokens(89, 11, 8)}
+
+    def run(rid, seq, portions):
+        tokens, worst = requests[rid], 0.0
+        want = plain_windowed_logits(w, tokens, store)
+        for n in portions:
+            old, new = seq.length, min(len(tokens), seq.length + n)
+            if new == old:
+                break
+            assert cache.reserve(seq, new)
+            got = runner.step([StepEntry(seq, tokens[old:new], list(range(new - old)))]).cpu().numpy()
+            for boundary in range((old // 4 + 1) * 4, new + 1, 4):
+                cache.publish(tokens, seq, boundary)
+            for i, row in enumerate(got):
+                err = np.abs(row - want[old + i]).max() / (tol * (1 + np.abs(want[old + i]).max()))
+                worst = max(worst, err)
+                assert err <= 1.0, f"{rid} position {old + i}: {err:.2f} of the bound"
+        assert seq.length == len(tokens)
+        return worst
+
+    a = cache.create()
+    worst = run("a", a, [3] * 20)                       # portions shorter than the window: every page is offered live
+    b = cache.reuse_prefix(requests["b"])
+    assert b.length == 24 and b.blocks[0] == a.blocks[0][:6]
+    # b computes position 24 next and reads keys from 15 on: pages 3..5 of the windowed group, the ones a wrote
+    assert b.blocks[1][:3] == [FREED] * 3 and FREED not in b.blocks[1][3:6]
+    assert set(b.blocks[1][3:6]) <= {e.pages[1] for e in cache._prefixes.values()}
+    worst = max(worst, run("b", b, [5, 1, 1, 9, 4]))
+    a.release(); b.release()
+    c = cache.reuse_prefix(requests["c"])               # only the cache holds the pages now
+    assert c.length == 20 and c.blocks[1][:2] == [FREED] * 2 and FREED not in c.blocks[1][2:5]
+    worst = max(worst, run("c", c, [2, 7, 6]))
+    c.release()
+    cache.clear_prefixes()
+    assert cache.free_pages() == [40, 40]
+    print(f"windowed prefix sharing {dtype}: worst {worst:.2f} of the bound")
