@@ -65,7 +65,8 @@ __device__ __forceinline__ float4 ldg_f4(const float* __restrict__ p) { return *
 
 // The norm prologue's inputs of one pass as they come from memory: for each of the wave's UN steps the lane's 16
 // values of its token (two groups of 8 along K) and the norm's weights for them.  `request` asks for all of
-// them; `operands` turns them into x * norm weight in bfloat16 and adds the squares of x to `square_sum`.
+// them; `squares` sums the squares of x; `operands` turns them into (x * scale) * norm weight in bfloat16, the
+// very numbers that the norm kernel stores.
 // `row` and `norm_w` point at the lane's first value of the pass (step s0); step s0 + 4 u lies 256 u values on.
 // K64: K is whole steps, a step is there or not for the whole wave (`steps_left` of them from s0 on, every
 // fourth).  Otherwise groups past the end of K are read from `safe_row` / `safe_w` instead (valid addresses:
@@ -107,8 +108,24 @@ struct NormInputs {
     }
   }
 
-  __device__ __forceinline__ void operands(bool BF, int steps_left, int k_left, uint4 (&xb)[UN][1][2],
-                                           float& square_sum) const {
+  // This lane's share of the sum of squares of its token over the pass.
+  __device__ __forceinline__ float squares(int steps_left, int k_left) const {
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float4 x0 = xf[u][h][0], x1 = xf[u][h][1];
+        float sq = fmaf(x0.x, x0.x, fmaf(x0.y, x0.y, fmaf(x0.z, x0.z, x0.w * x0.w)));
+        sq = fmaf(x1.x, x1.x, fmaf(x1.y, x1.y, fmaf(x1.z, x1.z, fmaf(x1.w, x1.w, sq))));
+        if (K64) sum += sq;                     // a step that is not there holds zeros
+        else sum = fmaf((4 * u < steps_left && 256 * u + 8 * h < k_left) ? 1.f : 0.f, sq, sum);
+      }
+    return sum;
+  }
+
+  // (a group past the end of K meets weights of the product that are zeros: what stands here for it does not count)
+  __device__ __forceinline__ void operands(bool BF, float scale, uint4 (&xb)[UN][1][2]) const {
 #pragma unroll
     for (int u = 0; u < UN; ++u)
 #pragma unroll
@@ -125,13 +142,10 @@ struct NormInputs {
           w0 = make_float4(__uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w));
           w1 = make_float4(__uint_as_float(c.x), __uint_as_float(c.y), __uint_as_float(c.z), __uint_as_float(c.w));
         }
-        float sq = fmaf(x0.x, x0.x, fmaf(x0.y, x0.y, fmaf(x0.z, x0.z, x0.w * x0.w)));
-        sq = fmaf(x1.x, x1.x, fmaf(x1.y, x1.y, fmaf(x1.z, x1.z, fmaf(x1.w, x1.w, sq))));
-        if (K64) square_sum += sq;                     // a step that is not there holds zeros
-        else square_sum = fmaf((4 * u < steps_left && 256 * u + 8 * h < k_left) ? 1.f : 0.f, sq, square_sum);
-        // (the weights of a group past the end of K are zeros: what stands here for it does not count)
-        xb[u][0][h] = make_uint4(pack_bf16x2(x0.x * w0.x, x0.y * w0.y), pack_bf16x2(x0.z * w0.z, x0.w * w0.w),
-                                 pack_bf16x2(x1.x * w1.x, x1.y * w1.y), pack_bf16x2(x1.z * w1.z, x1.w * w1.w));
+        xb[u][0][h] = make_uint4(pack_bf16x2((x0.x * scale) * w0.x, (x0.y * scale) * w0.y),
+                                 pack_bf16x2((x0.z * scale) * w0.z, (x0.w * scale) * w0.w),
+                                 pack_bf16x2((x1.x * scale) * w1.x, (x1.y * scale) * w1.y),
+                                 pack_bf16x2((x1.z * scale) * w1.z, (x1.w * scale) * w1.w));
       }
   }
 };
@@ -219,8 +233,10 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     normed.request(norm_row + 64 * s0, norm_w0 + size_t(64 * s0) * (a.norm_w_bf16 ? 2 : 4), a.norm_w_bf16, steps - s0,
                    k_end - (k_begin + 16 * lj + 64 * s0), a.residual, a.norm_w);
   };
-  load_weights(wave);
+  // NORM: the rows first (they come from the caches and are needed first: their sum of squares is exchanged
+  // between the waves while the weights, which take longest, are on their way)
   if constexpr (NORM) request_rows(wave);
+  load_weights(wave);
   __builtin_amdgcn_sched_barrier(0);   // keep these requests ahead of everything below
   // What the epilogue reads per output (bias, position, rotation frequency, cache slot) is requested now
   // as well: asked for after the sums are done, it would be one more trip to memory at the end of the kernel.
@@ -261,8 +277,27 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) acc[i][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  // NORM: 1 / sqrt(mean(x^2) + eps) of token lr, before anything is rounded: the activations are then the numbers
+  // that the norm kernel stores, whichever way a step is computed.  The four waves hold a quarter of the row's
+  // steps each; rows longer than one pass (4 UN steps) are read once more for their squares.  The weights asked
+  // for above are on their way meanwhile.
+  float row_scale = 1.f;
+  if constexpr (NORM) {
+    float square_sum = normed.squares(steps - wave, k_end - (k_begin + 16 * lj + 64 * wave));
+    for (int s0 = wave + 4 * UN; s0 < steps; s0 += 4 * UN) {
+      NormInputs<UN, K64> further;
+      further.request(norm_row + 64 * s0, norm_w0 + size_t(64 * s0) * (a.norm_w_bf16 ? 2 : 4), a.norm_w_bf16, steps - s0,
+                      k_end - (k_begin + 16 * lj + 64 * s0), a.residual, a.norm_w);
+      square_sum += further.squares(steps - s0, k_end - (k_begin + 16 * lj + 64 * s0));
+    }
+    square_sum += __shfl_xor(square_sum, 16, 64);   // the four lanes of a token hold a quarter of the wave's steps each
+    square_sum += __shfl_xor(square_sum, 32, 64);
+    if (lj == 0) squares[wave * 16 + lr] = square_sum;
+    __syncthreads();
+    row_scale = 1.0f / sqrtf((squares[lr] + squares[16 + lr] + squares[32 + lr] + squares[48 + lr]) / float(a.K) + a.eps);
+  }
+
   // this wave's steps of 64 along K: wave, wave + 4, ...; UN steps are loaded before they are multiplied
-  float square_sum = 0.f;   // NORM: this lane's share of the sum of squares of token lr
   for (int s0 = wave; s0 < steps; s0 += 4 * UN) {
     if (s0 != wave) {
       load_weights(s0);
@@ -271,9 +306,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
     uint4 xb[UN][TN][2];
     if constexpr (NORM) {
       // Lane (lr, lj) needs 16 values of token lr per step, as the matrix cores take them.  They come straight
-      // from the float32 residual, times the norm's weights (the same for every token), rounded to bfloat16;
-      // the token's scale follows in the epilogue.
-      normed.operands(a.norm_w_bf16, steps - s0, k_end - (k_begin + 16 * lj + 64 * s0), xb, square_sum);
+      // from the float32 residual, times the token's scale, times the norm's weights, rounded to bfloat16.
+      normed.operands(a.norm_w_bf16, row_scale, xb);
     } else {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
@@ -312,11 +346,6 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
       red[((wave * NT + i) * TN + tn) * 64 + lane] = make_float4(acc[i][tn][0], acc[i][tn][1], acc[i][tn][2], acc[i][tn][3]);
-  if (NORM) {   // the four lanes of a token hold a quarter of the wave's steps each
-    square_sum += __shfl_xor(square_sum, 16, 64);
-    square_sum += __shfl_xor(square_sum, 32, 64);
-    if (lj == 0) squares[wave * 16 + lr] = square_sum;
-  }
   __syncthreads();
 
   // The sum of the four waves for (tile, row of the tile, token tile tn, token et): row r of a tile lies in
@@ -328,9 +357,6 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       sum += reinterpret_cast<const float*>(&red[((w * NT + tile) * TN + tn) * 64 + (row >> 2) * 16 + et])[row & 3];
     return sum;
   };
-  // NORM: 1 / sqrt(mean(x^2) + eps) of this thread's token, from the four waves' shares of the sum
-  const float scale_of = NORM ? rsqrtf((squares[et] + squares[16 + et] + squares[32 + et] + squares[48 + et]) / float(a.K) + a.eps)
-                              : 1.f;
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     const int t = t0 + tn * 16 + et;
@@ -341,7 +367,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         const int p = 16 * o + ei, n = blockIdx.x * r + p;     // inner column p of the block
         if (p >= r || n >= a.partner || t >= a.T) continue;
         const int gate = p, up = p + r;                         // their places among the block's rows
-        const float gv = summed(gate >> 4, gate & 15, tn) * scale_of, uv = summed(up >> 4, up & 15, tn) * scale_of;
+        const float gv = summed(gate >> 4, gate & 15, tn), uv = summed(up >> 4, up & 15, tn);
         // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
         const float g = to_float(bf16_t{f32_to_bf16_bits(gv)}), u = to_float(bf16_t{f32_to_bf16_bits(uv)});
         reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
@@ -352,7 +378,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const float sum = (EPI == kEpiRope && NT == 1) ? summed(0, er + 8 * i, tn) : summed(i, ei, tn);
-      v[i] = (NORM ? sum * scale_of : sum) + param_value(bias_bits[i], a.bias_bf16);
+      v[i] = sum + param_value(bias_bits[i], a.bias_bf16);
     }
     if (t >= a.T || (EPI == kEpiRope && NT == 1 && ei >= 8)) continue;
     if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {

@@ -517,17 +517,6 @@ def _normed(res, w, eps):
     return bf16(x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * w)
 
 
-def _product(x, res, nw, eps, w, norm):
-    """x . w^T in float64.  With `norm` the activations are rmsnorm(res) * nw, rounded to bfloat16 where the
-    kernels with the norm folded in round them: the product of a value and its norm weight is rounded, and the
-    row's 1 / sqrt(mean(x^2) + eps) multiplies the finished sums (the same number, another place of rounding)."""
-    if not norm:
-        return x.astype(np.float64) @ w.astype(np.float64).T
-    r = res.astype(np.float64)
-    sums = bf16(r * nw).astype(np.float64) @ w.astype(np.float64).T
-    return sums / np.sqrt((r * r).mean(-1, keepdims=True) + eps)
-
-
 @pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64, 65, 200, 513])   # above 64: the tiled product's rotating epilogue
 # the last two: few rows with a long K, which eight waves of a block share instead of four
 @pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4),
@@ -560,7 +549,7 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
             call()
         return
     call()
-    qkv = bf16(_product(x, res, nw, eps, w, norm) + b)
+    qkv = bf16(x.astype(np.float64) @ w.astype(np.float64).T + b)
     want = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, hd, theta)
     got_q = q_out.float().cpu().numpy()
     scale = 1 + np.abs(want).max()
@@ -608,7 +597,7 @@ def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
             ops.gate_up_silu(t(w, torch.bfloat16), out, **args)
         return
     ops.gate_up_silu(t(w, torch.bfloat16), out, **args)
-    gu = bf16(_product(x, res, nw, eps, w, norm)).astype(np.float64)
+    gu = bf16(x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float64)
     g, u = gu[:, :I], gu[:, I:]
     want = g / (1 + np.exp(-g)) * u
     assert np.abs(out.float().cpu().numpy() - want).max() <= 2 ** -6 * (1 + np.abs(want).max())
