@@ -234,6 +234,9 @@ def main() -> int:
                         help="also time the batch decoding beside a prompt prefilled this many tokens a step (0: skip)")
     parser.add_argument("--second-preset", default="qwen2.5-7b",
                         help="sizes of the second model whose decode step and prefill go into `points` ('' or 'none': skip)")
+    parser.add_argument("--prefill-only", action="store_true",
+                        help="time nothing but the prefill of --prefill-tokens (for a profile of that step alone); "
+                             "prints a shorter line")
     parser.add_argument("--pressure", type=float, default=0.0, metavar="SHARE",
                         help="also run the batch from 512-token prompts in a pool of this share of the pages it needs")
     args = parser.parse_args()
@@ -250,6 +253,17 @@ def main() -> int:
     cfg = config_from_dict(raw)
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     element = 2 if args.dtype == "bf16" else 4
+
+    if args.prefill_only:
+        engine = make_engine(cfg, dtype, 1, args.prefill_tokens, args.prefill_tokens)
+        seconds = measure_prefill(engine, cfg, args.prefill_tokens)
+        flops = prefill_flops(engine.model.parts, args.prefill_tokens)
+        engine.close()
+        print(json.dumps({"metric": f"prefill tok/s at {args.prefill_tokens:,} tokens ({args.preset} sizes)",
+                          "value": round(args.prefill_tokens / seconds, 1), "unit": "tokens/s", "n_gpus": 1,
+                          "ms": round(seconds * 1000, 3), "dtype": args.dtype, "layers": cfg.num_hidden_layers,
+                          "frac": round(flops / seconds / MFMA_PEAK[args.dtype], 5)}))
+        return 0
 
     from sprout_lm_amd import ops
     measured = ops.probe_machine()
