@@ -23,6 +23,7 @@ class PagedGroup:
     spec: PagedKVSpec
     slots: list[int]              # cache slot ids that live in this group, in pool order
     pool: PagePool
+    page_tokens: int = 0          # tokens in one page of this group
     k: object = None              # device tensor [len(slots), pages, kv_heads, page_size, head_dim]
     v: object = None              # device tensor [len(slots), pages, kv_heads, head_dim, page_size]
 
@@ -62,8 +63,9 @@ class SequenceCache:
 
 @dataclass
 class _PrefixEntry:
-    """One full page of a prefix, in every group: the page's id, or None where a windowed group has given its
-    page back (the entry then still links the chain, and serves requests whose window lies behind it)."""
+    """`block_size` tokens of a prefix in every group: that group's pages of them, or None where a windowed
+    group has given them back (the entry then still links the chain, and serves requests whose window lies
+    behind it)."""
     pages: list
     last_used: int
 
@@ -82,7 +84,12 @@ class CacheManager:
         for slot, spec in enumerate(slot_specs):
             if isinstance(spec, PagedKVSpec):
                 groups, kind = self.groups, "paged"
-                make = lambda: PagedGroup(spec, [], PagePool(num_blocks))
+                tokens = spec.page_tokens or block_size
+                if isinstance(tokens, bool) or not isinstance(tokens, int) or tokens <= 0 or block_size % tokens:
+                    raise ValueError(f"Cache slot {slot}: pages of {tokens!r} tokens do not divide the cache's pages of "
+                                     f"{block_size}.")
+                # every group holds the same number of tokens, in pages of its own size
+                make = lambda: PagedGroup(spec, [], PagePool(num_blocks * (block_size // tokens)), tokens)
             elif isinstance(spec, StateSpec):
                 groups, kind = self.state_groups, "state"
                 make = lambda: StateGroup(spec, [])
@@ -113,8 +120,8 @@ class CacheManager:
             # keys [slot, page, head, token, dim]; values [slot, page, head, dim, token]: the keys of one
             # dimension lie together, which is how the P.V matrix product reads them
             n, kv, hd = len(g.slots), g.spec.kv_heads, g.spec.head_dim
-            g.k = torch.zeros((n, self.num_blocks, kv, self.block_size, hd), dtype=dtype, device=device)
-            g.v = torch.zeros((n, self.num_blocks, kv, hd, self.block_size), dtype=dtype, device=device)
+            g.k = torch.zeros((n, g.pool.num_pages, kv, g.page_tokens, hd), dtype=dtype, device=device)
+            g.v = torch.zeros((n, g.pool.num_pages, kv, hd, g.page_tokens), dtype=dtype, device=device)
         for g in self.state_groups:
             # one slot more than requests can hold: `spare_state_slot`, where the padding rows of a recorded
             # step keep their state, so that no part has to tell them from real rows
@@ -130,7 +137,7 @@ class CacheManager:
         """Device bytes of every pool and state tensor for cache elements of `element_size` bytes."""
         total = 0
         for g in self.groups:
-            total += 2 * len(g.slots) * self.num_blocks * g.spec.kv_heads * self.block_size * g.spec.head_dim * element_size
+            total += 2 * len(g.slots) * g.pool.num_pages * g.spec.kv_heads * g.page_tokens * g.spec.head_dim * element_size
         for g in self.state_groups:
             count = 1
             for n in g.spec.shape:
@@ -187,10 +194,12 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             first = 0 if g.spec.window is None else self._first_needed(g, n * bs) // bs
             for i in range(n):
-                page = entries[i].pages[gi] if i >= first else FREED
-                if page != FREED:
-                    g.pool.retain(page)
-                seq.blocks[gi].append(page)
+                if i >= first:
+                    for page in entries[i].pages[gi]:
+                        g.pool.retain(page)
+                    seq.blocks[gi].extend(entries[i].pages[gi])
+                else:
+                    seq.blocks[gi].extend([FREED] * (bs // g.page_tokens))
             if n:
                 seq.table_versions[gi] += 1
         seq.prefix_keys = keys[:n]
@@ -222,10 +231,15 @@ class CacheManager:
         key = seq.prefix_keys[n_pages - 1]
         if key in self._prefixes:
             return
-        # (a window may already have passed the page, when a long portion was computed in one step)
-        pages = [None if blocks[n_pages - 1] == FREED else blocks[n_pages - 1] for blocks in seq.blocks]
-        for g, page in zip(self.groups, pages):
-            if page is not None:
+        # every group's pages of these `bs` tokens (a window may already have passed some of them, when a long
+        # portion was computed in one step: then the entry holds none of that group)
+        pages = []
+        for g, blocks in zip(self.groups, seq.blocks):
+            per = bs // g.page_tokens
+            mine = blocks[(n_pages - 1) * per:n_pages * per]
+            pages.append(None if FREED in mine else list(mine))
+        for g, mine in zip(self.groups, pages):
+            for page in mine or ():
                 g.pool.retain(page)   # the cache's own reference, beside the live requests'
         self._clock += 1
         self._prefixes[key] = _PrefixEntry(pages, self._clock)
@@ -237,32 +251,32 @@ class CacheManager:
         if group is not None and self.groups[group].spec.window is not None:
             pool, best = self.groups[group].pool, None
             for entry in self._prefixes.values():
-                page = entry.pages[group]
-                if page is not None and pool.refs[page] == 1 and (best is None or entry.last_used < best.last_used):
+                mine = entry.pages[group]
+                if mine is not None and all(pool.refs[p] == 1 for p in mine) and (best is None or entry.last_used < best.last_used):
                     best = entry
             if best is not None:
-                pool.release(best.pages[group])
+                for page in best.pages[group]:
+                    pool.release(page)
                 best.pages[group] = None
                 self.evictions += 1
                 return True
         best_key, best = None, None
         for key, entry in self._prefixes.items():
-            if all(p is None or g.pool.refs[p] == 1 for g, p in zip(self.groups, entry.pages)):
+            if all(g.pool.refs[p] == 1 for g, mine in zip(self.groups, entry.pages) for p in mine or ()):
                 if best is None or entry.last_used < best.last_used:
                     best_key, best = key, entry
         if best is None:
             return False
         del self._prefixes[best_key]
-        for g, page in zip(self.groups, best.pages):
-            if page is not None:
+        for g, mine in zip(self.groups, best.pages):
+            for page in mine or ():
                 g.pool.release(page)
         self.evictions += 1
         return True
 
     def pages_needed(self, seq: SequenceCache, new_length: int) -> list[int]:
         """Pages each group must still allocate so that `seq` can hold `new_length` tokens."""
-        need = -(-new_length // self.block_size)
-        return [max(0, need - len(blocks)) for blocks in seq.blocks]
+        return [max(0, -(-new_length // g.page_tokens) - len(blocks)) for g, blocks in zip(self.groups, seq.blocks)]
 
     def reserve(self, seq: SequenceCache, new_length: int) -> bool:
         """Allocate pages in every group for tokens up to `new_length`.  All or nothing.
@@ -293,14 +307,14 @@ class CacheManager:
     def commit(self, seq: SequenceCache, new_length: int) -> None:
         """The step has written tokens up to `new_length`: record it and give back what windows have passed."""
         seq._live()
-        if new_length > min((len(b) for b in seq.blocks), default=new_length // self.block_size + 1) * self.block_size:
+        if any(new_length > len(blocks) * g.page_tokens for g, blocks in zip(self.groups, seq.blocks)):
             raise PageError("Committed more tokens than pages were reserved for.")
         seq.length = new_length
         for gi, (g, blocks) in enumerate(zip(self.groups, seq.blocks)):
             if g.spec.window is None:
                 continue
             # the next token (position new_length) reads keys >= new_length - window + 1
-            for i in range(self._first_needed(g, new_length) // self.block_size):
+            for i in range(self._first_needed(g, new_length) // g.page_tokens):
                 if blocks[i] != FREED:
                     g.pool.release(blocks[i])
                     blocks[i] = FREED
@@ -320,8 +334,8 @@ class CacheManager:
 
     def clear_prefixes(self) -> None:
         for entry in self._prefixes.values():
-            for g, page in zip(self.groups, entry.pages):
-                if page is not None:
+            for g, mine in zip(self.groups, entry.pages):
+                for page in mine or ():
                     g.pool.release(page)
         self._prefixes.clear()
 
@@ -333,9 +347,9 @@ class CacheManager:
         """Reference: src/kv-cache.ts:162-171, one record per group."""
         groups = []
         for gi, g in enumerate(self.groups):
-            cached = {e.pages[gi] for e in self._prefixes.values() if e.pages[gi] is not None}
+            cached = {p for e in self._prefixes.values() for p in e.pages[gi] or ()}
             groups.append({
-                "window": g.spec.window, "slots": list(g.slots), "total_pages": g.pool.num_pages,
+                "window": g.spec.window, "page_tokens": g.page_tokens, "slots": list(g.slots), "total_pages": g.pool.num_pages,
                 "free_pages": g.pool.num_free, "cached_pages": len(cached),
                 "pages": [{"id": i, "refs": r, "cached": i in cached, "active_refs": r - (i in cached)}
                           for i, r in enumerate(g.pool.refs)],

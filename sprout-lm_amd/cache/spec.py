@@ -6,11 +6,14 @@ from dataclasses import dataclass
 
 @dataclass(frozen=True)
 class PagedKVSpec:
-    """Keys and values in pages.  window None: every earlier key stays; else only the last `window`."""
+    """Keys and values in pages.  window None: every earlier key stays; else only the last `window`.
+    page_tokens None: pages of the cache manager's own size; else pages of this many tokens (a divisor of the
+    manager's size, which stays the unit in which prefixes are shared)."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
+    page_tokens: int | None = None
 
 
 @dataclass(frozen=True)

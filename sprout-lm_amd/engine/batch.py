@@ -133,14 +133,13 @@ class StepArrays:
         return self.arrays[self.names.index(name)]
 
 
-def step_arrays(entries: list[StepEntry], cache, table_width: int | None = None) -> StepArrays:
+def step_arrays(entries: list[StepEntry], cache, table_tokens: int | None = None) -> StepArrays:
     """Lay the entries out flat: token ids, positions, per-sequence start / length / context, the places of
-    wanted logits, state slots, the attention work lists, and per cache group the block tables (`table_width`
-    entries a row, by default as many as the longest table) and the cache slot of every token.
+    wanted logits, state slots, the attention work lists, and per cache group the block tables (a row holds the
+    pages of `table_tokens` tokens, by default as many as the longest table) and the cache slot of every token.
 
     Each entry's sequence must already hold pages for its new tokens (CacheManager.reserve).
     """
-    bs = cache.block_size
     q_lens = [len(e.tokens) for e in entries]
     starts = np.zeros(len(entries), dtype=np.int32)
     if entries:
@@ -163,7 +162,8 @@ def step_arrays(entries: list[StepEntry], cache, table_width: int | None = None)
         names.append(name)
         arrays.append(lists[name])
     for gi, group in enumerate(cache.groups):
-        width = table_width or max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
+        bs = group.page_tokens
+        width = -(-table_tokens // bs) if table_tokens else max(1, max((len(e.seq.blocks[gi]) for e in entries), default=1))
         tables = np.full((len(entries), width), -1, dtype=np.int32)
         slots = np.full(T, -1, dtype=np.int32)
         for s, e in enumerate(entries):

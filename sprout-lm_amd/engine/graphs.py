@@ -42,8 +42,7 @@ class _DecodeGraph:
         self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
         self.S = n_seqs
         cache = runner.cache
-        bs = cache.block_size
-        self.max_blocks = -(-ctx_bucket // bs)
+        self.max_blocks = [-(-ctx_bucket // g.page_tokens) for g in cache.groups]   # a table row's width, per group
         self.ctx_bucket = ctx_bucket
         S, G = n_seqs, len(cache.groups)
         # layout of the int32 staging buffer
@@ -58,8 +57,8 @@ class _DecodeGraph:
         for g in range(G):
             self.offsets[f"slots{g}"] = (total, S)
             total += (S + 3) // 4 * 4
-            self.offsets[f"tables{g}"] = (total, S * self.max_blocks)
-            total += (S * self.max_blocks + 3) // 4 * 4
+            self.offsets[f"tables{g}"] = (total, S * self.max_blocks[g])
+            total += (S * self.max_blocks[g] + 3) // 4 * 4
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
         self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
@@ -83,7 +82,7 @@ class _DecodeGraph:
         lists.update({f"tiles_all_{t}": (every, S) for t in ops.kernels.TILE_SIZES})
         lists["decode_seqs"] = (None, S)        # every sequence brings one token, in order: no list needed
         ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, S, lists, ctx_bucket, ctx_bucket)
-        ctx.group_tables = [view(f"tables{g}").view(S, self.max_blocks) for g in range(G)]
+        ctx.group_tables = [view(f"tables{g}").view(S, self.max_blocks[g]) for g in range(G)]
         ctx.group_slots = [view(f"slots{g}") for g in range(G)]
         ctx.n_tokens = ctx.n_seqs = ctx.n_logits = S
         ctx.max_q_len = 1
@@ -110,7 +109,6 @@ class _DecodeGraph:
         `sources[i] >= 0`: entry i's token is row sources[i] of an earlier step's sampled tokens, which
         the host does not know yet (its `tokens[0]` is None)."""
         cache, h, n, S = self.runner.cache, self.h, len(entries), self.S
-        bs = cache.block_size
         if self.copied is not None:
             self.copied.synchronize()      # the last launch's upload may still be reading the staging buffer
         lengths = np.fromiter((e.seq.length for e in entries), dtype=np.int32, count=n)
@@ -129,9 +127,10 @@ class _DecodeGraph:
             h["feed_source"][n:] = -1
             h["ctx_len"][n:] = 1
             self._rows = [None] * S
-        last_block = lengths // bs
         for g in range(len(cache.groups)):
-            tables = h[f"tables{g}"].reshape(S, self.max_blocks)
+            bs, width = cache.groups[g].page_tokens, self.max_blocks[g]
+            last_block = lengths // bs
+            tables = h[f"tables{g}"].reshape(S, width)
             slots = h[f"slots{g}"]
             if n != self._filled:
                 slots[n:] = -1
@@ -141,7 +140,7 @@ class _DecodeGraph:
                 blocks = e.seq.blocks[g]
                 key = (e.seq.uid, g, e.seq.table_versions[g])
                 if self._rows[i] is None or self._rows[i].get(g) != key:
-                    nb = min(len(blocks), self.max_blocks)
+                    nb = min(len(blocks), width)
                     tables[i, :nb] = blocks[:nb]
                     tables[i, nb:] = -1
                     if self._rows[i] is None:
@@ -184,7 +183,7 @@ class _PortionGraph:
     def __init__(self, runner, first, ctx_bucket: int):
         self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
         cache = runner.cache
-        self.table_width = -(-ctx_bucket // cache.block_size)
+        self.table_tokens = ctx_bucket      # a block-table row holds the pages of this many tokens
         self.sizes = [a.size for a in first.arrays]
         self.offsets, total = [], 0
         for n in self.sizes:
@@ -286,7 +285,7 @@ class DecodeGraphs:
             self._sightings[key] = seen
             if seen < record_at:
                 return None
-        step = step_arrays(entries, runner.cache, table_width=-(-bucket // runner.cache.block_size))
+        step = step_arrays(entries, runner.cache, table_tokens=bucket)
         if state is None:
             self._make_room()
             state = _PortionGraph(runner, step, bucket)

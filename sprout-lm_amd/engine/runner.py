@@ -123,7 +123,7 @@ class ModelRunner:
         if kind == "paged":
             group = self.cache.groups[g]
             return CacheSlotView(call.writes, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
-                                 slot_mapping=ctx.group_slots[g], page_size=self.cache.block_size)
+                                 slot_mapping=ctx.group_slots[g], page_size=group.page_tokens)
         group = self.cache.state_groups[g]
         return CacheSlotView(call.writes, state=group.data[index])
 
@@ -152,7 +152,7 @@ class ModelRunner:
         """The checks of `validate` for a step of single tokens, in one pass.  An entry whose token is still
         on the device (`sources[i] >= 0`) brings None in its place."""
         seen = set()
-        bs, limit, vocab = self.cache.block_size, self.max_positions, self.vocab_size
+        sizes, limit, vocab = [g.page_tokens for g in self.cache.groups], self.max_positions, self.vocab_size
         for i, e in enumerate(entries):
             seq, token = e.seq, e.tokens[0]
             if token is None and sources is not None and sources[i] >= 0:
@@ -168,9 +168,8 @@ class ModelRunner:
                 raise ValueError(f"Position {seq.length} is beyond the model's {limit} positions.")
             if e.want[0] != 0:
                 raise ValueError("Wanted logit places must index the entry's own tokens.")
-            need = seq.length // bs + 1
-            for blocks in seq.blocks:
-                if len(blocks) < need:
+            for bs, blocks in zip(sizes, seq.blocks):
+                if len(blocks) < seq.length // bs + 1:
                     raise ValueError("Pages for the entry's tokens were not reserved before the step.")
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:

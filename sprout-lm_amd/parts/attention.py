@@ -20,7 +20,8 @@ class Attention(Mixer):
     hidden, heads, kv_heads, head_dim: sizes.  qkv_bias / out_bias: whether the projections carry
     biases.  position: a PositionEncoding part.  window: None for all earlier keys, else how many
     of the latest keys a query sees.  own_kv False: the layer has no k/v projections and reads the
-    cache slot that another layer writes.
+    cache slot that another layer writes.  page_tokens: tokens in a page of this layer's cache (None: the
+    cache manager's own page size; else a divisor of it), e.g. small pages for a short window.
 
     The three input projections are kept as one matrix [(heads + 2 kv_heads) * head_dim, hidden]
     (rows of q, then k, then v), concatenated when the tensors are bound.
@@ -31,7 +32,8 @@ class Attention(Mixer):
     graph_safe_portions = True
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
-                 out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None):
+                 out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None,
+                 page_tokens: int | None = None):
         try:      # sizes no kernel takes are refused when the part is built, not at the first step
             ops.check_attention_sizes(heads, kv_heads, head_dim)
         except ops.KernelError as error:
@@ -40,11 +42,11 @@ class Attention(Mixer):
             raise ConfigError(f"A rotation needs an even head size, got {head_dim}.")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.position, self.qkv_bias, self.out_bias = position, qkv_bias, out_bias
-        self.window, self.own_kv = window, own_kv
+        self.window, self.own_kv, self.page_tokens = window, own_kv, page_tokens
         self.scale = 1.0 / math.sqrt(head_dim) if scale is None else scale
 
     def cache_spec(self):
-        return PagedKVSpec(self.kv_heads, self.head_dim, self.window)
+        return PagedKVSpec(self.kv_heads, self.head_dim, self.window, self.page_tokens)
 
     def cache_elements_per_token(self) -> int:
         return 2 * self.kv_heads * self.head_dim

@@ -21,8 +21,8 @@ def invariants(cache: CacheManager):
                 if page != FREED:
                     held[page] = held.get(page, 0) + 1
         for entry in cache._prefixes.values():
-            if entry.pages[gi] is not None:
-                held[entry.pages[gi]] = held.get(entry.pages[gi], 0) + 1
+            for page in entry.pages[gi] or ():
+                held[page] = held.get(page, 0) + 1
         free = list(g.pool._free)
         assert len(free) == len(set(free)), "a page is on the free list twice"
         for page in range(g.pool.num_pages):
@@ -232,7 +232,8 @@ def test_state_slots_are_per_request_and_come_back():
 @pytest.mark.parametrize("seed", range(12))
 def test_random_orders_never_lose_or_double_a_page(seed):
     rng = random.Random(seed)
-    specs = [[FULL], [FULL, WINDOWED], [WINDOWED], [PagedKVSpec(1, 8, window=5), FULL, WINDOWED]][seed % 4]
+    specs = [[FULL], [FULL, WINDOWED], [WINDOWED], [PagedKVSpec(1, 8, window=5), FULL, WINDOWED],
+             [FULL, PagedKVSpec(2, 16, window=10, page_tokens=2)], [PagedKVSpec(2, 16, page_tokens=1), WINDOWED]][seed % 6]
     cache = CacheManager(specs, block_size=4, num_blocks=12, max_sequences=5, prefix_caching=True)
     live = []
     prompts = [[rng.randrange(3) for _ in range(rng.randrange(1, 30))] for _ in range(8)]
@@ -258,4 +259,33 @@ def test_random_orders_never_lose_or_double_a_page(seed):
         seq.release()
     cache.clear_prefixes()
     invariants(cache)
-    assert cache.free_pages() == [12] * len(cache.groups)
+    assert cache.free_pages() == [g.pool.num_pages for g in cache.groups]
+
+
+def test_groups_with_pages_of_their_own_size():
+    """A windowed group asks for pages of 2 tokens in a cache whose pages (and prefix unit) are 8: it holds the same
+    number of tokens in four times the pages, gives back what its window of 10 has passed two tokens at a time,
+    and shares a prefix as four of its pages beside one of the other group's."""
+    small = PagedKVSpec(2, 16, window=10, page_tokens=2)
+    cache = CacheManager([FULL, small], block_size=8, num_blocks=6, max_sequences=3)
+    assert [g.page_tokens for g in cache.groups] == [8, 2] and [g.pool.num_pages for g in cache.groups] == [6, 24]
+    with pytest.raises(ValueError, match="do not divide"):
+        CacheManager([PagedKVSpec(2, 16, page_tokens=3)], block_size=8, num_blocks=4, max_sequences=1)
+    tokens = list(range(30))
+    a = cache.create()
+    assert cache.pages_needed(a, 17) == [3, 9]
+    feed(cache, a, tokens, portion=3)
+    assert [len(b) for b in a.blocks] == [4, 15]
+    # length 30: the next token reads keys from 21 on; pages of 2 before key 20 are back
+    assert a.blocks[1][:10] == [FREED] * 10 and FREED not in a.blocks[1][10:]
+    invariants(cache)
+    b = cache.reuse_prefix(tokens[:26])
+    # three units of 8 are offered (one token must stay); b computes position 24 next and reads keys from 15 on,
+    # which lie in the second unit: all of its four small pages come along, the first unit's do not
+    assert b.length == 24 and b.blocks[0] == a.blocks[0][:3]
+    assert b.blocks[1][:4] == [FREED] * 4 and FREED not in b.blocks[1][4:12] and len(b.blocks[1]) == 12
+    invariants(cache)
+    feed(cache, b, tokens[:26], portion=1)
+    assert b.blocks[1][:8] == [FREED] * 8                 # at length 26 keys before 17 are passed: pages up to key 15
+    a.release(); b.release(); cache.clear_prefixes()
+    assert cache.free_pages() == [6, 24]

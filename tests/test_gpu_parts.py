@@ -659,17 +659,19 @@ def register_windowed_toy():
         heads: int = 0
         kv_heads: int = 0
         window: int = 0
+        window_page: int = 0       # tokens in a page of the windowed layer's cache
         eps: float = 0.0
         theta: float = 0.0
 
         @classmethod
         def from_dict(cls, raw):
-            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "window", "eps", "theta")})
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "window", "window_page",
+                                              "eps", "theta")})
 
         def to_dict(self):
             return {"architectures": [self.architecture], "model_type": "toy_window", "hidden": self.hidden,
                     "inner": self.inner, "vocab": self.vocab, "heads": self.heads, "kv_heads": self.kv_heads,
-                    "window": self.window, "eps": self.eps, "theta": self.theta}
+                    "window": self.window, "window_page": self.window_page, "eps": self.eps, "theta": self.theta}
 
     def build(cfg):
         hd = cfg.hidden // cfg.heads
@@ -678,7 +680,7 @@ def register_windowed_toy():
             "hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.kv_heads, "head_dim": hd,
             "position": PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": cfg.theta}), **extra}, prefix)
         mlp = lambda prefix: PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner}, prefix)
-        mixers = [attention("l0.attn."), attention("l1.attn.", window=cfg.window)]
+        mixers = [attention("l0.attn."), attention("l1.attn.", window=cfg.window, page_tokens=cfg.window_page)]
         layers = [LayerPlan("pre_norm", {"mixer_norm": norm(f"l{i}.n1."), "mixer": m, "ffn_norm": norm(f"l{i}.n2."),
                                          "ffn": mlp(f"l{i}.mlp.")}) for i, m in enumerate(mixers)]
         return ModelPlan("ToyWindowForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
@@ -689,7 +691,8 @@ def register_windowed_toy():
     S.register_architecture("ToyWindowForCausalLM", WindowConfig, build, model_types=("toy_window",))
 
 
-WINDOWED = dict(model_type="toy_window", hidden=64, inner=96, vocab=89, heads=4, kv_heads=2, window=10, eps=1e-6, theta=1e4)
+WINDOWED = dict(model_type="toy_window", hidden=64, inner=96, vocab=89, heads=4, kv_heads=2, window=10, window_page=4,
+                eps=1e-6, theta=1e4)
 
 
 def plain_windowed_logits(w, tokens, store):
@@ -712,22 +715,25 @@ def plain_windowed_logits(w, tokens, store):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype):
-    """A model with a layer that keeps every key and one with a window of 10 (pages of 4): a second request takes
-    over the pages of a shared prefix in both cache groups, in the windowed one only those its window still covers
-    (the earlier places of its block table say `given back`), and computes on from there; a third one after the
-    first two have ended finds the pages in the cache alone.  Every logit row of the later requests against the
-    plain implementation, which knows no cache."""
+@pytest.mark.parametrize("window_page", [4, 2])
+def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype, window_page):
+    """A model with a layer that keeps every key and one with a window of 10 (pages of 4; the windowed layer's own
+    pages of 4 or of 2 tokens): a second request takes over the pages of a shared prefix in both cache groups, in
+    the windowed one only those its window still covers (the earlier places of its block table say `given back`),
+    and computes on from there; a third one after the first two have ended finds the pages in the cache alone.
+    Every logit row of the later requests against the plain implementation, which knows no cache."""
     register_windowed_toy()
     import sprout_lm_amd as S
     from sprout_lm_amd.cache import FREED
     from sprout_lm_amd.engine import ModelRunner, StepEntry
     from sprout_lm_amd.weights import write_model_folder
     folder = str(tmp_path / "windowed")
-    write_model_folder(folder, S.config_from_dict(WINDOWED), seed=17, dtype=torch.bfloat16, std=0.15)
+    write_model_folder(folder, S.config_from_dict(dict(WINDOWED, window_page=window_page)), seed=17, dtype=torch.bfloat16,
+                       std=0.15)
     runner = ModelRunner.from_folder(folder, dtype, block_size=4, num_blocks=40, max_sequences=3, prefix_caching=True)
     cache = runner.cache
-    assert cache.prefix_caching and [g.spec.window for g in cache.groups] == [None, 10]
+    per = 4 // window_page                                # the windowed group's pages in four tokens
+    assert cache.prefix_caching and [(g.spec.window, g.page_tokens) for g in cache.groups] == [(None, 4), (10, window_page)]
     from safetensors.torch import load_file
     w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
     store = P.bf16_round if dtype == "bfloat16" else P.f32
@@ -758,15 +764,15 @@ def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype):
     worst = run("a", a, [3] * 20)                       # portions shorter than the window: every page is offered live
     b = cache.reuse_prefix(requests["b"])
     assert b.length == 24 and b.blocks[0] == a.blocks[0][:6]
-    # b computes position 24 next and reads keys from 15 on: pages 3..5 of the windowed group, the ones a wrote
-    assert b.blocks[1][:3] == [FREED] * 3 and FREED not in b.blocks[1][3:6]
-    assert set(b.blocks[1][3:6]) <= {e.pages[1] for e in cache._prefixes.values()}
+    # b computes position 24 next and reads keys from 15 on: the windowed group's pages of tokens 12..23, which a wrote
+    assert b.blocks[1][:3 * per] == [FREED] * (3 * per) and FREED not in b.blocks[1][3 * per:6 * per]
+    assert set(b.blocks[1][3 * per:6 * per]) <= {p for e in cache._prefixes.values() for p in e.pages[1] or ()}
     worst = max(worst, run("b", b, [5, 1, 1, 9, 4]))
     a.release(); b.release()
     c = cache.reuse_prefix(requests["c"])               # only the cache holds the pages now
-    assert c.length == 20 and c.blocks[1][:2] == [FREED] * 2 and FREED not in c.blocks[1][2:5]
+    assert c.length == 20 and c.blocks[1][:2 * per] == [FREED] * (2 * per) and FREED not in c.blocks[1][2 * per:5 * per]
     worst = max(worst, run("c", c, [2, 7, 6]))
     c.release()
     cache.clear_prefixes()
-    assert cache.free_pages() == [40, 40]
+    assert cache.free_pages() == [40, 40 * per]
     print(f"windowed prefix sharing {dtype}: worst {worst:.2f} of the bound")
