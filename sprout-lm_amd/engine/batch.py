@@ -58,6 +58,32 @@ class Workspace:
         return flat[:n].view(shape)
 
 
+class KeptWorkspace(Workspace):
+    """Scratch tensors for recorded graphs that share them: a graph holds the addresses it was recorded with, so
+    a tensor is never freed or moved; a request that none of a name's tensors can hold gets a further one."""
+
+    def __init__(self, device):
+        super().__init__(device)
+        self._kept: dict[tuple[str, torch.dtype], list[torch.Tensor]] = {}
+
+    def get(self, name: str, shape, dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= s
+        fitting = [t for t in self._kept.get((name, dtype), ()) if t.numel() >= n]
+        if fitting:
+            flat = min(fitting, key=lambda t: t.numel())
+        else:
+            if self.frozen:
+                raise RuntimeError(f"Workspace buffer {name!r} would grow while a graph is recorded.")
+            flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._kept.setdefault((name, dtype), []).append(flat)
+        return flat[:n].view(shape)
+
+    def nbytes(self) -> int:
+        return sum(t.numel() * t.element_size() for kept in self._kept.values() for t in kept)
+
+
 class StepContext:
     def __init__(self, workspace: Workspace, act_dtype, attention_kind: int = 0):
         self.workspace = workspace

@@ -26,7 +26,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from .batch import CacheSlotView, StepContext, Workspace, context_from, step_arrays
+from .batch import CacheSlotView, KeptWorkspace, StepContext, Workspace, context_from, step_arrays
 
 
 def _bucket(n: int, floor: int = 1) -> int:
@@ -180,9 +180,10 @@ class _DecodeGraph:
 class _PortionGraph:
     """Static buffers and the recorded graph of one step shape with portions of prompts in it."""
 
-    def __init__(self, runner, first, ctx_bucket: int):
+    def __init__(self, runner, first, ctx_bucket: int, workspace):
         self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
         cache = runner.cache
+        self.last_used = 0
         self.table_tokens = ctx_bucket      # a block-table row holds the pages of this many tokens
         self.sizes = [a.size for a in first.arrays]
         self.offsets, total = [], 0
@@ -193,9 +194,11 @@ class _PortionGraph:
         self.host_np = self.host.numpy()
         self.dev = torch.zeros(max(total, 4), dtype=torch.int32, device=runner.device)
         views = [self.dev[o:o + n].view(a.shape) for o, n, a in zip(self.offsets, self.sizes, first.arrays)]
-        # buffers of its own: a graph holds their addresses.  The longest context is known to the kernels as its
-        # bucket only (how a long walk is shared out follows it), and the step has no values on the host.
-        self.ctx = context_from(first, views, len(cache.groups), Workspace(runner.device), runner.dtype,
+        # Descriptors of its own; the scratch tensors are shared with the other recorded steps of this kind (they
+        # run one after the other on one stream, and `workspace` never frees or moves a tensor).  The longest
+        # context is known to the kernels as its bucket only (how a long walk is shared out follows it), and the
+        # step has no values on the host.
+        self.ctx = context_from(first, views, len(cache.groups), workspace, runner.dtype,
                                 runner.attention_kind, max_decode_ctx=ctx_bucket, max_ctx=ctx_bucket)
         self.ctx.host = {}
         self.copied = None
@@ -252,11 +255,17 @@ def _record(state) -> None:
 class DecodeGraphs:
     def __init__(self, runner, max_graphs: int = 32):
         self.runner = weakref.proxy(runner)
-        self.graphs: dict[tuple, object] = {}     # decode steps: (sequences, context bucket); others: (shape, bucket)
+        self.graphs: dict[tuple, _DecodeGraph] = {}      # (sequences, context bucket) -> recorded decode step
         self.max_graphs = max_graphs
         self.replays = 0
+        # steps with portions of prompts: (tokens and wanted places request by request, context bucket) -> graph
+        self.portion_graphs: dict[tuple, _PortionGraph] = {}
+        self.max_portion_graphs = max(4, max_graphs // 2)
+        self.keep_recent = 64          # a graph used within this many such steps is not given up for a new shape
         self.portion_replays = 0
+        self.portion_steps = 0
         self._sightings: dict[tuple, int] = {}
+        self._portion_workspace = None
 
     def _context_bucket(self, longest: int) -> int:
         return min(_bucket(longest, 256), -(-self.runner.max_positions // 256) * 256)
@@ -277,7 +286,8 @@ class DecodeGraphs:
             return None
         bucket = self._context_bucket(max(e.seq.length + len(e.tokens) for e in entries))
         key = (tuple((len(e.tokens), len(e.want)) for e in entries), bucket)
-        state = self.graphs.pop(key, None)
+        self.portion_steps += 1
+        state = self.portion_graphs.pop(key, None)
         if state is None:
             seen = self._sightings.get(key, 0) + 1
             if len(self._sightings) > 4096:
@@ -285,11 +295,21 @@ class DecodeGraphs:
             self._sightings[key] = seen
             if seen < record_at:
                 return None
+            if len(self.portion_graphs) >= self.max_portion_graphs:
+                # Recording costs as much as dozens of steps: the least recently used graph makes room only if it
+                # has not run for a while.  (Shapes that take turns faster than that run eagerly.)
+                oldest = next(iter(self.portion_graphs))
+                if self.portion_steps - self.portion_graphs[oldest].last_used < self.keep_recent:
+                    return None
+                torch.cuda.current_stream().synchronize()
+                self.portion_graphs.pop(oldest)
         step = step_arrays(entries, runner.cache, table_tokens=bucket)
         if state is None:
-            self._make_room()
-            state = _PortionGraph(runner, step, bucket)
-        self.graphs[key] = state
+            if self._portion_workspace is None:
+                self._portion_workspace = KeptWorkspace(runner.device)
+            state = _PortionGraph(runner, step, bucket, self._portion_workspace)
+        self.portion_graphs[key] = state
+        state.last_used = self.portion_steps
         state.fill(step)
         state.launch()
         self.portion_replays += 1

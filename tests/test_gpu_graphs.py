@@ -207,5 +207,32 @@ def test_recorded_portions_at_real_layer_sizes_cross_a_context_bucket(tmp_path):
         ran.append(g)
         worst = max(worst, w)
     assert ran == [False, True, True, True, False, True, True, True]
-    assert set(runner._graphs.graphs) == {(((64, 1),), 256), (((64, 1),), 512)}
+    assert set(runner._graphs.portion_graphs) == {(((64, 1),), 256), (((64, 1),), 512)}
     print(f"recorded portions at real layer sizes: worst {worst:.2f} of the bound")
+
+
+def test_a_recorded_step_is_given_up_only_when_it_has_not_run_for_a_while(tmp_path):
+    """Recording a step costs as much as dozens of steps.  With room for two recorded shapes, a third shape that
+    keeps coming runs eagerly while both graphs are in use, and takes the place of the one that has not run for
+    `keep_recent` steps; the logits are the plain implementation's whichever way a step runs."""
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.engine.graphs import DecodeGraphs
+    folder = H.make_model_folder(str(tmp_path), "A")
+    vocab = H.CONFIGS["A"]["vocab_size"]
+    runner = ModelRunner.from_folder(folder, "bfloat16", block_size=16, num_blocks=24, max_sequences=2)
+    runner._graphs = DecodeGraphs(runner)
+    runner._graphs.max_portion_graphs, runner._graphs.keep_recent = 2, 6
+    tokens = {"a": H.random_tokens(vocab, 120, 900)}
+
+    def run(n):
+        """A fresh request fed its first `n` tokens as one step; whether that step ran from a graph."""
+        seqs, fed = {"a": runner.cache.create()}, {"a": 0}
+        from_graph, _ = fed_step(runner, seqs, tokens, fed, {"a": n}, folder, "bfloat16", f"{n} tokens")
+        seqs["a"].release()
+        return from_graph
+
+    assert [run(5), run(5), run(7), run(7)] == [False, True, False, True]       # two shapes recorded
+    assert [run(9), run(9), run(9)] == [False, False, False]                      # no room: both are in recent use
+    assert [run(5) for _ in range(6)] == [True] * 6                               # the graph of 7 tokens grows old
+    assert run(9) and set(k[0][0][0] for k in runner._graphs.portion_graphs) == {5, 9}
+    assert not run(7)                                                             # its graph is gone; 5 and 9 are recent
