@@ -3,11 +3,12 @@
 // them (64 elements at a time, interleaved), so that even a matrix with few rows keeps many loads in
 // flight, and their partial sums meet in LDS.  What can be folded in:
 //   prologue  NORM   the activations are RMSNorm(residual) * weight, computed by the block itself from the
-//                    float32 residual (up to 16 tokens).  The scale 1 / sqrt(mean(x^2) + eps) of a token is one
-//                    number, so it is applied to the sums after the product: the lanes turn x * weight into
-//                    matrix-core operands as the rows arrive, add up x^2 on the side, and the squares meet in
-//                    the same exchange through LDS as the partial products.  Nothing waits for the norm: the
-//                    residual rows travel together with the weights.
+//                    float32 residual, 16 tokens a block (further tokens are further blocks along the grid's
+//                    z).  A lane asks for its token's values of the wave's steps before the weights; the
+//                    squares of the four waves meet in LDS while the weights are on their way, and the lanes
+//                    then turn (x * scale) * weight into matrix-core operands in registers: the numbers that
+//                    the norm kernel would have stored, so a token's activations do not depend on which of
+//                    the two ways a step takes.
 //   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
 //             kEpiRope   the block's rows are rotation partners (dims d and d + head/2 of one head): two tiles
 //                        of 16, or (NT = 1, up to 16 tokens) one tile of 8 dimensions and their 8 partners, so
@@ -490,7 +491,7 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
 // many blocks it holds, so the matrix is cut for the CU that gets the most: bytes a block asks for (its gate and
 // up rows, and the activations, which every block reads whole) times blocks per CU, rounded up.  4,864 inner
 // columns: 256 blocks of 19 instead of 304 of 16, of which 48 CUs held two.  More than 16 columns (three tiles)
-// only with up to 16 tokens.
+// only where a block takes one tile of tokens (up to 16 tokens, or the norm prologue).
 static int silu_rows_per_block(int T, int I, int K, bool norm) {
   const int most = (T <= 16 || norm) ? 24 : 16;
   const int token_tiles = norm ? (T + 15) / 16 : 1;

@@ -86,9 +86,10 @@ class Attention(Mixer):
                 and ops.fused_supported(ops.FUSED_ROPE, T, self.w_qkv.shape[0], self.hidden, self.head_dim,
                                         self.position.rotary_dim, norm, variant=self.position.pairing))
 
-    # Folding the norm into the projection kernel (up to 16 tokens) saves a launch; the kernel asks for the
+    # Folding the norm into the projection kernel (up to 64 tokens) saves a launch; the kernel asks for the
     # residual rows before its weights, so the norm is computed while the weights are on their way.  Every
-    # block of the kernel normalises the rows by itself, so this pays for narrow models only (the library says).
+    # block of the kernel normalises its 16 tokens' rows by itself and every tile of 16 tokens reads the weights
+    # again, so this pays for narrow models and few blocks only (the library says: `ops.fused_norm_pays`).
     fuse_input_norm = True
 
     def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
