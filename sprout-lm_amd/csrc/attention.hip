@@ -69,7 +69,9 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                             const int32_t* tiles, int n_tiles, int tile_q, int max_tile_ctx, int mean_tile_walk,
                             const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
                             int64_t workspace_floats, void* out, int nq,
-                            int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind) {
+                            int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind,
+                            int scores) {
+  SP_REQUIRE(scores == 0, "sp_attention: no kernel for score stage %d (0 = the scaled product alone)", scores);
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
   SP_REQUIRE(hd > 0 && hd <= 256, "sp_attention: head size %d is outside 1..256", hd);
@@ -120,7 +122,8 @@ extern "C" int sp_attention_decode_project(void* stream, const void* q, int q_st
                                            const int32_t* q_start, const int32_t* ctx_len, const int32_t* decode_seqs,
                                            int n_decode, int max_decode_ctx, float* workspace, int64_t workspace_floats,
                                            const void* w_o, float* residual, int hidden, int nq, int nkv, int hd,
-                                           int page_size, int num_pages, int window, float scale) {
+                                           int page_size, int num_pages, int window, float scale, int scores) {
+  SP_REQUIRE(scores == 0, "sp_attention_decode_project: no kernel for score stage %d (0 = the scaled product alone)", scores);
   SP_REQUIRE(sp_attention_decode_project_takes(hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden),
              "sp_attention_decode_project: hd=%d page=%d heads=%d/%d sequences=%d context=%d hidden=%d is not taken",
              hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden);

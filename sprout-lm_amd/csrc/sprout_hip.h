@@ -74,12 +74,14 @@ int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions, 
 int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind, int* plan);
 int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
                                       int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx);
+// scores: what stands between q . k and the softmax, numbered like the variants above: 0 = the scaled product and
+// nothing else (the one the kernels have; a cap, a bias or sinks would be further numbers, refused until written).
 int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                  const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                  const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, int tile_q,
                  int max_tile_ctx, int mean_tile_walk, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                  float* workspace, int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size,
-                 int num_pages, int window, float scale, int kernel_kind);
+                 int num_pages, int window, float scale, int kernel_kind, int scores);
 
 // A step of one-query sequences only (bfloat16): attention with the output projection folded into the merge
 // of the key chunks: residual[q_start[seq], :] += attention(seq) . w_o^T with w_o [hidden, nq * hd] bfloat16
@@ -92,7 +94,7 @@ int sp_attention_decode_project(void* stream, const void* q, int q_stride, const
                                 const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                                 float* workspace, int64_t workspace_floats, const void* w_o, float* residual,
                                 int hidden, int nq, int nkv, int hd, int page_size, int num_pages, int window,
-                                float scale);
+                                float scale, int scores);
 
 // out[t, i] = act(gu[t, i]) * gu[t, I + i]
 int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation);

@@ -63,6 +63,7 @@ def _ptr(t):
 # kernels; anything else is refused (KernelError) before a launch.
 ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox")
 GATE_ACTIVATIONS = {"silu": 0}
+SCORE_STAGES = {"scaled_dot": 0}         # what stands between q . k and the softmax: the scale and nothing else
 MAX_HEAD_DIM = 256                       # the largest head size any attention kernel takes
 
 
@@ -242,7 +243,7 @@ def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: in
 
 def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
               batch: AttentionBatch, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
-              workspace=None, kind: int = 0, project=None) -> bool:
+              workspace=None, kind: int = 0, project=None, scores: str = "scaled_dot") -> bool:
     """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h).
 
     `workspace(n)` must return a float32 device tensor of at least n elements (default: a new one).
@@ -251,6 +252,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     residual += attention . w_o^T, `out` is left untouched and True is returned; otherwise False, and the
     projection is the caller's.
     """
+    scores_code = variant_code(SCORE_STAGES, scores, "score stage")
     for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
     T = out.shape[0]
@@ -302,7 +304,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                 block_tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
                 _ptr(decode) if decode is not None else None, n_decode, max_decode_ctx, _ptr(ws), need, w_o.data_ptr(),
                 residual.data_ptr(), hidden, nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
-                float(scale)))
+                float(scale), scores_code))
             return True
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
@@ -310,7 +312,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  n_tiles, tile_q, max_tile_ctx, int(batch.mean_walk), _ptr(decode) if n_decode else None, n_decode,
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
-                                 float(scale), kind))
+                                 float(scale), kind, scores_code))
     return False
 
 

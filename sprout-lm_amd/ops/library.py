@@ -24,11 +24,11 @@ def _declare(lib):
                           c_int, c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
                          c_int, c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_float, c_int],
+                         c_int, c_int, c_float, c_int, c_int],
         "sp_attention_decode_project_takes": [c_int] * 7,
         "sp_attention_decode_project": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void,
                                         c_int, c_int, c_void, c_i64, c_void, c_void, c_int, c_int, c_int, c_int, c_int,
-                                        c_int, c_int, c_float],
+                                        c_int, c_int, c_float, c_int],
         "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
         "sp_fused_supported": [c_int] * 8,
         "sp_fused_norm_pays": [c_int] * 3,

@@ -33,11 +33,14 @@ class Attention(Mixer):
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position, qkv_bias: bool = True,
                  out_bias: bool = False, window: int | None = None, own_kv: bool = True, scale: float | None = None,
-                 page_tokens: int | None = None):
+                 page_tokens: int | None = None, scores: str = "scaled_dot"):
         try:      # sizes no kernel takes are refused when the part is built, not at the first step
             ops.check_attention_sizes(heads, kv_heads, head_dim)
         except ops.KernelError as error:
             raise ConfigError(str(error)) from None
+        if scores not in ops.SCORE_STAGES:      # a cap, a bias or sinks between q . k and the softmax: a kernel variant
+            raise ConfigError(f"No attention kernel for score stage {scores!r}; there are kernels for: {sorted(ops.SCORE_STAGES)}.")
+        self.scores = scores
         if head_dim % 2 and getattr(position, "rotary_dim", 0):
             raise ConfigError(f"A rotation needs an even head size, got {head_dim}.")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
@@ -115,7 +118,7 @@ class Attention(Mixer):
         if ops.attention(q, q_stride, cache.k, cache.v, cache.block_tables, ctx.attention, attn, self.heads,
                          self.kv_heads, self.head_dim, self.window, self.scale,
                          workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
-                         kind=ctx.attention_kind, project=project):
+                         kind=ctx.attention_kind, project=project, scores=self.scores):
             return
         ops.gemm(attn, self.w_o, residual, bias=self.b_o, accumulate=True)
 

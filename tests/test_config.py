@@ -92,3 +92,7 @@ def test_sizes_that_no_kernel_takes_are_refused_when_the_parts_are_built():
     with pytest.raises(ops.KernelError, match="rotation pairing 'interleaved'"):
         ops.kernels.variant_code(ops.ROTARY_PAIRINGS, "interleaved", "rotation pairing")
     assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0}
+    with pytest.raises(ConfigError, match="score stage 'soft_cap'"):
+        PartPlan("mixer", "attention", {"hidden": 32, "heads": 2, "kv_heads": 1, "head_dim": 16, "scores": "soft_cap",
+                                        "position": PartPlan("position", "none", {"head_dim": 16})}).make()
+    assert ops.SCORE_STAGES == {"scaled_dot": 0}

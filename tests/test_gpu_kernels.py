@@ -448,6 +448,14 @@ def test_variants_without_a_kernel_are_refused_by_the_library_itself():
     assert not ops.fused_supported(ops.FUSED_SILU, 8, 9728, 896, variant="gelu")
     with pytest.raises(ops.KernelError, match="activation 'relu'"):
         ops.silu_mul(gu, out, activation="relu")
+    # what stands between q . k and the softmax is such a parameter of the attention entry points
+    q = torch.zeros(1, 32, device=DEV)
+    kp, vp = torch.zeros(2, 1, 8, 16, device=DEV), torch.zeros(2, 1, 16, 8, device=DEV)
+    batch = ops.AttentionBatch.build([1], [1], DEV)
+    tables = torch.zeros(1, 1, dtype=torch.int32, device=DEV)
+    assert ops.attention(q, 32, kp, vp, tables, batch, torch.zeros_like(q), 2, 1, 16, None, 0.25) is False
+    with pytest.raises(ops.KernelError, match="score stage 'soft_cap'"):
+        ops.attention(q, 32, kp, vp, tables, batch, torch.zeros_like(q), 2, 1, 16, None, 0.25, scores="soft_cap")
     torch.cuda.synchronize()
 
 
