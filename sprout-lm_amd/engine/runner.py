@@ -4,6 +4,7 @@ from __future__ import annotations
 import json
 import os
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -138,7 +139,12 @@ class ModelRunner:
             n = len(e.tokens)
             if n == 0:
                 raise ValueError("A step entry brings no tokens.")
-            if any(not isinstance(t, int) or isinstance(t, bool) or t < 0 or t >= self.vocab_size for t in e.tokens):
+            if n > 32:     # a long portion: checked as one array (a list that is not all integers has another kind)
+                ids = np.asarray(e.tokens)
+                bad = ids.dtype.kind not in "iu" or ids.ndim != 1 or int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size
+            else:
+                bad = any(not isinstance(t, int) or isinstance(t, bool) or t < 0 or t >= self.vocab_size for t in e.tokens)
+            if bad:
                 raise ValueError(f"Token ids must be integers in [0, {self.vocab_size}).")
             if e.seq.length + n > self.max_positions:
                 raise ValueError(f"Position {e.seq.length + n - 1} is beyond the model's {self.max_positions} positions.")
@@ -179,6 +185,9 @@ class ModelRunner:
         before the call returns; the kernels may still be running on the stream.
         """
         self.validate(entries)
+        return self._step_checked(entries)
+
+    def _step_checked(self, entries: list[StepEntry]) -> torch.Tensor:
         ctx = build_context(entries, self.cache, self.stager, self.workspace, self.dtype, self.attention_kind)
         logits = self.forward(ctx)
         for e in entries:
@@ -197,23 +206,27 @@ class ModelRunner:
             return self.finish_decode(pending)
         if self._sampler is None:
             self._sampler = Sampler(self.device, self.vocab_size)
-        logits = self.step_recorded(entries)
+        self.validate(entries)
+        logits = self._recorded_checked(entries, 2)
         if logits is None:
-            logits = self.step(entries)
+            logits = self._step_checked(entries)
         return self._sampler.sample(logits, params, counters)
 
     def step_recorded(self, entries: list[StepEntry], record_at: int = 2):
         """`step` from a recorded graph of the step's shape, where there is one or the shape has now come
         `record_at` times; None otherwise (nothing has been run then).  The logits lie in the graph's own buffer
         and are overwritten when the same shape runs again."""
-        if not self.use_graphs or not self.record_portions:
+        if not self.use_graphs or not self.record_portions or not self.parts.graph_safe_portions:
+            return None
+        self.validate(entries)
+        return self._recorded_checked(entries, record_at)
+
+    def _recorded_checked(self, entries: list[StepEntry], record_at: int):
+        if not self.use_graphs or not self.record_portions or not self.parts.graph_safe_portions:
             return None
         if self._graphs is None:
             from .graphs import DecodeGraphs
             self._graphs = DecodeGraphs(self)
-        if not self.parts.graph_safe_portions:
-            return None
-        self.validate(entries)
         return self._graphs.portion_step(entries, record_at)
 
     def launch_decode(self, entries: list[StepEntry], params, counters, feed=None):
