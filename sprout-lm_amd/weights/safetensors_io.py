@@ -46,51 +46,77 @@ class TensorInfo:
     end: int
 
 
+def _is_count(value) -> bool:
+    return isinstance(value, int) and not isinstance(value, bool)
+
+
+def _parse_header(path: str, file, size: int) -> tuple[dict, int]:
+    """The JSON header of a safetensors file and the number of bytes before the tensor data."""
+    lead = file.read(8)
+    if len(lead) != 8:
+        raise SafetensorsError(f"{path}: {size} bytes are too few for a safetensors file (8 bytes of header length first).")
+    (length,) = struct.unpack("<Q", lead)
+    if not 0 < length <= MAX_HEADER:
+        raise SafetensorsError(f"{path}: a header of {length} bytes is outside 1..{MAX_HEADER}.")
+    if 8 + length > size:
+        raise SafetensorsError(f"{path}: the header claims {length} bytes, the file has {size - 8} after its first 8.")
+    try:
+        header = json.loads(file.read(length).decode("utf-8"))
+    except (UnicodeDecodeError, json.JSONDecodeError) as error:
+        raise SafetensorsError(f"{path}: the header is not JSON ({error}).") from None
+    if not isinstance(header, dict):
+        raise SafetensorsError(f"{path}: the header is JSON but not an object of tensors.")
+    return header, 8 + length
+
+
+def _tensor_info(path: str, name: str, raw, data_size: int) -> TensorInfo:
+    """One header entry, checked by itself: a known dtype, a shape of positive sizes, and a byte range that holds
+    exactly that many elements inside the data."""
+    if not isinstance(raw, dict):
+        raise SafetensorsError(f"{path}: tensor {name!r} is described by {type(raw).__name__}, not by an object.")
+    dtype, shape, offsets = raw.get("dtype"), raw.get("shape"), raw.get("data_offsets")
+    if dtype not in _DTYPES:
+        raise SafetensorsError(f"{path}: tensor {name!r} has dtype {dtype!r}; this reader takes {sorted(_DTYPES)}.")
+    if not isinstance(shape, list) or not all(_is_count(n) and n > 0 for n in shape):
+        raise SafetensorsError(f"{path}: tensor {name!r} has shape {shape!r}; sizes must be positive integers.")
+    if not isinstance(offsets, list) or len(offsets) != 2 or not all(_is_count(n) for n in offsets):
+        raise SafetensorsError(f"{path}: tensor {name!r} has data_offsets {offsets!r}; two integers are expected.")
+    begin, end = offsets
+    nbytes = _DTYPES[dtype][0]
+    for n in shape:
+        nbytes *= n
+    if begin < 0 or end > data_size or end - begin != nbytes:
+        raise SafetensorsError(f"{path}: tensor {name!r} ({dtype} {shape}) needs {nbytes} bytes, its range "
+                               f"[{begin}, {end}) of {data_size} data bytes does not give them.")
+    return TensorInfo(dtype, tuple(shape), begin, end)
+
+
+def _check_tiling(path: str, entries: dict, data_size: int) -> None:
+    """The tensors' ranges, in order, must tile the data: no byte twice, none unaccounted for."""
+    at = 0
+    for name, info in sorted(entries.items(), key=lambda item: item[1].begin):
+        if info.begin != at:
+            what = "overlaps its predecessor" if info.begin < at else f"leaves bytes {at}..{info.begin - 1} unused"
+            raise SafetensorsError(f"{path}: tensor {name!r} begins at byte {info.begin} and {what}.")
+        at = info.end
+    if at != data_size:
+        raise SafetensorsError(f"{path}: the tensors end at byte {at}, the data at {data_size}.")
+
+
 class SafetensorsFile:
+    """A safetensors file, memory-mapped.  What the header says is checked before any tensor is handed out
+    (the checks of the reference's reader, src/safetensors.ts:26-66)."""
+
     def __init__(self, path: str):
         self.path = path
         size = os.path.getsize(path)
         self._file = open(path, "rb")
         try:
-            prefix = self._file.read(8)
-            if len(prefix) < 8:
-                raise SafetensorsError(f"{path}: truncated safetensors file.")
-            (header_size,) = struct.unpack("<Q", prefix)
-            if header_size <= 0 or header_size > MAX_HEADER or header_size + 8 > size:
-                raise SafetensorsError(f"{path}: invalid safetensors header length {header_size}.")
-            try:
-                parsed = json.loads(self._file.read(header_size).decode("utf-8"))
-            except (UnicodeDecodeError, json.JSONDecodeError):
-                raise SafetensorsError(f"{path}: invalid safetensors header.") from None
-            if not isinstance(parsed, dict):
-                raise SafetensorsError(f"{path}: invalid safetensors header.")
-            data_size = size - 8 - header_size
-            entries: dict[str, TensorInfo] = {}
-            for name, raw in parsed.items():
-                if name == "__metadata__":
-                    continue
-                ok = (isinstance(raw, dict) and raw.get("dtype") in _DTYPES and isinstance(raw.get("shape"), list)
-                      and all(isinstance(n, int) and not isinstance(n, bool) and n > 0 for n in raw["shape"])
-                      and isinstance(raw.get("data_offsets"), list) and len(raw["data_offsets"]) == 2
-                      and all(isinstance(n, int) and not isinstance(n, bool) for n in raw["data_offsets"]))
-                if not ok:
-                    raise SafetensorsError(f"{path}: unsupported or malformed tensor {name!r}.")
-                begin, end = raw["data_offsets"]
-                count = 1
-                for n in raw["shape"]:
-                    count *= n
-                if begin < 0 or end - begin != count * _DTYPES[raw["dtype"]][0] or end > data_size:
-                    raise SafetensorsError(f"{path}: invalid tensor offsets for {name!r}.")
-                entries[name] = TensorInfo(raw["dtype"], tuple(raw["shape"]), begin, end)
-            previous = 0
-            for info in sorted(entries.values(), key=lambda e: e.begin):
-                if info.begin != previous:
-                    raise SafetensorsError(f"{path}: safetensors data contains gaps or overlapping tensors.")
-                previous = info.end
-            if previous != data_size:
-                raise SafetensorsError(f"{path}: safetensors data size does not match its header.")
-            self.entries = entries
-            self._start = 8 + header_size
+            header, self._start = _parse_header(path, self._file, size)
+            data_size = size - self._start
+            self.entries = {name: _tensor_info(path, name, raw, data_size)
+                            for name, raw in header.items() if name != "__metadata__"}
+            _check_tiling(path, self.entries, data_size)
             # a private mapping: nothing is ever written to it, but tensors may then view its pages directly
             self._map = mmap.mmap(self._file.fileno(), 0, access=mmap.ACCESS_COPY) if size else None
         except Exception:
