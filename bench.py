@@ -290,8 +290,11 @@ def main() -> int:
     engine.close()
     del engine
     if not args.no_points and args.second_preset not in ("", "none", args.preset):
-        points.update(second_model_points(args.second_preset, dtype, element, args.batch, args.context, args.prefill_tokens,
-                                          min(args.steps, 24), args.dtype))
+        try:
+            points.update(second_model_points(args.second_preset, dtype, element, args.batch, args.context,
+                                              args.prefill_tokens, min(args.steps, 24), args.dtype))
+        except Exception as error:      # the headline above does not depend on the second model: say so and go on
+            print(f"bench.py: the points at {args.second_preset} sizes were not measured: {error}", file=sys.stderr)
     pressure = None
     if args.pressure:
         pressure = measure_pressure(cfg, dtype, args.batch, 512, 256, args.pressure)
