@@ -771,7 +771,22 @@ def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype, window_page):
     a.release(); b.release()
     c = cache.reuse_prefix(requests["c"])               # only the cache holds the pages now
     assert c.length == 20 and c.blocks[1][:2 * per] == [FREED] * (2 * per) and FREED not in c.blocks[1][2 * per:5 * per]
-    worst = max(worst, run("c", c, [2, 7, 6]))
+    # the last tokens of c one by one through recorded decode steps: block tables of two groups with pages of
+    # different sizes in the graph's static buffers
+    from sprout_lm_amd.sampling import SamplingParams
+    tokens_c, want_c = requests["c"], plain_windowed_logits(w, requests["c"], store)
+    requests["c"] = tokens_c[:-4]
+    worst = max(worst, run("c", c, [2, 7]))
+    requests["c"] = tokens_c
+    for position in range(len(tokens_c) - 4, len(tokens_c)):
+        assert cache.reserve(c, position + 1)
+        pending = runner.launch_decode([StepEntry(c, [tokens_c[position]], [0])], [SamplingParams()], [0])
+        assert pending is not None, "the step did not run from a recorded graph"
+        runner.finish_decode(pending)
+        err = np.abs(pending.logits[0].cpu().numpy() - want_c[position]).max() / (tol * (1 + np.abs(want_c[position]).max()))
+        worst = max(worst, err)
+        assert err <= 1.0, f"c position {position} through a recorded step: {err:.2f} of the bound"
+    assert c.length == len(tokens_c)
     c.release()
     cache.clear_prefixes()
     assert cache.free_pages() == [40, 40 * per]
