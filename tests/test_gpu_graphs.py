@@ -117,6 +117,34 @@ def test_recorded_steps_at_real_layer_sizes_match_plain(tmp_path):
     print(f"recorded steps at real layer sizes: worst {worst:.2f} of the bound")
 
 
+def test_recorded_steps_of_forty_sequences_at_real_layer_sizes(tmp_path):
+    """Between 17 and 64 sequences the decode kernels take the tokens in tiles along the grid (the q/k/v product
+    with the norm folded in by 16, the accumulating products by 32) and the output head runs on the pipelined
+    tiles: two layers with the sizes of Qwen2.5-0.5B, forty sequences at different positions (a recorded step of
+    64 rows, 24 of them padding), every logit row against the plain side."""
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.weights import write_model_folder
+    raw = dict(PRESETS["qwen2.5-0.5b"], num_hidden_layers=2)
+    folder = str(tmp_path / "half_b")
+    write_model_folder(folder, S.config_from_dict(raw), seed=13, dtype=torch.bfloat16, std=0.02)
+    n, steps = 40, 3
+    rng = np.random.default_rng(8)
+    tokens = {r: H.random_tokens(raw["vocab_size"], int(rng.integers(2, 40)) + steps, 200 + r) for r in range(n)}
+    runner = ModelRunner.from_folder(folder, "bfloat16", block_size=16, num_blocks=4 * n, max_sequences=n)
+    seqs = {r: runner.cache.create() for r in range(n)}
+    fed = {r: len(tokens[r]) - steps for r in range(n)}
+    entries = []
+    for r in range(n):
+        assert runner.cache.reserve(seqs[r], fed[r])
+        entries.append(StepEntry(seqs[r], tokens[r][:fed[r]], []))
+    assert runner.step(entries).shape[0] == 0
+    worst = decode_through_graphs(runner, seqs, tokens, fed, steps, folder, "forty sequences")
+    assert list(runner._graphs.graphs) == [(64, 256)]
+    print(f"recorded steps of {n} sequences at real layer sizes: worst {worst:.2f} of the bound")
+
+
 def fed_step(runner, seqs, tokens, fed, takes, folder, dtype, label, recorded=True):
     """One step in which request r brings its next `takes[r]` tokens and wants the logits of the last of them,
     through `step_recorded` (eagerly where that declines); every wanted row against the plain side.
