@@ -452,10 +452,11 @@ static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int split
 }
 
 // Whether the q/k/v product takes one gathered tile a block: with up to 16 tokens, where twice the blocks pull
-// the rows twice as fast; with more, every block reads all the activations again, which then costs more
-// (28 heads of 128 at a width of 3,584, 64 tokens: 36 us against about 20).  Head sizes that 32 does not divide
-// have no other way.
-static bool rope_one_tile(int T, int hd) { return T <= 16 || hd % 32 != 0; }
+// the rows twice as fast, as long as every block still finds a CU of its own (36 heads of 128: 288 blocks of
+// one tile against 144 of two, 14.0 against 13.1 us at 8 tokens, 16.2 against 13.9 at 16); with more tokens,
+// every block reads all the activations again, which then costs more (28 heads of 128 at a width of 3,584,
+// 64 tokens: 36 us against about 20).  Head sizes that 32 does not divide have no other way.
+static bool rope_one_tile(int T, int hd, int N = 0) { return hd % 32 != 0 || (T <= 16 && N / 16 <= 256); }
 // With the norm prologue a block takes 16 tokens whatever their number (further tiles of tokens are further
 // blocks, each normalising its own rows): one gathered tile a block as long as all the blocks find a CU of
 // their own, two tiles (half the blocks) beyond that, where a CU would have to pull for two blocks.
@@ -474,7 +475,7 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
     }
     return launch_fused<1, EPI, true>(s, a, blocks, splits);
   } else {
-    if (EPI == kEpiRope && rope_one_tile(a.T, a.hd)) {
+    if (EPI == kEpiRope && rope_one_tile(a.T, a.hd, a.N)) {
       if constexpr (EPI == kEpiRope) {
         if (a.T <= 16) return launch_fused<1, EPI, false, 1>(s, a, blocks, splits);
         if (a.T <= 32) return launch_fused<2, EPI, false, 1>(s, a, blocks, splits);
@@ -624,7 +625,7 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.page_shift = -1;
   if (page_size > 0 && (page_size & (page_size - 1)) == 0)
     for (a.page_shift = 0; (1 << a.page_shift) < page_size;) ++a.page_shift;
-  const bool one_tile = residual ? rope_one_tile_normed(T, N, hd) : rope_one_tile(T, hd);
+  const bool one_tile = residual ? rope_one_tile_normed(T, N, hd) : rope_one_tile(T, hd, N);
   const int blocks = (nq + 2 * nkv) * (hd / (one_tile ? 16 : 32));
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
