@@ -483,10 +483,12 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
       }
     }
     if (a.T <= 16) return launch_fused<1, EPI, false>(s, a, blocks, splits);
-    // More than 32 tokens: tiles of 32 along the grid's z.  A block that takes all 64 reads twice the activations
-    // for the same weight rows (64 tokens, 896 x 896: 4.9 us against 3.9; 896 x 4,864 the same either way), and
-    // tiles of 16 read the weights four times (4.4 and 9.1 us).
-    return launch_fused<2, EPI, false>(s, a, blocks, splits);
+    // More than 32 tokens: tiles of 32 along the grid's z while the matrix is small.  A block that takes all 64
+    // reads twice the activations for the same weight rows (64 tokens, 896 x 896: 4.9 us against 3.9; 896 x 4,864
+    // the same either way), tiles of 16 read the weights four times (4.4 and 9.1 us), and a large matrix is read
+    // once whatever that costs in activations (4,608 x 3,584: 20 us with all 64 tokens a block, 28 in tiles of 32).
+    if (a.T <= 32 || size_t(a.N) * a.K <= (size_t(2) << 20)) return launch_fused<2, EPI, false>(s, a, blocks, splits);
+    return launch_fused<4, EPI, false>(s, a, blocks, splits);
   }
 }
 
