@@ -174,7 +174,8 @@ int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const
     // Few rows.  Large accumulating products stream their weights through the pipelined tiles (K split over
     // blocks), whatever the number of tokens (3,584 x 18,944: 25.4 against 27.7 us at one token, 26.0 against 29.7
     // at 8, 26.6 against 32.8 at 16); the others split K between the waves of a block.
-    if (mode == kAccumulate && size_t(N) * K >= (size_t(6) << 20) && gemm_pipe_takes(T, N, K))
+    // (up to 16 tokens only where the matrix is that large: 3,584 x 3,584 at 8 tokens is 8.2 us fused, 8.8 tiled)
+    if (mode == kAccumulate && size_t(N) * K >= (size_t(T > 16 ? 6 : 32) << 20) && gemm_pipe_takes(T, N, K))
       return gemm_bf16_pipe(s, a, w, bias_dtype, bias, mode, out, T, N, K);
     if ((N + 15) / 16 < 2048) return gemm_decode_plain(s, a, w, bias_dtype, bias, mode, out, T, N, K);
     // Very wide (the output head): rows streamed per wave up to 16 tokens; with more, the streaming kernel stops
