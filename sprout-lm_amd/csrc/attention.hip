@@ -7,8 +7,8 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
-                      float* workspace);
-size_t attention_generic_workspace_floats(int n_tiles, int nq, int hd, int max_tile_ctx);
+                      float* workspace, bool single);
+size_t attention_generic_workspace_floats(int n_tiles, int nq, int nkv, int hd, int max_tile_ctx, bool single);
 bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
@@ -58,8 +58,8 @@ static int64_t workspace_floats_of(int hd, int page_size, int nq, int nkv, int n
 
 extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
                                                  int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx) {
-  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind))
-    return (int64_t)attention_generic_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
+  if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind))   // (n_decode == n_tiles: every sequence brings one query)
+    return (int64_t)attention_generic_workspace_floats(n_tiles, nq, nkv, hd, max_tile_ctx, n_decode > 0 && n_decode == n_tiles);
   return workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, n_tiles, max_tile_ctx);
 }
 
@@ -80,19 +80,22 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   int plan[2];
   sp_attention_plan(dtype, hd, page_size, nq, nkv, kernel_kind, plan);
   SP_REQUIRE(tile_q == plan[0], "sp_attention: tiles were built for %d queries, the kernel takes %d", tile_q, plan[0]);
-  SP_REQUIRE(plan[1] == 0 || n_decode == 0, "sp_attention: this kernel takes every sequence in the tile list");
+  // a kernel that takes every sequence in its tile list may be told that each brings one query: n_decode == n_tiles
+  SP_REQUIRE(plan[1] == 0 || n_decode == 0 || (n_decode == n_tiles && !decode_seqs),
+             "sp_attention: this kernel takes every sequence in the tile list");
   SP_REQUIRE(n_tiles >= 0 && n_decode >= 0 && (n_tiles == 0 || tiles), "sp_attention: missing tile list");
   hipStream_t s = (hipStream_t)stream;
   if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind)) {
     if (n_tiles == 0) return 0;
     SP_REQUIRE(max_tile_ctx >= 0, "sp_attention: negative context length");
-    const int64_t need = (int64_t)attention_generic_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
+    const bool single = n_decode > 0 && n_decode == n_tiles;
+    const int64_t need = (int64_t)attention_generic_workspace_floats(n_tiles, nq, nkv, hd, max_tile_ctx, single);
     SP_REQUIRE(need == 0 || (workspace && workspace_floats >= need),
                "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
                (long long)need);
     return attention_generic(s, dtype, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len,
                              ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale,
-                             max_tile_ctx, need ? workspace : nullptr);
+                             max_tile_ctx, need ? workspace : nullptr, single);
   }
   SP_REQUIRE(max_decode_ctx >= 0 && max_decode_ctx <= max_blocks * page_size,
              "sp_attention: decode context %d exceeds the block tables", max_decode_ctx);

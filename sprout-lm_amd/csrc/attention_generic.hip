@@ -3,6 +3,8 @@
 // One block works on 16 queries of one sequence and one head, walking the keys 32 at a time with a
 // running maximum and sum (all float32).  Keys are always walked from a multiple of 32, so the order
 // of the sums at a position does not depend on how the tokens were cut into steps.
+// GROUPED (a step in which every sequence brings one query): the 16 rows of a block are the query heads of one
+// key/value head instead (groups of up to 16), so a group's keys and values are fetched once, not once per head.
 // A step of few tiles and long contexts (decoding) would leave most of the chip idle: the keys are then
 // shared out in chunks (a multiple of 32 keys each) over gridDim.z blocks, which leave their maxima, sums
 // and unnormalised outputs in a workspace, and a second kernel joins them in the order of the chunks.
@@ -74,7 +76,7 @@ __device__ __forceinline__ void store_tile(float* KVs, int hd, const Divider& by
   }
 }
 
-template <typename T, int MAXD>  // MAXD = ceil(hd / 16) upper bound
+template <typename T, int MAXD, bool GROUPED>  // MAXD = ceil(hd / 16) upper bound
 __global__ __launch_bounds__(256) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
@@ -91,22 +93,26 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   constexpr int PS = AK + 1;
 
   const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
-  const int h = blockIdx.y;
+  const int G = nq / nkv;
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
-  const int nvalid = min(AQ, qlen - q_off);
+  // rows: GROUPED the heads blockIdx.y * G .. + G - 1 of the tile's one query; else the tile's queries of head blockIdx.y
+  const int nvalid = GROUPED ? (qlen - q_off > 0 ? G : 0) : min(AQ, qlen - q_off);
   if (nvalid <= 0) return;
   const int pos0 = ctx - qlen + q_off;
 
   for (int i = threadIdx.x; i < AQ * hd; i += 256) {
     const int r = i / hd, d = i % hd;
-    Qs[r * kv_stride + d] = r < nvalid ? to_float(q[size_t(qs + q_off + r) * q_stride + h * hd + d]) : 0.f;
+    const size_t at = GROUPED ? size_t(qs + q_off) * q_stride + (blockIdx.y * G + r) * hd + d
+                              : size_t(qs + q_off + r) * q_stride + blockIdx.y * hd + d;
+    Qs[r * kv_stride + d] = r < nvalid ? to_float(q[at]) : 0.f;
   }
 
   const int r = threadIdx.x / 16, c16 = threadIdx.x % 16;
-  const int my_pos = pos0 + r;
+  const int h = GROUPED ? blockIdx.y * G + min(r, G - 1) : blockIdx.y;      // this thread's row's head
+  const int my_pos = GROUPED ? pos0 : pos0 + r;
   TileSource src;
   src.bt = block_tables + size_t(seq) * max_blocks;
-  src.nkv = nkv; src.g = h / (nq / nkv); src.hd = hd; src.page_size = page_size; src.num_pages = num_pages;
+  src.nkv = nkv; src.g = GROUPED ? blockIdx.y : blockIdx.y / G; src.hd = hd; src.page_size = page_size; src.num_pages = num_pages;
   src.k_end = pos0 + nvalid;  // one past the last visible key of the tile
   src.k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int n_chunks = gridDim.z, first_key = blockIdx.z * chunk;   // this block's keys: first_key .. + chunk - 1
@@ -182,8 +188,10 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   }
   if (n_chunks > 1) {
     // [tile][row][head][chunk][hd + 2]: the unnormalised output, the maximum and the sum; rows past the tile's
-    // queries and chunks without a visible key leave zeros and a maximum of -inf
-    float* p = part + (((size_t(blockIdx.x) * AQ + r) * nq + h) * n_chunks + blockIdx.z) * (hd + 2);
+    // queries and chunks without a visible key leave zeros and a maximum of -inf.  (GROUPED: the one query is
+    // row 0 of its tile; rows past the group's heads have nothing to leave.)
+    if (GROUPED && r >= nvalid) return;
+    float* p = part + (((size_t(blockIdx.x) * AQ + (GROUPED ? 0 : r)) * nq + h) * n_chunks + blockIdx.z) * (hd + 2);
 #pragma unroll
     for (int i = 0; i < MAXD; ++i) {
       const int d = c16 + 16 * i;
@@ -194,7 +202,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   }
   if (r < nvalid) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* o = out + size_t(qs + q_off + r) * (size_t(nq) * hd) + h * hd;
+    T* o = out + size_t(qs + q_off + (GROUPED ? 0 : r)) * (size_t(nq) * hd) + h * hd;
 #pragma unroll
     for (int i = 0; i < MAXD; ++i) {
       const int d = c16 + 16 * i;
@@ -233,18 +241,21 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
 
 // How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
 // and long contexts; at most 32 chunks of at least 256 keys, whole groups of 32 keys each.
-static void generic_chunks(int n_tiles, int nq, int max_tile_ctx, int* n_chunks, int* chunk) {
+static void generic_chunks(int n_tiles, int rows_of_blocks, int max_tile_ctx, int* n_chunks, int* chunk) {
   *n_chunks = 1;
   *chunk = 0;
-  if (n_tiles * nq >= 1024 || max_tile_ctx < 512) return;
+  if (n_tiles * rows_of_blocks >= 1024 || max_tile_ctx < 512) return;
   const int keys = max(256, ((max_tile_ctx + 31) / 32 + AK - 1) / AK * AK);
   *chunk = keys;
   *n_chunks = (max_tile_ctx + keys - 1) / keys;
 }
 
-size_t attention_generic_workspace_floats(int n_tiles, int nq, int hd, int max_tile_ctx) {
+// Whether a step in which every sequence brings one query (`single`) takes the grouped form of the kernel.
+static bool generic_grouped(bool single, int nq, int nkv) { return single && nkv > 0 && nq % nkv == 0 && nq / nkv > 1 && nq / nkv <= AQ; }
+
+size_t attention_generic_workspace_floats(int n_tiles, int nq, int nkv, int hd, int max_tile_ctx, bool single) {
   int n_chunks, chunk;
-  generic_chunks(n_tiles, nq, max_tile_ctx, &n_chunks, &chunk);
+  generic_chunks(n_tiles, generic_grouped(single, nq, nkv) ? nkv : nq, max_tile_ctx, &n_chunks, &chunk);
   return n_chunks > 1 ? size_t(n_tiles) * AQ * nq * n_chunks * (hd + 2) : 0;
 }
 
@@ -253,19 +264,25 @@ int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const v
                              const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                              const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
                              void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
-                             float scale, int max_tile_ctx, float* workspace) {
+                             float scale, int max_tile_ctx, float* workspace, bool single) {
   const size_t lds = sizeof(float) * (size_t(AQ + AK) * (hd + 1) + AQ * (AK + 1));
+  const bool grouped = generic_grouped(single, nq, nkv);
   int n_chunks, chunk;
-  generic_chunks(n_tiles, nq, max_tile_ctx, &n_chunks, &chunk);
+  generic_chunks(n_tiles, grouped ? nkv : nq, max_tile_ctx, &n_chunks, &chunk);
   if (!workspace) n_chunks = 1;
-  dim3 grid(n_tiles, nq, n_chunks);
-#define SP_ATT(MAXD)                                                                                        \
-  attention_generic_kernel<T, MAXD><<<grid, 256, lds, s>>>(                                                 \
-      (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len, \
-      ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk)
-  if (hd <= 64) SP_ATT(4);
-  else if (hd <= 128) SP_ATT(8);
-  else SP_ATT(16);
+  dim3 grid(n_tiles, grouped ? nkv : nq, n_chunks);
+#define SP_ATT(MAXD)                                                                                           \
+  if (grouped)                                                                                                 \
+    attention_generic_kernel<T, MAXD, true><<<grid, 256, lds, s>>>(                                            \
+        (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len,  \
+        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk);         \
+  else                                                                                                         \
+    attention_generic_kernel<T, MAXD, false><<<grid, 256, lds, s>>>(                                           \
+        (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len,  \
+        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk)
+  if (hd <= 64) { SP_ATT(4); }
+  else if (hd <= 128) { SP_ATT(8); }
+  else { SP_ATT(16); }
 #undef SP_ATT
   if (check_launch("sp_attention (generic)")) return 1;
   if (n_chunks == 1) return 0;
@@ -278,17 +295,17 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
-                      float* workspace) {
+                      float* workspace, bool single) {
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,
-                                           num_pages, window, scale, max_tile_ctx, workspace);
+                                           num_pages, window, scale, max_tile_ctx, workspace, single);
   return launch_attention_generic<bf16_t>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                           q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages,
-                                          window, scale, max_tile_ctx, workspace);
+                                          window, scale, max_tile_ctx, workspace, single);
 }
 
 }  // namespace sprout

@@ -275,6 +275,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     decode, n_decode = (None, 0) if every else batch.lists["decode_seqs"]
     _ints(tiles, 2 * n_tiles, "tiles")
     max_decode_ctx = batch.max_decode_ctx if n_decode else 0
+    # a kernel that takes every sequence in its tile list is told when each of them brings one query
+    one_query_each = every and n_tiles == n_seqs and batch.lists[f"tiles_multi_{tile_q}"][1] == 0
     if n_decode:
         if decode is not None:         # None: sequences 0 .. n_decode - 1
             _ints(decode, n_decode, "decode_seqs")
@@ -284,6 +286,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         if max_decode_ctx > block_tables.shape[1] * page_size:
             raise KernelError("attention: a decode context is longer than its block table")
     max_tile_ctx = min(batch.max_ctx, block_tables.shape[1] * page_size) if n_tiles else 0
+    if one_query_each:
+        n_decode = n_tiles
     need = library().sp_attention_workspace_floats(_code(q, "q"), hd, page_size, nq, nkv, kind, n_decode, max_decode_ctx,
                                                    n_tiles, max_tile_ctx)
     ws = None
@@ -291,7 +295,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         ws = workspace(need) if workspace is not None else torch.empty(need, dtype=torch.float32, device=q.device)
         if ws.dtype != torch.float32 or ws.numel() < need:
             raise KernelError("attention: workspace too small")
-    if project is not None and kind == 0 and n_tiles == 0 and n_decode and need and q.dtype == torch.bfloat16:
+    if project is not None and kind == 0 and n_tiles == 0 and n_decode and need and q.dtype == torch.bfloat16 and not every:
         w_o, residual = project
         hidden = w_o.shape[0]
         if (w_o.dtype == torch.bfloat16 and w_o.is_contiguous() and tuple(w_o.shape) == (hidden, nq * hd)
@@ -309,7 +313,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
                                  batch.q_len.data_ptr(), batch.ctx_len.data_ptr(), _ptr(tiles) if n_tiles else None,
-                                 n_tiles, tile_q, max_tile_ctx, int(batch.mean_walk), _ptr(decode) if n_decode else None, n_decode,
+                                 n_tiles, tile_q, max_tile_ctx, int(batch.mean_walk),
+                                 _ptr(decode) if n_decode and decode is not None else None, n_decode,
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
                                  float(scale), kind, scores_code))

@@ -276,6 +276,21 @@ def test_attention_mixed_batches(nq, nkv, hd, page, batch, dtype, kind):
     assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,page", [(4, 2, 64, 16), (14, 2, 64, 16), (16, 1, 32, 8), (5, 5, 48, 16), (20, 1, 16, 4),
+                                            (6, 3, 80, 12)])
+@pytest.mark.parametrize("window", [None, 300])
+def test_attention_one_query_each_on_the_float32_kernel(dtype, nq, nkv, hd, page, window):
+    """A step in which every sequence brings one query: the float32-arithmetic kernel then takes the query heads of
+    a key/value head as the rows of a block (groups of 2 to 16; one head a group and groups of 20 go the other way),
+    with the keys of long contexts shared out in chunks and joined.  One far key of the second sequence stands out."""
+    seqs = [(700, 1), (2049, 1), (33, 1), (1, 1), (512, 1), (257, 1)]
+    got, want = run_attention(dtype, nq, nkv, hd, page, seqs, window=window, kind=1, spike=(1, 1800), seed=nq)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    assert not np.isnan(got).any()
+    assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
 @pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
 @pytest.mark.parametrize("window", [1, 5, 16, 33, 100])
 def test_attention_window_edges(dtype, kind, window):
