@@ -41,9 +41,11 @@ __device__ __forceinline__ void wait_loads_then_barrier() {
 }
 
 // A block of WAVES_M x WAVES_N waves, each with WM x WN tiles of 32 x 32: BM = 32 WM WAVES_M tokens by
-// BN = 32 WN WAVES_N weight rows.
+// BN = 32 WN WAVES_N weight rows.  Blocks of up to four waves ask for the registers of two waves a SIMD: with
+// all 512 to itself the compiler keeps the accumulators in one half of them and copies all of them to the
+// other half and back around every turn of the ring.
 template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_pipe_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2 : 1)) void gemm_pipe_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
                                                         const TB* __restrict__ bias, void* __restrict__ out, int T,
                                                         int N, int K, int k_per_split, RopeArgs rope) {
   constexpr int NW = WAVES_M * WAVES_N;
