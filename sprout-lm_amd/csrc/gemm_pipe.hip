@@ -16,13 +16,14 @@ bool gemm_pipe_takes(int T, int N, int K) {
 struct PipeShape { int bm, bn, per_cu; float step_us; };
 static const PipeShape kPipeShapes[] = {
     {256, 256, 1, 2.05f},   // 8 waves, 2 stages
-    {256, 128, 1, 1.37f},   // 4 waves, 3 stages
+    {256, 128, 1, 1.25f},   // 4 waves, 3 stages
     {128, 128, 1, 0.72f},   // 4 waves, 4 stages
     {64, 64, 2, 0.41f},     // 4 waves, 4 stages
     {64, 256, 1, 0.75f},    // 8 waves, 3 stages (few tokens)
     {64, 128, 2, 0.7f},     // 4 waves, 3 stages (few tokens)
     {384, 256, 1, 3.3f},    // 8 waves, 2 stages (all of the LDS): where it saves a round of blocks
     {64, 64, 2, 0.45f},     // 2 waves with two tile columns each, 4 stages (few tokens: most blocks)
+    {256, 160, 1, 2.0f},    // 4 waves in a column, five tile columns each, 3 stages: where 256 x 256 leaves CUs idle
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -54,17 +55,21 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     }
     return;
   }
-  for (int c : {0, 1, 2, 3, 5, 6}) {
+  for (int c : {0, 1, 2, 3, 5, 6, 8}) {
     // (64 x 128 fills the chip where 128 x 128 leaves CUs idle and 64 x 64 needs a second round: 2,048 tokens,
     // 1,152 rows, K = 896: 14.8 us against 17.2 and 15.1)
     if (c == 3 && paired) continue;   // one tile column a wave: no lane holds both of a pair
+    // 256 x 160: an odd number of tile columns a wave pairs nothing either.  (2,048 tokens, K = 3,584: 4,608 rows
+    // make 232 blocks instead of 144 of 256 x 256, 83 us against 91; 5,120 rows at K = 27,648 make 256 instead of 160,
+    // 607 us against 658; with a short K its blocks cost more than their share, 57 us against 51 at 9,728 rows, K = 896)
+    if (c == 8 && paired) continue;
     const PipeShape& p = kPipeShapes[c];
     // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
     // and blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
     // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180
     // on 256 x 256, for all the round of blocks they save; with one token tile, 264 tokens, 55,296 rows,
     // K = 5,120, their 253 us are the best there is)
-    const float step_us = steps <= 16 ? p.step_us : c == 5 ? 0.8f : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.step_us;
+    const float step_us = steps <= 16 ? p.step_us : c == 5 ? 0.8f : c == 8 ? 1.4f : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.step_us;
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;

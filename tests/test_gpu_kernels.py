@@ -24,6 +24,8 @@ def bf16(x):
                                    (700, 896, 4864), (65, 2100, 448),
                                    (300, 4608, 3584), (40, 3584, 18944), (24, 3584, 3584), (520, 9728, 896),
                                    (1100, 13400, 192),    # blocks of 384 tokens save a round of blocks
+                                   # blocks of 256 x 160 fill the chip where 256 x 256 do not; the second with K in two
+                                   (2000, 5000, 1088), (777, 5000, 3584),
                                    # few tiles and a long K
                                    (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
