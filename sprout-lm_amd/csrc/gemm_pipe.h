@@ -220,8 +220,8 @@ inline int pipe_shape(hipStream_t s, const void* x, const void* w, const void* b
   pipe_choice(T, N, K, mode == kAccumulate, &shape, &splits);
   switch (shape) {
     case 0: return launch_pipe<4, 2, 2, 4, 2, TB>(s, x, w, bias, mode, out, T, N, K, splits);
-    case 1: return launch_pipe<4, 2, 2, 2, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
-    case 2: return launch_pipe<2, 2, 2, 2, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
+    case 1: return launch_pipe<2, 2, 4, 2, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
+    case 2: return launch_pipe<1, 2, 4, 2, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 4: return launch_pipe<1, 2, 2, 4, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 5: return launch_pipe<1, 2, 2, 2, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 6: return launch_pipe<6, 2, 2, 4, 2, TB>(s, x, w, bias, mode, out, T, N, K, splits);

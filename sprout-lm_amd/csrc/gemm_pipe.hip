@@ -13,17 +13,20 @@ bool gemm_pipe_takes(int T, int N, int K) {
 
 // Tile shapes of the pipelined kernel, largest first, with what was measured of them on a full chip:
 // microseconds per step of 64 along K and block, blocks per CU (LDS), and bytes a block fetches per step.
-struct PipeShape { int bm, bn, per_cu; float step_us; };
+struct PipeShape { int bm, bn, per_cu; float short_us, long_us; };   // a step of a walk of up to 16 steps, of a longer one
 static const PipeShape kPipeShapes[] = {
-    {256, 256, 1, 2.05f},   // 8 waves, 2 stages
-    {256, 128, 1, 1.25f},   // 4 waves, 3 stages
-    {128, 128, 1, 0.72f},   // 4 waves, 4 stages
-    {64, 64, 2, 0.41f},     // 4 waves, 4 stages
-    {64, 256, 1, 0.75f},    // 8 waves, 3 stages (few tokens)
-    {64, 128, 2, 0.7f},     // 4 waves, 3 stages (few tokens)
-    {384, 256, 1, 3.3f},    // 8 waves, 2 stages (all of the LDS): where it saves a round of blocks
-    {64, 64, 2, 0.45f},     // 2 waves with two tile columns each, 4 stages (few tokens: most blocks)
-    {256, 160, 1, 2.0f},    // 4 waves in a column, five tile columns each, 3 stages: where 256 x 256 leaves CUs idle
+    {256, 256, 1, 2.05f, 2.05f},   // 8 waves, 2 stages
+    {256, 128, 1, 1.4f, 1.05f},    // 8 waves, 3 stages (on 4 waves of 128 x 64 sums each: 1.25 us)
+    {128, 128, 1, 0.72f, 0.64f},   // 8 waves, 4 stages (on 4 waves: 0.72 us)
+    {64, 64, 2, 0.41f, 0.41f},     // 4 waves, 4 stages
+    {64, 256, 1, 0.75f, 0.75f},    // 8 waves, 3 stages (few tokens)
+    // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
+    {64, 128, 2, 0.7f, 0.8f},      // 4 waves, 3 stages (few tokens)
+    {384, 256, 1, 3.3f, 3.3f},     // 8 waves, 2 stages (all of the LDS): where it saves a round of blocks
+    {64, 64, 2, 0.45f, 0.45f},     // 2 waves with two tile columns each, 4 stages (few tokens: most blocks)
+    // 4 waves in a column, five tile columns each, 3 stages: where 256 x 256 leaves CUs idle; with a short K its
+    // blocks cost more than their share (9,728 rows, K = 896: 57 us against 51)
+    {256, 160, 1, 2.0f, 1.4f},
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -48,7 +51,7 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
         const int rounds = (tiles * sp + slots - 1) / slots;
         // a CU pulls about 30 GB/s of weight rows, however many blocks it holds: the CU with the most blocks
         const float pull_us = float((tiles * sp + 255) / 256) * float(p.bn) * float(K / sp) * 2.f / 30e3f;
-        float t = fmaxf(fmaxf(stream_us, pull_us), rounds * float((steps + sp - 1) / sp) * p.step_us) + 2.0f;
+        float t = fmaxf(fmaxf(stream_us, pull_us), rounds * float((steps + sp - 1) / sp) * p.short_us) + 2.0f;
         if (sp > 1) t += 2.7e-6f * float(T) * float(N) * sp;
         if (t < best) { best = t; *shape = c; *splits = sp; }
       }
@@ -64,12 +67,11 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     // 607 us against 658; with a short K its blocks cost more than their share, 57 us against 51 at 9,728 rows, K = 896)
     if (c == 8 && paired) continue;
     const PipeShape& p = kPipeShapes[c];
-    // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
-    // and blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
+    // blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
     // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180
     // on 256 x 256, for all the round of blocks they save; with one token tile, 264 tokens, 55,296 rows,
     // K = 5,120, their 253 us are the best there is)
-    const float step_us = steps <= 16 ? p.step_us : c == 5 ? 0.8f : c == 8 ? 1.4f : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.step_us;
+    const float step_us = steps <= 16 ? p.short_us : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.long_us;
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;

@@ -10,12 +10,12 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
   int shape, splits;
   pipe_choice(T, 2 * I, K, false, &shape, &splits, true);
   if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
   if (shape == 7) return launch_pipe_mode<1, 2, 2, 1, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  return launch_pipe_mode<2, 2, 2, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  return launch_pipe_mode<1, 2, 4, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
 }
 
 // q, k, v = x . w^T + bias with w [(nq + 2 nkv) * hd, K]; q and k heads rotated; q to q_out [T, nq * hd], k and v
@@ -25,14 +25,14 @@ static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const 
                      const RopeArgs& rope) {
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
-  if (shape == 1) return launch_pipe_mode<4, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
-  if (shape == 2) return launch_pipe_mode<2, 2, 2, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
+  if (shape == 2) return launch_pipe_mode<1, 2, 4, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   set_error("sp_qkv_rope_cache: no rotating epilogue for %d tokens, %d rows, K = %d", T, N, K);
   return 1;
 }
 
-// Taken where the plain product would run on blocks of 256 x 128, 128 x 128 or 64 x 128 (4 waves, two tile columns each).  Blocks of 64 x 64 have one tile
+// Taken where the plain product would run on blocks of 256 x 128, 128 x 128 or 64 x 128 (two tile columns a wave).  Blocks of 64 x 64 have one tile
 // column per wave (no lane holds both of a pair), and with few tokens they fill the chip better than anything
 // larger (256 tokens at 14 + 2 + 2 heads of 64: 7.6 us and a rotation kernel of 5 against 17).  The blocks of
 // 8 waves hold 128 sums per lane, all the registers a lane has there: the epilogue's own would be spilled
