@@ -549,6 +549,17 @@ def _normed(res, w, eps):
                                               (2, 1, 80, 160, 4), (5, 1, 64, 320, 8), (3, 3, 128, 384, 16)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
+    check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm)
+
+
+# 28 + 4 + 4 heads of 128: the rotating epilogue on blocks of 256 x 128 (1,024 tokens) and of 128 x 128 (513 tokens at
+# K = 3,584), eight waves each
+@pytest.mark.parametrize("T,K", [(1024, 264), (1024, 896), (513, 3584)])
+def test_fused_qkv_rope_cache_on_blocks_of_eight_waves(T, K):
+    check_fused_qkv_rope_cache(T, 28, 4, 128, K, 16, False)
+
+
+def check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     from sprout_lm_amd import ops
     taken = ops.fused_supported(ops.FUSED_ROPE, T, (nq + 2 * nkv) * hd, K, hd, hd, norm)
     rng = np.random.default_rng(T * 7 + hd)
@@ -604,7 +615,8 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
 
 @pytest.mark.parametrize("T,I,K", [(t_, i_, k_) for t_ in [1, 8, 16, 33, 64, 65, 200, 513]
                                    for i_, k_ in [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)]]
-                         + [(1100, 6700, 128), (2048, 4864, 896)])   # the last two: blocks of 384 tokens
+                         + [(1100, 6700, 128), (2048, 4864, 896),   # blocks of 384 tokens
+                            (1024, 2432, 264), (200, 1000, 3584)])  # blocks of 256 x 128 and 128 x 128 on eight waves
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
