@@ -18,7 +18,7 @@ static const PipeShape kPipeShapes[] = {
     {256, 256, 1, 2.05f, 2.05f},   // 8 waves, 2 stages
     {256, 128, 1, 1.4f, 1.05f},    // 8 waves, 3 stages (on 4 waves of 128 x 64 sums each: 1.25 us)
     {128, 128, 1, 0.72f, 0.64f},   // 8 waves, 4 stages (on 4 waves: 0.72 us)
-    {64, 64, 2, 0.41f, 0.41f},     // 4 waves, 4 stages
+    {64, 64, 2, 0.41f, 0.5f},      // 4 waves, 4 stages
     {64, 256, 1, 0.75f, 0.75f},    // 8 waves, 3 stages (few tokens)
     // two blocks of 64 x 128 on a CU get in each other's way on a long K (measured at 56 and 296 steps)
     {64, 128, 2, 0.7f, 0.8f},      // 4 waves, 3 stages (few tokens)
@@ -27,6 +27,11 @@ static const PipeShape kPipeShapes[] = {
     // 4 waves in a column, five tile columns each, 3 stages: where 256 x 256 leaves CUs idle; with a short K its
     // blocks cost more than their share (9,728 rows, K = 896: 57 us against 51)
     {256, 160, 1, 2.0f, 1.4f},
+    // 64 x 128 on 8 waves of one tile each, 3 stages; two on a CU take as long as one after the other.  Many
+    // tokens by few weight rows: 2,048 tokens, 896 rows, K = 4,864: 33.9 us against 37.0 on 4 waves and 37.6 on
+    // 64 x 64; 1,024 tokens with K in two 22.6 against 23.6 and 23.4; below that 64 x 64 is ahead
+    // (512 tokens: 16.5 against 15.8, 256: 14.7 against 12.3)
+    {64, 128, 1, 0.45f, 0.42f},
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -58,7 +63,7 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     }
     return;
   }
-  for (int c : {0, 1, 2, 3, 5, 6, 8}) {
+  for (int c : {0, 1, 2, 3, 5, 6, 8, 9}) {
     // (64 x 128 fills the chip where 128 x 128 leaves CUs idle and 64 x 64 needs a second round: 2,048 tokens,
     // 1,152 rows, K = 896: 14.8 us against 17.2 and 15.1)
     if (c == 3 && paired) continue;   // one tile column a wave: no lane holds both of a pair
@@ -66,6 +71,7 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     // make 232 blocks instead of 144 of 256 x 256, 83 us against 91; 5,120 rows at K = 27,648 make 256 instead of 160,
     // 607 us against 658; with a short K its blocks cost more than their share, 57 us against 51 at 9,728 rows, K = 896)
     if (c == 8 && paired) continue;
+    if (c == 9 && (paired || T < 1024)) continue;   // one tile a wave
     const PipeShape& p = kPipeShapes[c];
     // blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
     // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180

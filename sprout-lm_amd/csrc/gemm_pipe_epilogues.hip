@@ -25,6 +25,7 @@ static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const 
                      const RopeArgs& rope) {
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
+  if (shape == 9) shape = 5;
   if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 2) return launch_pipe_mode<1, 2, 4, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
@@ -41,7 +42,9 @@ bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
   if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
-  return shape == 1 || shape == 2 || shape == 5;
+  // (64 x 128 on 8 waves has one tile column a wave; the rotation then runs on 64 x 128 on 4 waves, which still
+  // beats the plain product and a rotation kernel after it)
+  return shape == 1 || shape == 2 || shape == 5 || shape == 9;
 }
 
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,

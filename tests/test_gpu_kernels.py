@@ -26,6 +26,8 @@ def bf16(x):
                                    (1100, 13400, 192),    # blocks of 384 tokens save a round of blocks
                                    # blocks of 256 x 160 fill the chip where 256 x 256 do not; the second with K in two
                                    (2000, 5000, 1088), (777, 5000, 3584),
+                                   # many tokens by few rows: 64 x 128 on eight waves; the second with K in four
+                                   (1100, 900, 1088), (2000, 130, 2432),
                                    # few tiles and a long K
                                    (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
