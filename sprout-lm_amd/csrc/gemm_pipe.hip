@@ -28,10 +28,10 @@ static const PipeShape kPipeShapes[] = {
     // blocks cost more than their share (9,728 rows, K = 896: 57 us against 51)
     {256, 160, 1, 2.0f, 1.4f},
     // 64 x 128 on 8 waves of one tile each, 3 stages; two on a CU take as long as one after the other.  Many
-    // tokens by few weight rows: 2,048 tokens, 896 rows, K = 4,864: 33.9 us against 37.0 on 4 waves and 37.6 on
-    // 64 x 64; 1,024 tokens with K in two 22.6 against 23.6 and 23.4; below that 64 x 64 is ahead
-    // (512 tokens: 16.5 against 15.8, 256: 14.7 against 12.3)
-    {64, 128, 1, 0.45f, 0.42f},
+    // tokens by few weight rows, with operands that come from memory: 1,024 tokens, 896 rows, K = 4,864 in two:
+    // 25.2 us against 26.3 on 64 x 64 and 30.7 on 128 x 128; 2,048 tokens: 42.7 against 45.8, where 128 x 128 with
+    // K in two takes 37.3; below 1,024 tokens 64 x 64 is ahead (512 tokens: 16.3 against 15.5)
+    {64, 128, 1, 0.45f, 0.52f},
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
