@@ -18,14 +18,32 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
   return launch_pipe_mode<1, 2, 4, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
 }
 
+// The block shape on which the rotating epilogue runs, or -1 where the plain product and a rotation kernel after
+// it do better.  It follows the plain product's choice where that pairs tile columns (256 x 128, 128 x 128,
+// 64 x 128); 64 x 128 on 8 waves has one tile column a wave, and the rotation then runs on 64 x 128 on 4 waves,
+// which still beats the plain product and a rotation kernel after it.  Blocks of 64 x 64 pair nothing either: there
+// 64 x 128 takes the rotation once its blocks fill half of the chip (14 + 2 + 2 heads of 64 at K = 896, 1,024
+// tokens: 14.5 us against 17.6 apart, 512 tokens: 15.2 against 13.8; 28 + 4 + 4 heads of 128 at K = 3,584, 256
+// tokens: 36.5 against 42.5).  The blocks of 256 x 256 hold 128 sums per lane, all the registers a lane has there:
+// the epilogue's own would be spilled (measured at 28 + 4 + 4 heads of 128, 2,048 tokens: 332 us against 106 and a
+// rotation kernel of 18), and 256 x 160 has five tile columns a wave.
+static int rope_shape(int T, int N, int K) {
+  int shape, splits;
+  pipe_choice(T, N, K, false, &shape, &splits);
+  if (shape == 9) shape = 5;
+  if (shape == 3 && ((T + 63) / 64) * ((N + 127) / 128) >= 128) shape = 5;
+  // (and with the rotation 128 x 128 on 8 waves beats 64 x 128 on 4 once its blocks fill half of the chip: 14 + 2 + 2
+  // heads of 64 at K = 896, 2,048 tokens: 20.2 us against 23.0; 1,024 tokens: 19.2 against 14.5)
+  if (shape == 5 && ((T + 127) / 128) * ((N + 127) / 128) >= 128) shape = 2;
+  return shape == 1 || shape == 2 || shape == 5 ? shape : -1;
+}
+
 // q, k, v = x . w^T + bias with w [(nq + 2 nkv) * hd, K]; q and k heads rotated; q to q_out [T, nq * hd], k and v
 // into the paged pools.  Head sizes that are multiples of 64, more than 64 tokens.
 template <typename TB>
 static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const TB* bias, void* q_out, int T, int N, int K,
                      const RopeArgs& rope) {
-  int shape, splits;
-  pipe_choice(T, N, K, false, &shape, &splits);
-  if (shape == 9) shape = 5;
+  const int shape = rope_shape(T, N, K);
   if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 2) return launch_pipe_mode<1, 2, 4, 2, 4, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
   if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kRope, TB>(s, 1, x, w, bias, q_out, T, N, K, K, rope);
@@ -33,18 +51,8 @@ static int pipe_rope(hipStream_t s, const uint16_t* x, const uint16_t* w, const 
   return 1;
 }
 
-// Taken where the plain product would run on blocks of 256 x 128, 128 x 128 or 64 x 128 (two tile columns a wave).  Blocks of 64 x 64 have one tile
-// column per wave (no lane holds both of a pair), and with few tokens they fill the chip better than anything
-// larger (256 tokens at 14 + 2 + 2 heads of 64: 7.6 us and a rotation kernel of 5 against 17).  The blocks of
-// 8 waves hold 128 sums per lane, all the registers a lane has there: the epilogue's own would be spilled
-// (measured at 28 + 4 + 4 heads of 128, 2,048 tokens: 332 us against 106 and a rotation kernel of 18).
 bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
-  if (!(T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K))) return false;
-  int shape, splits;
-  pipe_choice(T, N, K, false, &shape, &splits);
-  // (64 x 128 on 8 waves has one tile column a wave; the rotation then runs on 64 x 128 on 4 waves, which still
-  // beats the plain product and a rotation kernel after it)
-  return shape == 1 || shape == 2 || shape == 5 || shape == 9;
+  return T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K) && rope_shape(T, N, K) >= 0;
 }
 
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
