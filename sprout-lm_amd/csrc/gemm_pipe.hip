@@ -77,7 +77,9 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180
     // on 256 x 256, for all the round of blocks they save; with one token tile, 264 tokens, 55,296 rows,
     // K = 5,120, their 253 us are the best there is)
-    const float step_us = steps <= 16 ? p.short_us : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.long_us;
+    // (64 x 128 on a short K beside many tokens: 256 tokens, 9,728 rows, K = 896 with the gating: 16.3 us against
+    // 13.8 on 128 x 128)
+    const float step_us = steps <= 16 ? (c == 5 ? 0.8f : p.short_us) : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.long_us;
     const int tiles = ((T + p.bm - 1) / p.bm) * ((N + p.bn - 1) / p.bn), slots = 256 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;
