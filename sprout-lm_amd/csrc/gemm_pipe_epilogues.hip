@@ -55,6 +55,34 @@ bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
   return T > 64 && hd % 64 == 0 && N % hd == 0 && gemm_pipe_takes(T, N, K) && rope_shape(T, N, K) >= 0;
 }
 
+// Rows and columns of every block shape, by its index in gemm_pipe.hip's list.
+static const int kShapeRows[] = {256, 256, 128, 64, 64, 64, 384, 64, 256, 64};
+static const int kShapeCols[] = {256, 128, 128, 64, 256, 128, 256, 64, 160, 128};
+
+}  // namespace sprout
+
+// What the pipelined product would do with T x N x K: kind 0 store, 1 accumulate, 2 gated (N = 2 I rows of w),
+// 3 rotating (head size hd).  plan = {block rows, block columns, splits of K}.  Returns 1 where the pipelined kernel
+// (for kind 3: its rotating epilogue) does not take the product, else 0.  Runs nothing: for tests and tools.
+extern "C" int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan) {
+  using namespace sprout;
+  if (T < 1 || N < 1 || K < 1 || kind < 0 || kind > 3 || !plan || !gemm_pipe_takes(T, N, K)) return 1;
+  int shape, splits = 1;
+  if (kind == 3) {
+    if (!gemm_pipe_rope_takes(T, N, K, hd)) return 1;
+    shape = rope_shape(T, N, K);
+  } else {
+    pipe_choice(T, N, K, kind == 1, &shape, &splits, kind == 2);
+  }
+  if (shape < 0 || shape >= int(sizeof(kShapeRows) / sizeof(kShapeRows[0]))) return 1;
+  plan[0] = kShapeRows[shape];
+  plan[1] = kShapeCols[shape];
+  plan[2] = splits;
+  return 0;
+}
+
+namespace sprout {
+
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
                         const int32_t* positions, const float* inv_freq, const int32_t* slot_mapping, void* k_pool,
                         void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, const float* table) {

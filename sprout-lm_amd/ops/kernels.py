@@ -346,6 +346,20 @@ def fused_norm_pays(T: int, N: int, K: int) -> bool:
     return bool(library().sp_fused_norm_pays(T, N, K))
 
 
+PLAN_STORE, PLAN_ACCUMULATE, PLAN_GATED, PLAN_ROTATING = 0, 1, 2, 3
+
+
+def pipe_plan(kind: int, T: int, N: int, K: int, hd: int = 0):
+    """(block rows, block columns, splits of K) that the tiled product for many tokens would take for T x N x K,
+    or None where that kernel (for PLAN_ROTATING its rotating epilogue) does not take the product.  Runs nothing
+    and needs no GPU."""
+    import ctypes
+    plan = (ctypes.c_int * 3)()
+    if library().sp_pipe_plan(kind, T, N, K, hd, plan):
+        return None
+    return tuple(plan)
+
+
 def _activations(x, residual, norm_weight, K: int, what: str):
     """Checks the two ways activations reach a fused kernel; returns (x ptr, residual ptr, norm dtype, norm ptr, T)."""
     if residual is not None:

@@ -1,0 +1,88 @@
+"""The tiled product's choice of block shape and split, asked of the library without running a kernel (no GPU):
+invariants over a sweep of sizes, and the decisions that measurements on the GPU settled."""
+import itertools
+
+import pytest
+
+from sprout_lm_amd import ops
+
+
+
+@pytest.fixture(autouse=True, scope="module")
+def built_library():
+    """The plan is asked of the compiled library, which needs hipcc where it is not built yet, but no GPU."""
+    try:
+        ops.library()
+    except Exception as e:      # no compiler here: nothing to ask
+        pytest.skip(f"the kernel library cannot be built or loaded here: {e}")
+
+
+SHAPES = {(256, 256), (256, 128), (128, 128), (64, 64), (64, 256), (64, 128), (384, 256), (256, 160)}
+PAIRED = {(256, 256), (256, 128), (128, 128), (64, 256), (64, 128), (384, 256)}    # an even number of tile columns a wave
+ROTATING = {(256, 128), (128, 128), (64, 128)}
+
+
+def sizes():
+    tokens = [1, 5, 16, 17, 64, 65, 128, 200, 256, 264, 512, 777, 1024, 1100, 2048, 4096, 8192]
+    rows = [64, 130, 896, 1152, 3584, 4608, 5120, 9728, 37888, 151936]
+    depth = [64, 192, 896, 1088, 3584, 4864, 5120, 18944, 27648]
+    return itertools.product(tokens, rows, depth)
+
+
+@pytest.mark.parametrize("kind", [ops.PLAN_STORE, ops.PLAN_ACCUMULATE, ops.PLAN_GATED])
+def test_plan_invariants(kind):
+    for T, N, K in sizes():
+        plan = ops.pipe_plan(kind, T, N, K)
+        if N * K * 2 >= 1 << 32:      # a tile's offset into the weights has 32 bits: another kernel's product
+            assert plan is None, (T, N, K)
+            continue
+        assert plan is not None, (T, N, K)          # K is a multiple of 64 everywhere here
+        rows, cols, splits = plan
+        assert (rows, cols) in SHAPES and splits >= 1
+        if kind == ops.PLAN_GATED:
+            # gate and up rows alternate between a wave's tile columns (64 x 64 for up to 64 tokens is two waves with
+            # two tile columns each; for more tokens it is four waves with one)
+            assert (rows, cols) in PAIRED or T <= 64, (T, N, K, plan)
+        if kind != ops.PLAN_ACCUMULATE:
+            assert splits == 1, (T, N, K, plan)                  # only float atomics can join partial sums
+        assert splits == 1 or K // 64 // splits >= 8, (T, N, K, plan)
+        if T > 64:   # few tokens have shapes of their own
+            assert (rows, cols) != (64, 256)
+
+
+def test_products_the_kernel_does_not_take():
+    assert ops.pipe_plan(ops.PLAN_STORE, 300, 100, 70) is None          # K is no multiple of 64
+    assert ops.pipe_plan(ops.PLAN_STORE, 300, 100, 0) is None
+    assert ops.pipe_plan(7, 300, 128, 128) is None
+    assert ops.pipe_plan(ops.PLAN_ROTATING, 64, 1152, 896, 64) is None  # up to 64 tokens: the decode kernels rotate
+    assert ops.pipe_plan(ops.PLAN_ROTATING, 300, 18 * 48, 896, 48) is None   # head sizes that are no multiple of 64
+
+
+def test_rotating_epilogue_shapes():
+    for T, (nq, nkv, hd, K) in itertools.product([65, 128, 256, 264, 512, 1024, 2048, 4096],
+                                                  [(14, 2, 64, 896), (28, 4, 128, 3584), (40, 8, 128, 5120), (4, 4, 128, 256)]):
+        plan = ops.pipe_plan(ops.PLAN_ROTATING, T, (nq + 2 * nkv) * hd, K, hd)
+        assert plan is None or (plan[:2] in ROTATING and plan[2] == 1), (T, nq, nkv, hd, K, plan)
+
+
+def test_decisions_that_measurements_settled():
+    """(kind, T, N, K[, hd]) -> plan: each of these was timed against the other shapes with operands from memory."""
+    settled = {
+        (ops.PLAN_STORE, 2048, 37888, 3584): (256, 256, 1),       # fills the chip: the largest blocks
+        (ops.PLAN_STORE, 2048, 4608, 3584): (256, 160, 1),        # 232 blocks where 256 x 256 make 144
+        (ops.PLAN_ACCUMULATE, 2048, 5120, 27648): (256, 160, 1),  # 256 blocks where 256 x 256 make 160
+        (ops.PLAN_ACCUMULATE, 2048, 3584, 3584): (256, 128, 1),
+        (ops.PLAN_ACCUMULATE, 2048, 896, 4864): (128, 128, 2),
+        (ops.PLAN_ACCUMULATE, 2048, 896, 896): (64, 64, 1),
+        (ops.PLAN_GATED, 2048, 9728, 896): (384, 256, 1),
+        (ops.PLAN_GATED, 256, 9728, 896): (128, 128, 1),
+        (ops.PLAN_ROTATING, 2048, 1152, 896, 64): (128, 128, 1),
+        (ops.PLAN_ROTATING, 1024, 1152, 896, 64): (64, 128, 1),
+        (ops.PLAN_ROTATING, 512, 1152, 896, 64): None,            # 64 x 64 and a rotation kernel after it
+        (ops.PLAN_ROTATING, 2048, 4608, 3584, 128): None,         # 256 x 160 and a rotation kernel after it
+        (ops.PLAN_ROTATING, 1024, 4608, 3584, 128): (256, 128, 1),
+        (ops.PLAN_ROTATING, 512, 4608, 3584, 128): (128, 128, 1),
+        (ops.PLAN_ROTATING, 256, 4608, 3584, 128): (64, 128, 1),
+    }
+    for args, want in settled.items():
+        assert ops.pipe_plan(*args) == want, (args, ops.pipe_plan(*args), want)
