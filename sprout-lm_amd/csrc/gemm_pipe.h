@@ -227,7 +227,6 @@ inline int pipe_shape(hipStream_t s, const void* x, const void* w, const void* b
     case 6: return launch_pipe<6, 2, 2, 4, 2, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 7: return launch_pipe<1, 2, 2, 1, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     case 8: return launch_pipe<2, 5, 4, 1, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
-    case 9: return launch_pipe<1, 1, 2, 4, 3, TB>(s, x, w, bias, mode, out, T, N, K, splits);
     default: return launch_pipe<1, 1, 2, 2, 4, TB>(s, x, w, bias, mode, out, T, N, K, splits);
   }
 }

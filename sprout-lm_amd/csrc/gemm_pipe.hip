@@ -27,11 +27,6 @@ static const PipeShape kPipeShapes[] = {
     // 4 waves in a column, five tile columns each, 3 stages: where 256 x 256 leaves CUs idle; with a short K its
     // blocks cost more than their share (9,728 rows, K = 896: 57 us against 51)
     {256, 160, 1, 2.0f, 1.4f},
-    // 64 x 128 on 8 waves of one tile each, 3 stages; two on a CU take as long as one after the other.  Many
-    // tokens by few weight rows, with operands that come from memory: 1,024 tokens, 896 rows, K = 4,864 in two:
-    // 25.2 us against 26.3 on 64 x 64 and 30.7 on 128 x 128; 2,048 tokens: 42.7 against 45.8, where 128 x 128 with
-    // K in two takes 37.3; below 1,024 tokens 64 x 64 is ahead (512 tokens: 16.3 against 15.5)
-    {64, 128, 1, 0.45f, 0.52f},
 };
 
 // Picks the shape and the split of K with the least estimated time.  Fetching tiles from L2 bounds these
@@ -63,7 +58,7 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     }
     return;
   }
-  for (int c : {0, 1, 2, 3, 5, 6, 8, 9}) {
+  for (int c : {0, 1, 2, 3, 5, 6, 8}) {
     // (64 x 128 fills the chip where 128 x 128 leaves CUs idle and 64 x 64 needs a second round: 2,048 tokens,
     // 1,152 rows, K = 896: 14.8 us against 17.2 and 15.1)
     if (c == 3 && paired) continue;   // one tile column a wave: no lane holds both of a pair
@@ -71,7 +66,6 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     // make 232 blocks instead of 144 of 256 x 256, 83 us against 91; 5,120 rows at K = 27,648 make 256 instead of 160,
     // 607 us against 658; with a short K its blocks cost more than their share, 57 us against 51 at 9,728 rows, K = 896)
     if (c == 8 && paired) continue;
-    if (c == 9 && (paired || T < 1024)) continue;   // one tile a wave
     const PipeShape& p = kPipeShapes[c];
     // blocks of 384 x 256, with all of the LDS in two stages, fetch slowly on a long K once there are more
     // token tiles than the 8 that run together on an XCD (4,096 tokens, 4,608 rows, K = 3,584: 241 us against 180

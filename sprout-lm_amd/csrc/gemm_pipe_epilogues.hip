@@ -20,9 +20,8 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
 
 // The block shape on which the rotating epilogue runs, or -1 where the plain product and a rotation kernel after
 // it do better.  It follows the plain product's choice where that pairs tile columns (256 x 128, 128 x 128,
-// 64 x 128); 64 x 128 on 8 waves has one tile column a wave, and the rotation then runs on 64 x 128 on 4 waves,
-// which still beats the plain product and a rotation kernel after it.  Blocks of 64 x 64 pair nothing either: there
-// 64 x 128 takes the rotation once its blocks fill half of the chip (14 + 2 + 2 heads of 64 at K = 896, 1,024
+// 64 x 128).  Blocks of 64 x 64 have one tile column a wave and pair nothing: there 64 x 128 takes the rotation
+// once its blocks fill half of the chip (14 + 2 + 2 heads of 64 at K = 896, 1,024
 // tokens: 14.5 us against 17.6 apart, 512 tokens: 15.2 against 13.8; 28 + 4 + 4 heads of 128 at K = 3,584, 256
 // tokens: 36.5 against 42.5).  The blocks of 256 x 256 hold 128 sums per lane, all the registers a lane has there:
 // the epilogue's own would be spilled (measured at 28 + 4 + 4 heads of 128, 2,048 tokens: 332 us against 106 and a
@@ -30,7 +29,6 @@ int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, 
 static int rope_shape(int T, int N, int K) {
   int shape, splits;
   pipe_choice(T, N, K, false, &shape, &splits);
-  if (shape == 9) shape = 5;
   if (shape == 3 && ((T + 63) / 64) * ((N + 127) / 128) >= 128) shape = 5;
   // (and with the rotation 128 x 128 on 8 waves beats 64 x 128 on 4 once its blocks fill half of the chip: 14 + 2 + 2
   // heads of 64 at K = 896, 2,048 tokens: 20.2 us against 23.0; 1,024 tokens: 19.2 against 14.5)
@@ -56,13 +54,14 @@ bool gemm_pipe_rope_takes(int T, int N, int K, int hd) {
 }
 
 // Rows and columns of every block shape, by its index in gemm_pipe.hip's list.
-static const int kShapeRows[] = {256, 256, 128, 64, 64, 64, 384, 64, 256, 64};
-static const int kShapeCols[] = {256, 128, 128, 64, 256, 128, 256, 64, 160, 128};
+static const int kShapeRows[] = {256, 256, 128, 64, 64, 64, 384, 64, 256};
+static const int kShapeCols[] = {256, 128, 128, 64, 256, 128, 256, 64, 160};
+static const int kShapeWaves[] = {8, 8, 8, 4, 8, 4, 8, 2, 4};
 
 }  // namespace sprout
 
 // What the pipelined product would do with T x N x K: kind 0 store, 1 accumulate, 2 gated (N = 2 I rows of w),
-// 3 rotating (head size hd).  plan = {block rows, block columns, splits of K}.  Returns 1 where the pipelined kernel
+// 3 rotating (head size hd).  plan = {block rows, block columns, splits of K, waves of a block}.  Returns 1 where the pipelined kernel
 // (for kind 3: its rotating epilogue) does not take the product, else 0.  Runs nothing: for tests and tools.
 extern "C" int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan) {
   using namespace sprout;
@@ -78,6 +77,7 @@ extern "C" int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan) {
   plan[0] = kShapeRows[shape];
   plan[1] = kShapeCols[shape];
   plan[2] = splits;
+  plan[3] = kShapeWaves[shape];
   return 0;
 }
 

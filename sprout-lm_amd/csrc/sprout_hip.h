@@ -34,7 +34,8 @@ int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, in
 // Whether folding the norm into the product (norm = 1 above) is faster than a norm kernel before it.
 int sp_fused_norm_pays(int T, int N, int K);
 // What the tiled product for many tokens would do with T x N x K, without running anything: kind 0 store,
-// 1 accumulate, 2 gated (N = 2 I), 3 rotating (head size hd); plan = {block rows, block columns, splits of K}.
+// 1 accumulate, 2 gated (N = 2 I), 3 rotating (head size hd); plan = {block rows, block columns, splits of K,
+// waves of a block}.
 // Returns 1 where that kernel (for kind 3 its rotating epilogue) does not take the product.
 int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan);
 int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,

@@ -350,11 +350,11 @@ PLAN_STORE, PLAN_ACCUMULATE, PLAN_GATED, PLAN_ROTATING = 0, 1, 2, 3
 
 
 def pipe_plan(kind: int, T: int, N: int, K: int, hd: int = 0):
-    """(block rows, block columns, splits of K) that the tiled product for many tokens would take for T x N x K,
-    or None where that kernel (for PLAN_ROTATING its rotating epilogue) does not take the product.  Runs nothing
-    and needs no GPU."""
+    """(block rows, block columns, splits of K, waves of a block) that the tiled product for many tokens would take
+    for T x N x K, or None where that kernel (for PLAN_ROTATING its rotating epilogue) does not take the product.
+    Runs nothing and needs no GPU."""
     import ctypes
-    plan = (ctypes.c_int * 3)()
+    plan = (ctypes.c_int * 4)()
     if library().sp_pipe_plan(kind, T, N, K, hd, plan):
         return None
     return tuple(plan)

@@ -26,7 +26,7 @@ def bf16(x):
                                    (1100, 13400, 192),    # blocks of 384 tokens save a round of blocks
                                    # blocks of 256 x 160 fill the chip where 256 x 256 do not; the second with K in two
                                    (2000, 5000, 1088), (777, 5000, 3584),
-                                   # many tokens by few rows: 64 x 128 on eight waves; the second with K in four
+                                   # many tokens by few rows; the second with K in four
                                    (1100, 900, 1088), (2000, 130, 2432),
                                    # few tiles and a long K
                                    (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432)])
@@ -50,6 +50,45 @@ def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     acc = t(base)
     ops.gemm(A, W, acc, accumulate=True)                    # the residual sum is float32
     assert np.abs(acc.cpu().numpy() - (base + want)).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
+
+
+# One product for every block shape of the tiled kernel, whole and with K split: (accumulate, T, N, K) -> (block rows,
+# block columns, waves, K split?).  The plan is asserted, so that a change of the cost model that moves a size to
+# another shape says so here instead of leaving a shape without a test.
+BLOCK_SHAPE_SIZES = {
+    (0, 65, 130, 64): (64, 64, 4, False), (1, 260, 130, 3584): (64, 64, 4, True),
+    (0, 130, 13400, 64): (64, 128, 4, False), (1, 260, 2000, 18944): (64, 128, 4, True),
+    (0, 264, 7000, 64): (128, 128, 8, False), (1, 65, 4608, 2048): (128, 128, 8, True),
+    (0, 264, 13400, 64): (256, 128, 8, False), (1, 2730, 130, 9728): (256, 128, 8, True),
+    (0, 513, 13400, 1088): (256, 160, 4, False), (1, 3640, 257, 9728): (256, 160, 4, True),
+    (0, 513, 13400, 64): (256, 256, 8, False), (1, 1300, 3584, 9728): (256, 256, 8, True),
+    (0, 1100, 13400, 64): (384, 256, 8, False), (1, 1040, 5000, 27648): (384, 256, 8, True),
+}
+
+
+@pytest.mark.parametrize("case", sorted(BLOCK_SHAPE_SIZES))
+def test_tiled_product_on_every_block_shape(case):
+    from sprout_lm_amd import ops
+    accumulate, T, N, K = case
+    rows, cols, splits, waves = ops.pipe_plan(ops.PLAN_ACCUMULATE if accumulate else ops.PLAN_STORE, T, N, K)
+    assert (rows, cols, waves, splits > 1) == BLOCK_SHAPE_SIZES[case], "this size has moved to another block shape"
+    gen = torch.Generator(device=DEV).manual_seed(T + N)
+    x = torch.randn(T, K, device=DEV, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV, generator=gen) * K ** -0.5).to(torch.bfloat16)
+    want = x.float() @ w.float().T          # float32 product of the same bfloat16 operands
+    if accumulate:
+        before = torch.randn(T, N, device=DEV, generator=gen)
+        out = before.clone()
+        ops.gemm(x, w, out, accumulate=True)
+        err = (out - (before + want)).abs().max().item()
+        assert err <= 2e-5 * max(1.0, math.sqrt(K) / 8) * (1 + want.abs().max().item()), err
+    else:
+        bias = torch.randn(N, device=DEV, generator=gen).to(torch.bfloat16)
+        out = torch.empty(T, N, dtype=torch.bfloat16, device=DEV)
+        ops.gemm(x, w, out, bias=bias)
+        want = want + bias.float()
+        err = (out.float() - want).abs().max().item()
+        assert err <= 2 ** -7 * (1 + want.abs().max().item()), err
 
 
 @pytest.mark.parametrize("T,N,K", [(8, 151, 96), (16, 64, 1024), (7, 2050, 132), (13, 33, 4), (1, 896, 4864), (16, 1, 260)])
