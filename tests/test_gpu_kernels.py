@@ -593,11 +593,22 @@ def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm)
 
 
-# 28 + 4 + 4 heads of 128: the rotating epilogue on blocks of 256 x 128 (1,024 tokens) and of 128 x 128 (513 tokens at
-# K = 3,584), eight waves each
-@pytest.mark.parametrize("T,K", [(1024, 264), (1024, 896), (513, 3584)])
-def test_fused_qkv_rope_cache_on_blocks_of_eight_waves(T, K):
-    check_fused_qkv_rope_cache(T, 28, 4, 128, K, 16, False)
+# The rotating epilogue on each block shape that takes it: (T, nq, nkv, hd, K) -> (block rows, block columns, waves).
+# The plan is asserted: a size that has moved to another shape says so.
+ROTATING_SHAPE_SIZES = {
+    (200, 28, 4, 128, 896): (64, 128, 4), (264, 28, 4, 128, 3584): (64, 128, 4), (1024, 14, 2, 64, 896): (64, 128, 4),
+    (400, 28, 4, 128, 448): (128, 128, 8), (513, 28, 4, 128, 3584): (128, 128, 8), (2048, 14, 2, 64, 896): (128, 128, 8),
+    (1024, 28, 4, 128, 448): (256, 128, 8), (1024, 28, 4, 128, 896): (256, 128, 8),
+}
+
+
+@pytest.mark.parametrize("case", sorted(ROTATING_SHAPE_SIZES))
+def test_fused_qkv_rope_cache_on_every_block_shape(case):
+    from sprout_lm_amd import ops
+    T, nq, nkv, hd, K = case
+    rows, cols, splits, waves = ops.pipe_plan(ops.PLAN_ROTATING, T, (nq + 2 * nkv) * hd, K, hd)
+    assert (rows, cols, waves) == ROTATING_SHAPE_SIZES[case] and splits == 1, "this size has moved to another block shape"
+    check_fused_qkv_rope_cache(T, nq, nkv, hd, K, 16, False)
 
 
 def check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
@@ -657,7 +668,8 @@ def check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
 @pytest.mark.parametrize("T,I,K", [(t_, i_, k_) for t_ in [1, 8, 16, 33, 64, 65, 200, 513]
                                    for i_, k_ in [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)]]
                          + [(1100, 6700, 128), (2048, 4864, 896),   # blocks of 384 tokens
-                            (1024, 2432, 264), (200, 1000, 3584)])  # blocks of 256 x 128 and 128 x 128 on eight waves
+                            (1024, 2432, 264), (200, 1000, 3584),   # blocks of 256 x 128 and 128 x 128 on eight waves
+                            (513, 18944, 896), (264, 18944, 448)])  # blocks of 256 x 256 and of 64 x 128
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops

@@ -87,3 +87,25 @@ def test_decisions_that_measurements_settled():
     for args, want in settled.items():
         got = ops.pipe_plan(*args)
         assert (got[:3] if got else None) == want, (args, got, want)
+
+
+def test_kernel_tests_reach_every_block_shape():
+    """The sizes that tests/test_gpu_kernels.py runs on the GPU, asked here for their plans: every block shape of the
+    plain, the gated and the rotating product is reached by at least one of them."""
+    import importlib
+    kernels = importlib.import_module("tests.test_gpu_kernels")
+    plain = {(rows, cols, waves, split) for rows, cols, waves, split in kernels.BLOCK_SHAPE_SIZES.values()}
+    assert {(r, c) for r, c, _, _ in plain} == SHAPES - {(64, 256)} and {s for _, _, _, s in plain} == {False, True}
+    for (accumulate, T, N, K), (rows, cols, waves, split) in kernels.BLOCK_SHAPE_SIZES.items():
+        got = ops.pipe_plan(ops.PLAN_ACCUMULATE if accumulate else ops.PLAN_STORE, T, N, K)
+        assert (got[0], got[1], got[3], got[2] > 1) == (rows, cols, waves, split), (T, N, K, got)
+    rotating = set()
+    for (T, nq, nkv, hd, K), shape in kernels.ROTATING_SHAPE_SIZES.items():
+        got = ops.pipe_plan(ops.PLAN_ROTATING, T, (nq + 2 * nkv) * hd, K, hd)
+        assert (got[0], got[1], got[3]) == shape, (T, nq, nkv, hd, K, got)
+        rotating.add(shape[:2])
+    assert rotating == ROTATING
+    marks = [m for m in kernels.test_fused_gate_up_silu_and_normed_product.pytestmark
+             if m.name == "parametrize" and m.args[0] == "T,I,K"]
+    gated = {ops.pipe_plan(ops.PLAN_GATED, T, 2 * I, K)[:2] for T, I, K in marks[0].args[1] if T > 64 and K % 64 == 0}
+    assert gated >= {(64, 128), (128, 128), (256, 128), (256, 256), (384, 256)}, gated
