@@ -840,11 +840,20 @@ static bool staged_prefill(int page_size) { return page_size >= 8 && (page_size 
 // (each wave then takes 64 keys of a stage).  Three teams were slower than two or four at every size.
 // A portion of 2,048 tokens at a context of 32,768: 835 -> 472 us (14 heads of 64), 2,350 -> 1,470 us (28 of 128).
 struct StagedShape { int hpb, wpt; bool ahead; };
-static StagedShape staged_shape(int nq, int nkv, int hd) {
+static StagedShape staged_shape(int nq, int nkv, int hd, int n_tiles) {
   const int G = nq / nkv;
   if (G <= 1) return {1, 4, false};
   if (G == 2) return {2, 4, hd > 64};
-  return hd > 64 ? StagedShape{4, 2, false} : StagedShape{4, 4, true};
+  if (hd > 64) return {4, 2, false};
+  // Head sizes up to 64: four heads a block stage every key once for four heads, but a portion of a prompt has
+  // few tiles, and four heads a block then leave most CUs without one.  As many heads a block as still give every
+  // CU a block (14 heads of 64 in 2 groups, time to the first token over 4 layers: 4,096 tokens in portions of
+  // 256: 4.88 ms with four heads a block, 4.80 with two, 4.62 with one; 8,192 in portions of 1,024: 5.64, 5.05,
+  // 5.47; 2,048 at once: 1.07, 1.16, 1.09; 16,384 in portions of 2,048: 9.38, 10.76, 11.42).  At a head size of
+  // 128 the block of four heads on two waves each was the fastest at every portion size.
+  if (n_tiles * nkv * ((G + 3) / 4) >= 256) return {4, 4, true};
+  if (n_tiles * nkv * ((G + 1) / 2) >= 256) return {2, 4, false};
+  return {1, 4, false};
 }
 // Whether the tiles are taken in pairs (a long walk and a short one per block), and with which teams.
 static bool staged_paired(int n_tiles, int nq, int nkv, int hd, int splits, int max_tile_ctx, int mean_tile_walk,
@@ -870,7 +879,7 @@ static bool staged_paired(int n_tiles, int nq, int nkv, int hd, int splits, int 
 
 int attention_prefill_splits(int n_tiles, int nq, int nkv, int hd, int page_size, int max_tile_ctx) {
   if (!staged_prefill(page_size)) return 1;
-  const StagedShape shape = staged_shape(nq, nkv, hd);
+  const StagedShape shape = staged_shape(nq, nkv, hd, n_tiles);
   const int G = nq / nkv;
   const int blocks = n_tiles * nkv * ((G + shape.hpb - 1) / shape.hpb), stages = (max_tile_ctx + kStageKeys - 1) / kStageKeys;
   const int enough = 2048 / (shape.wpt * shape.hpb);   // blocks that hold 2,048 waves: two rounds of the chip's CUs
@@ -909,7 +918,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
       const int per_split = (stages + splits - 1) / splits;
       float* part_o = splits > 1 ? prefill_ws : nullptr;
       float* part_ml = splits > 1 ? prefill_ws + size_t(n_tiles) * 16 * NQT * nq * splits * HD : nullptr;
-      StagedShape shape = staged_shape(nq, nkv, HD);
+      StagedShape shape = staged_shape(nq, nkv, HD, n_tiles);
       const bool paired = staged_paired(n_tiles, nq, nkv, HD, splits, max_tile_ctx, mean_tile_walk, &shape);
       const dim3 grid(paired ? (n_tiles + 1) / 2 : n_tiles, nkv * ((nq / nkv + shape.hpb - 1) / shape.hpb), splits);
 #define SP_STAGED(HPB, WPT, AHEAD, PAIRED)                                                                      \
