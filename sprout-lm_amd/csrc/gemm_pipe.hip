@@ -79,8 +79,12 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
       if (sp > 1 && (!may_split || steps / sp < 8)) break;
       const int blocks = tiles * sp, full = blocks / slots, rest = blocks % slots;
       const float per_block = float((steps + sp - 1) / sp) * step_us + 1.0f;
-      // a round that does not fill the chip runs somewhat faster: fewer blocks share the caches
-      float t = full * per_block + (rest ? per_block * (0.7f + 0.3f * float(rest) / slots) : 0.f);
+      // a round that does not fill the chip runs somewhat faster: fewer blocks share the caches; much faster for
+      // the blocks of 384 x 256 with one tile of tokens, whose two stages hold all of the LDS and wait for their tiles
+      // the most (264 tokens, 37,888 rows, K = 3,584 with the gating: 148 blocks take 2.25 us a step, 126 us
+      // against 134 on 128 x 128)
+      const float alone = c == 6 && full == 0 && T <= p.bm ? 0.3f : 0.7f;
+      float t = full * per_block + (rest ? per_block * (alone + (1.f - alone) * float(rest) / slots) : 0.f);
       if (sp > 1) t += 2.7e-6f * float(T) * float(N) * sp;      // float atomics into the output
       if (t < best) { best = t; *shape = c; *splits = sp; }
     }

@@ -59,7 +59,7 @@ BLOCK_SHAPE_SIZES = {
     (0, 65, 130, 64): (64, 64, 4, False), (1, 260, 130, 3584): (64, 64, 4, True),
     (0, 130, 13400, 64): (64, 128, 4, False), (1, 260, 2000, 18944): (64, 128, 4, True),
     (0, 264, 7000, 64): (128, 128, 8, False), (1, 65, 4608, 2048): (128, 128, 8, True),
-    (0, 264, 13400, 64): (256, 128, 8, False), (1, 2730, 130, 9728): (256, 128, 8, True),
+    (0, 1024, 4608, 448): (256, 128, 8, False), (1, 2730, 130, 9728): (256, 128, 8, True),
     (0, 513, 13400, 1088): (256, 160, 4, False), (1, 3640, 257, 9728): (256, 160, 4, True),
     (0, 513, 13400, 64): (256, 256, 8, False), (1, 1300, 3584, 9728): (256, 256, 8, True),
     (0, 1100, 13400, 64): (384, 256, 8, False), (1, 1040, 5000, 27648): (384, 256, 8, True),
@@ -669,7 +669,7 @@ def check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
                                    for i_, k_ in [(4864, 896), (224, 96), (176, 240), (1000, 264), (331, 72), (160, 2312)]]
                          + [(1100, 6700, 128), (2048, 4864, 896),   # blocks of 384 tokens
                             (1024, 2432, 264), (200, 1000, 3584),   # blocks of 256 x 128 and 128 x 128 on eight waves
-                            (513, 18944, 896), (264, 18944, 448)])  # blocks of 256 x 256 and of 64 x 128
+                            (513, 18944, 896), (130, 9472, 448), (264, 18944, 448)])  # blocks of 256 x 256, of 64 x 128, one of 384
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     from sprout_lm_amd import ops
