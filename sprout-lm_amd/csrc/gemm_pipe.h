@@ -40,6 +40,21 @@ __device__ __forceinline__ void wait_loads_then_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
+// How the tiles of a product are numbered over the blocks of a launch (the kernel and its launch agree on it):
+// every XCD has `own` blocks for the weight tiles that are its own (`full` of them, token tiles in whole groups of
+// `group`), then `run` blocks of the `left` weight tiles that are dealt out.
+struct PipeTiles { int tiles_t, full, left, group, own, run; };
+__host__ __device__ inline PipeTiles pipe_tiles(int tiles_t, int tiles_n) {
+  PipeTiles p;
+  p.tiles_t = tiles_t;
+  p.full = tiles_n / 8;
+  p.left = tiles_n % 8;
+  p.group = tiles_t < 8 ? tiles_t : 8;
+  p.own = p.full * p.group * ((tiles_t + p.group - 1) / p.group);
+  p.run = (p.left * tiles_t + 7) / 8;
+  return p;
+}
+
 // A block of WAVES_M x WAVES_N waves, each with WM x WN tiles of 32 x 32: BM = 32 WM WAVES_M tokens by
 // BN = 32 WN WAVES_N weight rows.  Blocks of up to four waves ask for the registers of two waves a SIMD: with
 // all 512 to itself the compiler keeps the accumulators in one half of them and copies all of them to the
@@ -62,13 +77,23 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   // Which tile: blocks go round the 8 XCDs (block b runs on XCD b % 8, each with an L2 of its own), so XCD c
   // takes the weight tiles c, c + 8, ... and nobody else fetches them; within an XCD the blocks that run
   // together are up to 8 token tiles of the same few weight tiles, so that w is read from memory once
-  // whatever the number of tokens, and x stays in the caches.
-  const int tiles_t = (T + BM - 1) / BM, tiles_n = ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN;
-  const int per_xcd = (tiles_n + 7) / 8, group = min(tiles_t, 8);
+  // whatever the number of tokens, and x stays in the caches.  The weight tiles left over when their number is no
+  // multiple of 8 are dealt out by token tile, an equal run of their blocks to every XCD: four left-over weight
+  // tiles would otherwise be a quarter more blocks on four of the XCDs, and fewer than 8 weight tiles idle XCDs.
+  const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
   const int xcd = blockIdx.x & 7, i_xcd = blockIdx.x >> 3;
-  const int g = i_xcd / (per_xcd * group), rest = i_xcd % (per_xcd * group);
-  const int tile_n = (rest / group) * 8 + xcd, tile_t = g * group + rest % group;
-  if (tile_n >= tiles_n || tile_t >= tiles_t) return;
+  int tile_n, tile_t;
+  if (i_xcd < tiles.own) {
+    const int g = i_xcd / (tiles.full * tiles.group), rest = i_xcd % (tiles.full * tiles.group);
+    tile_n = (rest / tiles.group) * 8 + xcd;
+    tile_t = g * tiles.group + rest % tiles.group;
+    if (tile_t >= tiles.tiles_t) return;
+  } else {
+    const int j = i_xcd - tiles.own, k = xcd * tiles.run + j;
+    if (j >= tiles.run || k >= tiles.left * tiles.tiles_t) return;
+    tile_n = 8 * tiles.full + k / tiles.tiles_t;
+    tile_t = k % tiles.tiles_t;
+  }
   const int t0 = tile_t * BM, n0 = tile_n * BN;
   const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
   const int steps = (k_end - k_begin) / 64;
@@ -187,10 +212,9 @@ inline int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const 
     }
     raised = true;
   }
-  // the kernel's own numbering of tiles: 8 XCDs x weight tiles per XCD x token tiles in whole groups
-  const int tiles_t = (T + BM - 1) / BM, tiles_n = ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN;
-  const int per_xcd = (tiles_n + 7) / 8, group = min(tiles_t, 8), groups = (tiles_t + group - 1) / group;
-  dim3 grid(8 * per_xcd * group * groups, 1, splits);
+  // the kernel's own numbering of tiles
+  const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
+  dim3 grid(8 * (tiles.own + tiles.run), 1, splits);
   gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope);
   return check_launch("sp_gemm (pipelined)");
 }

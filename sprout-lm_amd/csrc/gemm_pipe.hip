@@ -74,14 +74,16 @@ void pipe_choice(int T, int N, int K, bool may_split, int* shape, int* splits, b
     // (64 x 128 on a short K beside many tokens: 256 tokens, 9,728 rows, K = 896 with the gating: 16.3 us against
     // 13.8 on 128 x 128)
     const float step_us = steps <= 16 ? (c == 5 ? 0.8f : p.short_us) : (c == 6 && (T + p.bm - 1) / p.bm > 8) ? 4.3f : p.long_us;
-    // Blocks are counted on the XCD that holds the most: XCD c runs the weight tiles c, c + 8, ... with all their
-    // token tiles and splits on its 32 CUs, so 28 weight tiles are four on XCDs 0 to 3 and three on the others
-    // (264 tokens, 3,584 rows, K = 18,944 on 128 x 128 with K in three: 252 blocks in all, but 36 on XCD 0, whose
-    // second round makes it 106 us where 256 x 128 with K in four, 32 a XCD, takes 89).
-    const int tiles_t = (T + p.bm - 1) / p.bm, tiles_n = (N + p.bn - 1) / p.bn, slots = 32 * p.per_cu;
+    // Blocks are counted on the XCD that holds the most, as the kernel numbers them: XCD c runs the weight tiles
+    // c, c + 8, ... with all their token tiles and splits on its 32 CUs, and an equal run of the blocks of the
+    // weight tiles that are left over (264 tokens, 3,584 rows, K = 18,944 on 128 x 128 with K in three: 252
+    // blocks in all, which were 36 on XCD 0 before the left-over tiles were dealt out: a second round, 106 us
+    // where 256 x 128 with K in four, 32 a XCD, takes 89).
+    const PipeTiles tiles = pipe_tiles((T + p.bm - 1) / p.bm, (N + p.bn - 1) / p.bn);
+    const int slots = 32 * p.per_cu;
     for (int sp : {1, 2, 3, 4, 6, 8}) {
       if (sp > 1 && (!may_split || steps / sp < 8)) break;
-      const int blocks = (tiles_n + 7) / 8 * tiles_t * sp, full = blocks / slots, rest = blocks % slots;
+      const int blocks = (tiles.full * tiles.tiles_t + tiles.run) * sp, full = blocks / slots, rest = blocks % slots;
       const float per_block = float((steps + sp - 1) / sp) * step_us + 1.0f;
       // a round that does not fill the chip runs somewhat faster: fewer blocks share the caches; much faster for
       // the blocks of 384 x 256 with one tile of tokens, whose two stages hold all of the LDS and wait for their tiles

@@ -58,11 +58,11 @@ def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
 BLOCK_SHAPE_SIZES = {
     (0, 65, 130, 64): (64, 64, 4, False), (1, 260, 130, 3584): (64, 64, 4, True),
     (0, 130, 13400, 64): (64, 128, 4, False), (1, 260, 2000, 18944): (64, 128, 4, True),
-    (0, 264, 7000, 64): (128, 128, 8, False), (1, 65, 2570, 3584): (128, 128, 8, True),
-    (0, 1024, 4608, 448): (256, 128, 8, False), (1, 130, 2570, 18944): (256, 128, 8, True),
-    (0, 4104, 1152, 448): (256, 160, 4, False), (1, 777, 1152, 9728): (256, 160, 4, True),
-    (0, 513, 13400, 64): (256, 256, 8, False), (1, 2056, 2000, 9728): (256, 256, 8, True),
-    (0, 1100, 13400, 64): (384, 256, 8, False), (1, 264, 13400, 9728): (384, 256, 8, True),
+    (0, 264, 7000, 64): (128, 128, 8, False), (1, 65, 4608, 3584): (128, 128, 8, True),
+    (0, 1024, 4608, 448): (256, 128, 8, False), (1, 200, 2570, 18944): (256, 128, 8, True),
+    (0, 2056, 3590, 1088): (256, 160, 4, False), (1, 4104, 900, 9728): (256, 160, 4, True),
+    (0, 513, 13400, 64): (256, 256, 8, False), (1, 1034, 4030, 9728): (256, 256, 8, True),
+    (0, 1100, 13400, 64): (384, 256, 8, False), (1, 260, 13400, 9728): (384, 256, 8, True),
 }
 
 
