@@ -307,7 +307,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
   constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
   constexpr int STAGE_BYTES = (kStageKeys * KP + HD * VP) * 2;
-  constexpr int MERGE_BYTES = WPT * 16 * NQT * (HD + 2) * 4;
+  constexpr int MERGE_BYTES = WPT * 16 * NQT * (HD + 4) * 4;
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE_BYTES > MERGE_BYTES ? STAGE_BYTES : MERGE_BYTES];
   __shared__ int32_t s_table[kMaxTableLds];
   uint16_t* ks = reinterpret_cast<uint16_t*>(smem);
@@ -446,9 +446,11 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
     }
   }
 
-  // merge the waves of each team in turn: [wave][row][HD + 2] floats = (O^T row ..., maximum, sum)
+  // merge the waves of each team in turn: [wave][row][HD + 4] floats = (O^T row ..., maximum, sum, two unused).
+  // A pitch of HD + 4 floats puts the 16 rows that a quarter of a wave writes or reads as 16 bytes each on
+  // different LDS banks (HD + 2 with single floats collided three and four ways).
   float* mg = reinterpret_cast<float*>(smem);
-  constexpr int MP = HD + 2;
+  constexpr int MP = HD + 4;
 #pragma unroll 1
   for (int turn = 0; turn < HPB; ++turn) {
     if (first_head + turn >= G) break;
@@ -462,8 +464,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
         float* row = mg + (size_t(wave) * 16 * NQT + 16 * qt + lr) * MP;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) row[16 * dt + 4 * lj + r4] = o[qt][dt][r4];
+          *reinterpret_cast<float4*>(row + 16 * dt + 4 * lj) = make_float4(o[qt][dt][0], o[qt][dt][1], o[qt][dt][2], o[qt][dt][3]);
         if (lj == 0) { row[HD] = m[qt]; row[HD + 1] = l; }
       }
     }
@@ -480,8 +481,8 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
         const float* src = mg + (size_t(w) * 16 * NQT + row) * MP;
         const float f = exp2f(src[HD] - mx);
         den += f * src[HD + 1];
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) num[r4] += f * src[d + r4];
+        const float4 part = *reinterpret_cast<const float4*>(src + d);
+        num[0] += f * part.x; num[1] += f * part.y; num[2] += f * part.z; num[3] += f * part.w;
       }
       if (n_splits > 1) {
         // partial result of this block's keys: sums against the maximum mx, for the merge kernel
