@@ -112,7 +112,9 @@ __device__ __forceinline__ float max_over_quarters(float x) {
 // MASKED false: every key of the step is visible to every existing row (the caller has checked), and
 // rows that do not exist compute values nobody reads.  The running maximum m is in log2 units and
 // starts at kNoKeyYet.
-template <int DT, int NQT, bool MASKED, bool LAZY>
+// CONTIG: the step's keys in the order 8 lj + 4 kt + r (a lane's eight keys in a row, as the staged kernel reads its
+// values from LDS in one piece) instead of 16 kt + 4 lj + r; whoever loads the step lays its key rows out to match.
+template <int DT, int NQT, bool MASKED, bool LAZY, bool CONTIG>
 __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                                  floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT],
                                                  int key0, int k_lo, const int (&qpos)[NQT], int window,
@@ -139,12 +141,12 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
       const int span = hi - lo;
       const unsigned limit = span >= 0 ? unsigned(span) : 0u;
       const int base = span >= 0 ? lo : key0 + 64;          // key - base < 0 for every key of the step: none passes
-      const int first = key0 + 4 * lj - base;
+      const int first = key0 + (CONTIG ? 8 : 4) * lj - base;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4)
-          s[qt][kt][r4] = unsigned(first + 16 * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
+          s[qt][kt][r4] = unsigned(first + (CONTIG ? 4 : 16) * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
     }
     float raw = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
     raw = vmax3(raw, s[qt][0][3], s[qt][1][0]);
@@ -185,15 +187,15 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 
 // `first_pos`: smallest position among the rows that exist; a step whose 32 keys all lie at or before
 // it (and inside [k_lo, ...) with no window) needs no masking.
-template <int DT, int NQT, bool LAZY = true>
+template <int DT, int NQT, bool LAZY = true, bool CONTIG = false>
 __device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                             floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT], int key0,
                                             int k_lo, const int (&qpos)[NQT], int window, float scale2,
                                             int first_pos) {
   if (window <= 0 && key0 >= k_lo && key0 + 31 <= first_pos)
-    attend_step_impl<DT, NQT, false, LAZY>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step_impl<DT, NQT, false, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
   else
-    attend_step_impl<DT, NQT, true, LAZY>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step_impl<DT, NQT, true, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
 }
 
 template <int DT>
@@ -287,6 +289,10 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
 // The sequence's page numbers are copied to LDS first, so that a fetch is one trip to memory.
 // Needs pages of 8, 16, 32, ... tokens (a power of two).
 constexpr int kStageKeys = 128;
+// LDS row of key r of a stage: the keys of each step of 32 lie in the order in which the two score tiles take them
+// (attend_step's CONTIG order): key 8 a + 4 t + b of the step in row 16 t + 4 a + b, so that lane row 4 a + b of
+// tile t reads row 16 t + (its own number) as it would without the permutation.
+__device__ __forceinline__ constexpr int step_row(int r) { return (r & ~31) | ((r & 4) << 2) | (((r & 31) >> 3) << 2) | (r & 3); }
 constexpr int kMaxTableLds = 2048;    // page numbers held in LDS; longer tables are read from memory
 
 template <int DT, int NQT, int HPB, int WPT, bool AHEAD, bool PAIRED>
@@ -300,8 +306,15 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   constexpr int THREADS = 64 * WPT * HPB;
   constexpr int WAVE_KEYS = kStageKeys / WPT;          // keys of a stage that one wave of a team takes
-  constexpr int KP = HD + 8;                  // key row pitch in LDS (elements): 16 bytes of padding
-  constexpr int VP = kStageKeys + 8;          // value row pitch: the stage's keys + 16 bytes of padding
+  // Key row pitch in LDS (elements).  A 16-byte LDS read serves lanes {0-3, 12-15, 20-27} of each half-wave in
+  // one pass and the other 16 in a second (measured with two lanes at a time on one bank), not 16 lanes in a
+  // row: with 16 bytes of padding the rows of those lanes met two to a bank (8 cycles an instruction instead
+  // of 4); 32 bytes of padding keep them apart while the row is a whole number of 64 bytes.
+  constexpr int KP = HD + (DT % 2 == 0 ? 16 : 8);
+  // Value row pitch: the stage's keys + 32 bytes, for the same reason.  A lane reads its eight keys of a step in
+  // one piece of 16 bytes (4 cycles an instruction); as two pieces of 8 bytes 32 bytes apart the compiler made one
+  // ds_read2_b64 of them, which took 16 cycles at the old pitch and 8 at the best (counted on the pattern alone).
+  constexpr int VP = kStageKeys + 16;
   constexpr int KCHUNKS = kStageKeys * (HD / 8);      // 16-byte pieces of the stage's keys ...
   const int page_size = 1 << page_shift, page_mask = page_size - 1;   // pages are a power of two of tokens
   constexpr int CHUNKS = 2 * KCHUNKS;                 // ... and of its values
@@ -412,7 +425,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
       const int i = threadIdx.x + THREADS * u;
       if (i < KCHUNKS) {
         const int r = i / (HD / 8), c = i % (HD / 8);
-        *reinterpret_cast<uint4*>(&ks[r * KP + 8 * c]) = stage[u];
+        *reinterpret_cast<uint4*>(&ks[step_row(r) * KP + 8 * c]) = stage[u];
       } else if (i < CHUNKS) {
         const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
         *reinterpret_cast<uint4*>(&vs[d * VP + 8 * c]) = stage[u];
@@ -435,13 +448,14 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
                                   : as_bf16x8(make_uint4(0, 0, 0, 0));
           }
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-          for (int kt = 0; kt < 2; ++kt)
-            r.va[dt][kt] = *reinterpret_cast<const uint2*>(&vs[(16 * dt + lr) * VP + skey + 16 * kt + 4 * lj]);
+        for (int dt = 0; dt < DT; ++dt) {
+          const uint4 v = *reinterpret_cast<const uint4*>(&vs[(16 * dt + lr) * VP + skey + 8 * lj]);
+          r.va[dt][0] = make_uint2(v.x, v.y);
+          r.va[dt][1] = make_uint2(v.z, v.w);
+        }
         // (the unpaired block of 16 waves has no register to spare: the lazy form made it spill 36 instead of 2,
         // 529 -> 690 us for 2,048 queries over 32,768 keys; the paired one gained with it, 290 -> 264 us at 8,192)
-        attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED)>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+        attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED), true>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
       }
     }
   }
