@@ -393,8 +393,31 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   // as this one lies in LDS, so its trip to memory runs while this one is being used (the registers stay
   // occupied meanwhile: worth it where there are few per thread).
   uint4 stage[PER_THREAD];
+  // Which pieces of 16 bytes a thread moves.  Where the numbers divide (ROWWISE), all its key pieces lie in one key
+  // row (piece kc + KT v of row kr, KT threads a row) and all its value pieces in one block of 8 keys (dims
+  // vd + VD v), so that the page is looked up and the address formed once for the keys and once for the values
+  // instead of once a piece: that arithmetic was a third of the vector instructions of a stage at a head size of
+  // 128.  Otherwise piece threadIdx.x + THREADS u of the stage's 2 KCHUNKS, whatever it is.
+  constexpr int PER_K = KCHUNKS / THREADS, PER_V = KCHUNKS / THREADS;     // keys and values hold as many pieces
+  constexpr bool ROWWISE = KCHUNKS % THREADS == 0 && (HD / 8) % (PER_K > 0 ? PER_K : 1) == 0 && THREADS % 16 == 0;
+  constexpr int KT = ROWWISE ? (HD / 8) / PER_K : 1, VD = THREADS / 16;
+  const int kr = threadIdx.x / KT, kc = threadIdx.x % KT, vc = threadIdx.x % 16, vd = threadIdx.x / 16;
   auto fetch_from = [&](int key0, auto in_lds) __attribute__((always_inline)) {
     const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
+    if constexpr (ROWWISE) {
+      int key = key0 + kr, kb = key0 + 8 * vc;
+      if (!interior) {
+        key = min(max(key, k_lo), k_hi);
+        kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+      }
+      const uint16_t* krow = kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * kc;
+      const uint16_t* vcol = vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(vd)) << page_shift) + (kb & page_mask);
+#pragma unroll
+      for (int v = 0; v < PER_K; ++v) stage[v] = ldg128(krow + 8 * KT * v);
+#pragma unroll
+      for (int v = 0; v < PER_V; ++v) stage[PER_K + v] = ldg128(vcol + (size_t(VD * v) << page_shift));
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < PER_THREAD; ++u) {
       const int i = threadIdx.x + THREADS * u;
@@ -420,15 +443,22 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
     if (!AHEAD) fetch(key0);
     __syncthreads();   // the last stage has been used
+    if constexpr (ROWWISE) {
 #pragma unroll
-    for (int u = 0; u < PER_THREAD; ++u) {
-      const int i = threadIdx.x + THREADS * u;
-      if (i < KCHUNKS) {
-        const int r = i / (HD / 8), c = i % (HD / 8);
-        *reinterpret_cast<uint4*>(&ks[step_row(r) * KP + 8 * c]) = stage[u];
-      } else if (i < CHUNKS) {
-        const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
-        *reinterpret_cast<uint4*>(&vs[d * VP + 8 * c]) = stage[u];
+      for (int v = 0; v < PER_K; ++v) *reinterpret_cast<uint4*>(&ks[step_row(kr) * KP + 8 * (kc + KT * v)]) = stage[v];
+#pragma unroll
+      for (int v = 0; v < PER_V; ++v) *reinterpret_cast<uint4*>(&vs[(vd + VD * v) * VP + 8 * vc]) = stage[PER_K + v];
+    } else {
+#pragma unroll
+      for (int u = 0; u < PER_THREAD; ++u) {
+        const int i = threadIdx.x + THREADS * u;
+        if (i < KCHUNKS) {
+          const int r = i / (HD / 8), c = i % (HD / 8);
+          *reinterpret_cast<uint4*>(&ks[step_row(r) * KP + 8 * c]) = stage[u];
+        } else if (i < CHUNKS) {
+          const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
+          *reinterpret_cast<uint4*>(&vs[d * VP + 8 * c]) = stage[u];
+        }
       }
     }
     __syncthreads();
