@@ -132,6 +132,8 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
       for (int c = 0; c < HC; ++c) s[qt][kt] = mfma16(r.ka[kt][c], qop[qt][c], s[qt][kt]);
     }
 
+  float raw[NQT];
+  bool grown = false;
 #pragma unroll
   for (int qt = 0; qt < NQT; ++qt) {
     if (MASKED) {
@@ -148,16 +150,23 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
         for (int r4 = 0; r4 < 4; ++r4)
           s[qt][kt][r4] = unsigned(first + (CONTIG ? 4 : 16) * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
     }
-    float raw = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
-    raw = vmax3(raw, s[qt][0][3], s[qt][1][0]);
-    raw = vmax3(raw, s[qt][1][1], s[qt][1][2]);
-    raw = vmax(raw, s[qt][1][3]);
+    raw[qt] = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
+    raw[qt] = vmax3(raw[qt], s[qt][0][3], s[qt][1][0]);
+    raw[qt] = vmax3(raw[qt], s[qt][1][1], s[qt][1][2]);
+    raw[qt] = vmax(raw[qt], s[qt][1][3]);
     // LAZY: the lane's own 8 keys decide whether anything has to be done about the maximum, and the row's other
     // three lanes are asked only then (-inf when the lane sees no key of the step): ten instructions less per
     // step and tile of rows.  Otherwise the row's maximum is formed first.
-    if (!LAZY) raw = max_over_quarters(raw);
-    if (__builtin_amdgcn_ballot_w64(raw * scale2 > m[qt] + kRescaleStep) != 0) {
-      const float top = (LAZY ? max_over_quarters(raw) : raw) * scale2;
+    if (!LAZY) raw[qt] = max_over_quarters(raw[qt]);
+    grown = grown || raw[qt] * scale2 > m[qt] + kRescaleStep;
+  }
+  // One test for all the tiles of rows: the code that follows it is then one straight run for all of them, which
+  // the compiler interleaves (a test a tile cut it into pieces that each waited for its own chain of exponentials
+  // and matrix instructions).  A tile whose maximum has not grown goes through the rescaling with a factor of one.
+  if (__builtin_amdgcn_ballot_w64(grown) != 0) {
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt) {
+      const float top = (LAZY ? max_over_quarters(raw[qt]) : raw[qt]) * scale2;
       const float mx = top > m[qt] + kRescaleStep ? top : m[qt];   // finite: m starts finite
       const float alpha = __builtin_amdgcn_exp2f(m[qt] - mx);
       m[qt] = mx;
@@ -165,6 +174,9 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha;
     }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
     const float mx = m[qt];
     float p[2][4], sum = 0.f;
 #pragma unroll
@@ -391,8 +403,10 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   }
   // A stage travels memory -> registers -> LDS.  With AHEAD the registers are asked for the next stage as soon
   // as this one lies in LDS, so its trip to memory runs while this one is being used (the registers stay
-  // occupied meanwhile: worth it where there are few per thread).
-  uint4 stage[PER_THREAD];
+  // occupied meanwhile: worth it where there are few per thread).  (Two sets of registers, each asked for the stage
+  // after the next, changed nothing: 30.6 against 30.1 us at 14 heads of 64 and 2,048 tokens.  A block does not
+  // wait for its stages; its waves wait for each other at the barriers and for their own chains of dependent
+  // instructions, two waves a SIMD.)
   // Which pieces of 16 bytes a thread moves.  Where the numbers divide (ROWWISE), all its key pieces lie in one key
   // row (piece kc + KT v of row kr, KT threads a row) and all its value pieces in one block of 8 keys (dims
   // vd + VD v), so that the page is looked up and the address formed once for the keys and once for the values
@@ -402,7 +416,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   constexpr bool ROWWISE = KCHUNKS % THREADS == 0 && (HD / 8) % (PER_K > 0 ? PER_K : 1) == 0 && THREADS % 16 == 0;
   constexpr int KT = ROWWISE ? (HD / 8) / PER_K : 1, VD = THREADS / 16;
   const int kr = threadIdx.x / KT, kc = threadIdx.x % KT, vc = threadIdx.x % 16, vd = threadIdx.x / 16;
-  auto fetch_from = [&](int key0, auto in_lds) __attribute__((always_inline)) {
+  auto fetch_from = [&](uint4 (&stage)[PER_THREAD], int key0, auto in_lds) __attribute__((always_inline)) {
     const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
     if constexpr (ROWWISE) {
       int key = key0 + kr, kb = key0 + 8 * vc;
@@ -434,15 +448,13 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
       }
     }
   };
-  auto fetch = [&](int key0) __attribute__((always_inline)) {
-    if (table_in_lds) fetch_from(key0, std::true_type{});
-    else fetch_from(key0, std::false_type{});
+  auto fetch = [&](uint4 (&stage)[PER_THREAD], int key0) __attribute__((always_inline)) {
+    if (table_in_lds) fetch_from(stage, key0, std::true_type{});
+    else fetch_from(stage, key0, std::false_type{});
   };
-  __syncthreads();   // the page numbers are in LDS
-  if (AHEAD && range_lo <= range_hi) fetch(range_lo);
-  for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
-    if (!AHEAD) fetch(key0);
-    __syncthreads();   // the last stage has been used
+  // the registers of a fetched stage into LDS, between two barriers: the last stage has been used; this one is there
+  auto to_lds = [&](const uint4 (&stage)[PER_THREAD]) __attribute__((always_inline)) {
+    __syncthreads();
     if constexpr (ROWWISE) {
 #pragma unroll
       for (int v = 0; v < PER_K; ++v) *reinterpret_cast<uint4*>(&ks[step_row(kr) * KP + 8 * (kc + KT * v)]) = stage[v];
@@ -462,10 +474,12 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
       }
     }
     __syncthreads();
-    if (AHEAD && key0 + kStageKeys <= range_hi) fetch(key0 + kStageKeys);
+  };
+  // this wave's keys of the stage that lies in LDS, 32 at a time
+  auto use_stage = [&](int key0) __attribute__((always_inline)) {
 #pragma unroll
     for (int sub = 0; sub < WAVE_KEYS / 32; ++sub) {
-      const int skey = WAVE_KEYS * wave + 32 * sub;     // this wave's keys of the stage, 32 at a time
+      const int skey = WAVE_KEYS * wave + 32 * sub;
       const int wkey = key0 + skey;
       if (has_head && wkey <= k_hi && wkey + 32 > k_lo) {
         KVStep<DT> r;
@@ -488,6 +502,15 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
         attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED), true>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
       }
     }
+  };
+  uint4 stage[PER_THREAD];
+  __syncthreads();   // the page numbers are in LDS
+  if (AHEAD && range_lo <= range_hi) fetch(stage, range_lo);
+  for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
+    if (!AHEAD) fetch(stage, key0);
+    to_lds(stage);
+    if (AHEAD && key0 + kStageKeys <= range_hi) fetch(stage, key0 + kStageKeys);
+    use_stage(key0);
   }
 
   // merge the waves of each team in turn: [wave][row][HD + 4] floats = (O^T row ..., maximum, sum, two unused).
