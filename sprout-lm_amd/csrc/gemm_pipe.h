@@ -54,6 +54,21 @@ __host__ __device__ inline PipeTiles pipe_tiles(int tiles_t, int tiles_n) {
   p.run = (p.left * tiles_t + 7) / 8;
   return p;
 }
+// The tile of block `block` of the 8 (own + run) blocks of a launch, or false for a block with nothing to do.
+__host__ __device__ inline bool pipe_tile_of(const PipeTiles& tiles, int block, int* tile_t, int* tile_n) {
+  const int xcd = block & 7, i_xcd = block >> 3;
+  if (i_xcd < tiles.own) {
+    const int g = i_xcd / (tiles.full * tiles.group), rest = i_xcd % (tiles.full * tiles.group);
+    *tile_n = (rest / tiles.group) * 8 + xcd;
+    *tile_t = g * tiles.group + rest % tiles.group;
+    return *tile_t < tiles.tiles_t;
+  }
+  const int j = i_xcd - tiles.own, k = xcd * tiles.run + j;
+  if (j >= tiles.run || k >= tiles.left * tiles.tiles_t) return false;
+  *tile_n = 8 * tiles.full + k / tiles.tiles_t;
+  *tile_t = k % tiles.tiles_t;
+  return true;
+}
 
 // A block of WAVES_M x WAVES_N waves, each with WM x WN tiles of 32 x 32: BM = 32 WM WAVES_M tokens by
 // BN = 32 WN WAVES_N weight rows.  Blocks of up to four waves ask for the registers of two waves a SIMD: with
@@ -81,19 +96,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   // multiple of 8 are dealt out by token tile, an equal run of their blocks to every XCD: four left-over weight
   // tiles would otherwise be a quarter more blocks on four of the XCDs, and fewer than 8 weight tiles idle XCDs.
   const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
-  const int xcd = blockIdx.x & 7, i_xcd = blockIdx.x >> 3;
   int tile_n, tile_t;
-  if (i_xcd < tiles.own) {
-    const int g = i_xcd / (tiles.full * tiles.group), rest = i_xcd % (tiles.full * tiles.group);
-    tile_n = (rest / tiles.group) * 8 + xcd;
-    tile_t = g * tiles.group + rest % tiles.group;
-    if (tile_t >= tiles.tiles_t) return;
-  } else {
-    const int j = i_xcd - tiles.own, k = xcd * tiles.run + j;
-    if (j >= tiles.run || k >= tiles.left * tiles.tiles_t) return;
-    tile_n = 8 * tiles.full + k / tiles.tiles_t;
-    tile_t = k % tiles.tiles_t;
-  }
+  if (!pipe_tile_of(tiles, blockIdx.x, &tile_t, &tile_n)) return;
   const int t0 = tile_t * BM, n0 = tile_n * BN;
   const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
   const int steps = (k_end - k_begin) / 64;

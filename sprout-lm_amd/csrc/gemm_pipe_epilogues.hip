@@ -81,6 +81,19 @@ extern "C" int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan) {
   return 0;
 }
 
+// The tile of every block of a launch over tiles_t token tiles and tiles_n weight tiles, as the kernel numbers them:
+// tile_of[2 b] = token tile and tile_of[2 b + 1] = weight tile of block b, both -1 for a block with nothing to do.
+// Returns the number of blocks (8 for each place on an XCD), or -1; writes at most `room` blocks.  Runs nothing.
+extern "C" int sp_pipe_tiles(int tiles_t, int tiles_n, int* tile_of, int room) {
+  using namespace sprout;
+  if (tiles_t < 1 || tiles_n < 1 || !tile_of) return -1;
+  const PipeTiles tiles = pipe_tiles(tiles_t, tiles_n);
+  const int blocks = 8 * (tiles.own + tiles.run);
+  for (int b = 0; b < blocks && b < room; ++b)
+    if (!pipe_tile_of(tiles, b, &tile_of[2 * b], &tile_of[2 * b + 1])) tile_of[2 * b] = tile_of[2 * b + 1] = -1;
+  return blocks;
+}
+
 namespace sprout {
 
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,

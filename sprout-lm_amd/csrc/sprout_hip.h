@@ -38,6 +38,9 @@ int sp_fused_norm_pays(int T, int N, int K);
 // waves of a block}.
 // Returns 1 where that kernel (for kind 3 its rotating epilogue) does not take the product.
 int sp_pipe_plan(int kind, int T, int N, int K, int hd, int* plan);
+// How that kernel numbers its blocks: tile_of[2 b], tile_of[2 b + 1] = token tile and weight tile of block b (which
+// runs on XCD b % 8), -1 for a block with nothing to do; returns the number of blocks.  Runs nothing.
+int sp_pipe_tiles(int tiles_t, int tiles_n, int* tile_of, int room);
 int sp_gemm_decode(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
                    const void* w, int bias_dtype, const void* bias, int mode, void* out, int T, int N, int K);
 // q, k, v projection (+ bias), rotation of q and k, q to q_out [T, nq * hd], k and v into the paged pools.

@@ -360,6 +360,19 @@ def pipe_plan(kind: int, T: int, N: int, K: int, hd: int = 0):
     return tuple(plan)
 
 
+def pipe_tiles(tiles_t: int, tiles_n: int) -> list:
+    """For every block of the tiled product's launch over tiles_t token tiles and tiles_n weight tiles, in the order
+    of the blocks (block b runs on XCD b % 8): (token tile, weight tile), or None for a block with nothing to do.
+    Runs nothing and needs no GPU."""
+    import ctypes
+    blocks = library().sp_pipe_tiles(tiles_t, tiles_n, (ctypes.c_int * 2)(), 0)
+    if blocks < 0:
+        raise KernelError(f"sp_pipe_tiles: no tiles for {tiles_t} x {tiles_n}")
+    out = (ctypes.c_int * (2 * blocks))()
+    library().sp_pipe_tiles(tiles_t, tiles_n, out, blocks)
+    return [None if out[2 * b] < 0 else (out[2 * b], out[2 * b + 1]) for b in range(blocks)]
+
+
 def _activations(x, residual, norm_weight, K: int, what: str):
     """Checks the two ways activations reach a fused kernel; returns (x ptr, residual ptr, norm dtype, norm ptr, T)."""
     if residual is not None:

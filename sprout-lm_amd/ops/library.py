@@ -33,6 +33,7 @@ def _declare(lib):
         "sp_fused_supported": [c_int] * 8,
         "sp_fused_norm_pays": [c_int] * 3,
         "sp_pipe_plan": [c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
+        "sp_pipe_tiles": [c_int, c_int, ctypes.POINTER(c_int), c_int],
         "sp_gemm_decode": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_void, c_int,
                            c_int, c_int],
         "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,

@@ -109,3 +109,29 @@ def test_kernel_tests_reach_every_block_shape():
              if m.name == "parametrize" and m.args[0] == "T,I,K"]
     gated = {ops.pipe_plan(ops.PLAN_GATED, T, 2 * I, K)[:2] for T, I, K in marks[0].args[1] if T > 64 and K % 64 == 0}
     assert gated >= {(64, 128), (128, 128), (256, 128), (256, 256), (384, 256)}, gated
+
+
+def test_blocks_are_numbered_so_that_every_tile_runs_once_and_the_xcds_share_them():
+    """The tiled product's numbering of its blocks (block b runs on XCD b % 8): every (token tile, weight tile) is
+    some block's, once; a weight tile of the whole eights lies on one XCD with all its token tiles (nobody else
+    fetches it); and no XCD holds more blocks than its even share of the left-over tiles, rounded up."""
+    for tiles_t in list(range(1, 20)) + [33, 64]:
+        for tiles_n in list(range(1, 41)) + [148, 149, 593]:
+            blocks = ops.pipe_tiles(tiles_t, tiles_n)
+            assert len(blocks) % 8 == 0
+            seen, per_xcd, home = {}, [0] * 8, {}
+            for b, tile in enumerate(blocks):
+                if tile is None:
+                    continue
+                t, n = tile
+                assert 0 <= t < tiles_t and 0 <= n < tiles_n and tile not in seen, (tiles_t, tiles_n, b, tile)
+                seen[tile] = b
+                per_xcd[b % 8] += 1
+                if n < tiles_n // 8 * 8:
+                    assert home.setdefault(n, b % 8) == b % 8 == n % 8, (tiles_t, tiles_n, b, tile)
+            assert len(seen) == tiles_t * tiles_n
+            left = tiles_n % 8
+            assert max(per_xcd) == tiles_n // 8 * tiles_t + -(-left * tiles_t // 8), (tiles_t, tiles_n, per_xcd)
+    with pytest.raises(ops.KernelError):
+        ops.pipe_tiles(0, 5)
+
