@@ -68,6 +68,8 @@ class _PrefixEntry:
     behind it)."""
     pages: list
     last_used: int
+    parent: bytes = b""        # key of the entry one page earlier in the chain
+    tokens: tuple = ()         # the page's own tokens: a hit is believed only if they, and the parent, are the same
 
 
 class CacheManager:
@@ -133,17 +135,29 @@ class CacheManager:
         """A state slot that no request ever holds (the last row of every state tensor)."""
         return self.max_sequences
 
+    @staticmethod
+    def pool_bytes(slot_specs, block_size: int, num_blocks: int, max_sequences: int, element_size: int) -> int:
+        """Device bytes of the pools and state tensors that a manager of these options would allocate for cache
+        elements of `element_size` bytes.  Plain arithmetic on the specs: nothing is built, so an absurd option
+        costs nothing before the memory budget refuses it."""
+        total = 0
+        for spec in slot_specs:
+            if isinstance(spec, PagedKVSpec):
+                # every pool holds num_blocks * block_size tokens, whatever its page size
+                total += 2 * num_blocks * block_size * spec.kv_heads * spec.head_dim * element_size
+            elif isinstance(spec, StateSpec):
+                count = 1
+                for n in spec.shape:
+                    count *= n
+                total += (max_sequences + 1) * count * _DTYPE_BYTES.get(spec.dtype, 4)
+            else:
+                raise TypeError(f"Unknown cache spec {spec!r}.")
+        return total
+
     def storage_bytes(self, element_size: int) -> int:
         """Device bytes of every pool and state tensor for cache elements of `element_size` bytes."""
-        total = 0
-        for g in self.groups:
-            total += 2 * len(g.slots) * g.pool.num_pages * g.spec.kv_heads * g.page_tokens * g.spec.head_dim * element_size
-        for g in self.state_groups:
-            count = 1
-            for n in g.spec.shape:
-                count *= n
-            total += len(g.slots) * (self.max_sequences + 1) * count * _DTYPE_BYTES.get(g.spec.dtype, 4)
-        return total
+        specs = [g.spec for g in self.groups for _ in g.slots] + [g.spec for g in self.state_groups for _ in g.slots]
+        return self.pool_bytes(specs, self.block_size, self.num_blocks, self.max_sequences, element_size)
 
     # ------------------------------------------------------------------ sequences
     def create(self) -> SequenceCache:
@@ -174,9 +188,11 @@ class CacheManager:
         keys, entries = [], []
         end = bs
         while end < len(tokens):
-            key = self._chain(key, tokens[end - bs:end])
+            parent, key = key, self._chain(key, tokens[end - bs:end])
             entry = self._prefixes.get(key)
-            if entry is None:
+            # The reference keys its index by the tokens themselves (src/kv-cache.ts:103,118) and cannot take one
+            # prefix for another; a hash can, so a hit also has to show the same tokens behind the same parent.
+            if entry is None or entry.parent != parent or entry.tokens != tuple(tokens[end - bs:end]):
                 break
             keys.append(key)
             entries.append(entry)
@@ -229,8 +245,8 @@ class CacheManager:
             parent = seq.prefix_keys[-1] if seq.prefix_keys else b""
             seq.prefix_keys.append(self._chain(parent, tokens[i * bs:(i + 1) * bs]))
         key = seq.prefix_keys[n_pages - 1]
-        if key in self._prefixes:
-            return
+        parent = seq.prefix_keys[n_pages - 2] if n_pages > 1 else b""
+        mine_tokens = tuple(tokens[(n_pages - 1) * bs:n_pages * bs])
         # every group's pages of these `bs` tokens (a window may already have passed some of them, when a long
         # portion was computed in one step: then the entry holds none of that group)
         pages = []
@@ -238,11 +254,23 @@ class CacheManager:
             per = bs // g.page_tokens
             mine = blocks[(n_pages - 1) * per:n_pages * per]
             pages.append(None if FREED in mine else list(mine))
+        known = self._prefixes.get(key)
+        if known is not None:
+            # The first publisher wins.  Where the entry has meanwhile given a windowed group's pages back (pool
+            # pressure), a later publisher of the same tokens puts its own there, or that prefix would stay
+            # half-shared for as long as its chain is in use.
+            if known.parent == parent and known.tokens == mine_tokens:
+                for gi, (g, mine) in enumerate(zip(self.groups, pages)):
+                    if known.pages[gi] is None and mine is not None:
+                        for page in mine:
+                            g.pool.retain(page)
+                        known.pages[gi] = mine
+            return
         for g, mine in zip(self.groups, pages):
             for page in mine or ():
                 g.pool.retain(page)   # the cache's own reference, beside the live requests'
         self._clock += 1
-        self._prefixes[key] = _PrefixEntry(pages, self._clock)
+        self._prefixes[key] = _PrefixEntry(pages, self._clock, parent, mine_tokens)
 
     def _evict_one(self, group: int | None = None) -> bool:
         """Make a page free: drop the least recently used prefix entry that only the cache still holds.  For a

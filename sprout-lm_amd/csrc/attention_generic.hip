@@ -35,7 +35,7 @@ struct Divider {
 
 struct TileSource {
   const int32_t* bt;
-  int nkv, g, hd, page_size, num_pages, k_lo, k_end;
+  int nkv, g, hd, page_size, num_pages, max_blocks, k_lo, k_end;
   Divider by_hd, by_page;
 };
 
@@ -52,7 +52,7 @@ __device__ __forceinline__ void load_tile(const TileSource& src, const T* __rest
       if (j >= src.k_lo && j < src.k_end) {
         int logical, slot;
         src.by_page.divmod(j, logical, slot);
-        const int page = src.bt[logical];
+        const int page = logical < src.max_blocks ? src.bt[logical] : -1;   // never past the sequence's table row
         if (page >= 0 && page < src.num_pages) {
           const size_t base = (size_t(page) * src.nkv + src.g) * src.page_size * src.hd;
           v = to_float(pool[base + (VALUES ? size_t(d) * src.page_size + slot : size_t(slot) * src.hd + d)]);
@@ -112,8 +112,9 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   const int my_pos = GROUPED ? pos0 : pos0 + r;
   TileSource src;
   src.bt = block_tables + size_t(seq) * max_blocks;
-  src.nkv = nkv; src.g = GROUPED ? blockIdx.y : blockIdx.y / G; src.hd = hd; src.page_size = page_size; src.num_pages = num_pages;
-  src.k_end = pos0 + nvalid;  // one past the last visible key of the tile
+  src.nkv = nkv; src.g = GROUPED ? blockIdx.y : blockIdx.y / G; src.hd = hd; src.page_size = page_size; src.num_pages = num_pages; src.max_blocks = max_blocks;
+  // one past the last visible key of the tile (GROUPED: its rows are heads of one query, at pos0)
+  src.k_end = pos0 + (GROUPED ? 1 : nvalid);
   src.k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int n_chunks = gridDim.z, first_key = blockIdx.z * chunk;   // this block's keys: first_key .. + chunk - 1
   if (blockIdx.z + 1 < n_chunks) src.k_end = min(src.k_end, first_key + chunk);   // the last chunk: all that is left

@@ -1,4 +1,4 @@
-// Embedding gather, RMSNorm, SiLU-gated product, casts, and rotation + cache write.
+// Embedding gather, RMSNorm, SiLU-gated product, and rotation + cache write.
 // All arithmetic is float32; only loads and stores see the storage type.
 #include "common.h"
 #include "sprout_hip.h"
@@ -89,14 +89,6 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   const float u = to_float(gu[size_t(t) * 2 * I + I + i]);
   const float s = g / (1.0f + expf(-g));
   out[size_t(t) * I + i] = from_float<T>(s * u);
-}
-
-// ---------------------------------------------------------------- cast
-template <typename TS, typename TD>
-__global__ void cast_kernel(const TS* __restrict__ src, TD* __restrict__ dst, int64_t n) {
-  int64_t i = int64_t(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t step = int64_t(gridDim.x) * blockDim.x;
-  for (; i < n; i += step) dst[i] = from_float<TD>(to_float(src[i]));
 }
 
 // ---------------------------------------------------------------- rotation + cache write
@@ -297,20 +289,6 @@ extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, i
   else if (dtype == kBF16) silu_mul_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, I);
   else SP_REQUIRE(false, "sp_silu_mul: unsupported dtype %d", dtype);
   return check_launch("sp_silu_mul");
-}
-
-extern "C" int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n) {
-  SP_REQUIRE(n >= 0, "sp_cast: bad size");
-  if (n == 0) return 0;
-  hipStream_t s = (hipStream_t)stream;
-  const int blocks = (int)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
-  if (src_dtype == kF32 && dst_dtype == kBF16)
-    cast_kernel<float, bf16_t><<<blocks, 256, 0, s>>>((const float*)src, (bf16_t*)dst, n);
-  else if (src_dtype == kBF16 && dst_dtype == kF32)
-    cast_kernel<bf16_t, float><<<blocks, 256, 0, s>>>((const bf16_t*)src, (float*)dst, n);
-  else
-    SP_REQUIRE(false, "sp_cast: unsupported dtypes %d -> %d", src_dtype, dst_dtype);
-  return check_launch("sp_cast");
 }
 
 extern "C" int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T) {

@@ -108,7 +108,6 @@ int sp_attention_decode_project(void* stream, const void* q, int q_stride, const
 int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation);
 
 // dst (dst_dtype) = src (src_dtype), n elements
-int sp_cast(void* stream, int src_dtype, const void* src, int dst_dtype, void* dst, int64_t n);
 
 // tokens[i] = previous[source[i]] for every i < n with source[i] >= 0 (others are left as they are):
 // feeds tokens sampled by a step that the host has not read yet into the next step.  previous holds at

@@ -60,11 +60,14 @@ class Workspace:
 
 class KeptWorkspace(Workspace):
     """Scratch tensors for recorded graphs that share them: a graph holds the addresses it was recorded with, so
-    a tensor is never freed or moved; a request that none of a name's tensors can hold gets a further one."""
+    a tensor is never moved, and freed only when every graph that used it has been given up (`release`); a request
+    that none of a name's tensors can hold gets a further one.  `owner` names the graph that is asking."""
 
     def __init__(self, device):
         super().__init__(device)
         self._kept: dict[tuple[str, torch.dtype], list[torch.Tensor]] = {}
+        self._users: dict[int, set] = {}      # id(tensor) -> owners that were handed it
+        self.owner = None
 
     def get(self, name: str, shape, dtype) -> torch.Tensor:
         n = 1
@@ -78,10 +81,42 @@ class KeptWorkspace(Workspace):
                 raise RuntimeError(f"Workspace buffer {name!r} would grow while a graph is recorded.")
             flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._kept.setdefault((name, dtype), []).append(flat)
+        self._users.setdefault(id(flat), set()).add(self.owner)
         return flat[:n].view(shape)
+
+    def release(self, owner) -> None:
+        """`owner`'s graph is gone (and the stream has been waited for): free what no other graph uses."""
+        for key, kept in list(self._kept.items()):
+            for flat in list(kept):
+                users = self._users.get(id(flat), set())
+                users.discard(owner)
+                if not users:
+                    kept.remove(flat)
+                    self._users.pop(id(flat), None)
+            if not kept:
+                del self._kept[key]
 
     def nbytes(self) -> int:
         return sum(t.numel() * t.element_size() for kept in self._kept.values() for t in kept)
+
+
+class OwnedNames:
+    """A workspace that keeps the named buffers for itself and asks `shared` for every other: what a recorded step
+    returns to its caller (the logits) must not be overwritten by the next recorded step of another shape."""
+
+    def __init__(self, shared: Workspace, own: tuple, device):
+        self.shared, self.own, self.private = shared, own, Workspace(device)
+
+    @property
+    def frozen(self):
+        return self.shared.frozen
+
+    @frozen.setter
+    def frozen(self, value):
+        self.shared.frozen = self.private.frozen = value
+
+    def get(self, name: str, shape, dtype) -> torch.Tensor:
+        return (self.private if name in self.own else self.shared).get(name, shape, dtype)
 
 
 class StepContext:

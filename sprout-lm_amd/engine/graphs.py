@@ -20,13 +20,14 @@ step's (`batch.step_arrays`).
 from __future__ import annotations
 
 import gc
+import itertools
 import weakref
 
 import numpy as np
 import torch
 
 from .. import ops
-from .batch import CacheSlotView, KeptWorkspace, StepContext, Workspace, context_from, step_arrays
+from .batch import CacheSlotView, KeptWorkspace, OwnedNames, StepContext, Workspace, context_from, step_arrays
 
 
 def _bucket(n: int, floor: int = 1) -> int:
@@ -180,7 +181,10 @@ class _DecodeGraph:
 class _PortionGraph:
     """Static buffers and the recorded graph of one step shape with portions of prompts in it."""
 
+    _uids = itertools.count(1)
+
     def __init__(self, runner, first, ctx_bucket: int, workspace):
+        self.uid = next(self._uids)          # names this graph to the shared workspace
         self.runner = runner if isinstance(runner, weakref.ProxyTypes) else weakref.proxy(runner)
         cache = runner.cache
         self.last_used = 0
@@ -198,8 +202,10 @@ class _PortionGraph:
         # run one after the other on one stream, and `workspace` never frees or moves a tensor).  The longest
         # context is known to the kernels as its bucket only (how a long walk is shared out follows it), and the
         # step has no values on the host.
-        self.ctx = context_from(first, views, len(cache.groups), workspace, runner.dtype,
-                                runner.attention_kind, max_decode_ctx=ctx_bucket, max_ctx=ctx_bucket)
+        # The logits are what the caller gets: they live in a tensor of this graph's own.
+        self.shared_workspace = workspace
+        self.ctx = context_from(first, views, len(cache.groups), OwnedNames(workspace, ("logits",), runner.device),
+                                runner.dtype, runner.attention_kind, max_decode_ctx=ctx_bucket, max_ctx=ctx_bucket)
         self.ctx.host = {}
         self.copied = None
         self.graph = None
@@ -225,6 +231,7 @@ class _PortionGraph:
 
     def _body(self):
         self.ctx.shared.clear()            # see _DecodeGraph._body
+        self.shared_workspace.owner = self.uid
         self.logits = self.runner.forward(self.ctx)
 
 
@@ -279,7 +286,7 @@ class DecodeGraphs:
     def portion_step(self, entries, record_at: int = 2):
         """Run a step that is not one token a request from a recorded graph, if its shape has been seen
         `record_at` times (the step that reaches the count is the one recorded).  Returns the float32 logits
-        at the wanted places (the graph's own buffer: valid until the same shape runs again), or None if the step
+        at the wanted places (the graph's own tensor: valid until the same shape runs again), or None if the step
         is not taken this way: then nothing was launched.  The sequences' lengths are advanced."""
         runner = self.runner
         if not runner.parts.graph_safe_portions or not entries:
@@ -302,7 +309,7 @@ class DecodeGraphs:
                 if self.portion_steps - self.portion_graphs[oldest].last_used < self.keep_recent:
                     return None
                 torch.cuda.current_stream().synchronize()
-                self.portion_graphs.pop(oldest)
+                self._portion_workspace.release(self.portion_graphs.pop(oldest).uid)
         step = step_arrays(entries, runner.cache, table_tokens=bucket)
         if state is None:
             if self._portion_workspace is None:

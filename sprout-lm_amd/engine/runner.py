@@ -77,7 +77,7 @@ class ModelRunner:
         """Count the weights and the cache pools of a model that is not loaded yet against the device's free
         memory; raises MemoryBudgetError if they do not fit.  Returns (weight bytes, pool bytes)."""
         weights = weight_bytes(parts.expected_tensors(), dtype, stored)
-        pools = CacheManager(parts.cache_slot_specs, block_size, num_blocks, max_sequences, False).storage_bytes(dtype.itemsize)
+        pools = CacheManager.pool_bytes(parts.cache_slot_specs, block_size, num_blocks, max_sequences, dtype.itemsize)
         check_budget(weights, pools, free_device_bytes(device), budget)
         return weights, pools
 
@@ -214,8 +214,8 @@ class ModelRunner:
 
     def step_recorded(self, entries: list[StepEntry], record_at: int = 2):
         """`step` from a recorded graph of the step's shape, where there is one or the shape has now come
-        `record_at` times; None otherwise (nothing has been run then).  The logits lie in the graph's own buffer
-        and are overwritten when the same shape runs again."""
+        `record_at` times; None otherwise (nothing has been run then).  The logits lie in a tensor of that graph's
+        own: they stay until a step of the same shape runs again, whatever other steps run meanwhile."""
         if not self.use_graphs or not self.record_portions or not self.parts.graph_safe_portions:
             return None
         self.validate(entries)

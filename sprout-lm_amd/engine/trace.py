@@ -10,9 +10,12 @@ Steps are read from standard input, one JSON object a line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
 
 For a step in which logits are wanted, `<out>/<step>.f32` holds them as little-endian float32
-[wanted, vocab], in the order of the entries and of `want`.  After every step the line
-`done <step>` is printed.  The analogue in the reference is scripts/reference.py:20-44, which
-writes last-position logits of whole sequences.
+[wanted, vocab], in the order of the entries and of `want`, and `<out>/index.jsonl` gains a line
+`{"step": s, "file": "<s>.f32", "rows": [{"row": r, "request": id, "position": p}, ...]}` that says which
+request and which position of it every row belongs to (the reference's reference.json does the same for
+its files, scripts/reference.py:39-43).  After every step the line `done <step>` is printed.  The
+analogue in the reference is scripts/reference.py:20-44, which writes last-position logits of whole
+sequences.
 """
 from __future__ import annotations
 
@@ -34,12 +37,14 @@ class TraceSession:
     def __init__(self, runner):
         self.runner = runner
         self.live = {}
+        self.last_rows = []
 
     def run_step(self, record):
         """Run the step's entries as one batch, free what `end` names; returns the logits or None."""
         from .batch import StepEntry
         cache = self.runner.cache
         entries = []
+        self.last_rows = []       # (request, position) of every wanted row of this step, in the order of the logits
         for item in record.get("entries", []):
             seq = self.live.get(item["id"])
             if seq is None:
@@ -47,7 +52,9 @@ class TraceSession:
             tokens = [int(t) for t in item["tokens"]]
             if not cache.reserve(seq, seq.length + len(tokens)):
                 raise PoolTooSmall(item["id"])
-            entries.append(StepEntry(seq, tokens, [int(w) for w in item.get("want", [])]))
+            want = [int(w) for w in item.get("want", [])]
+            self.last_rows += [(item["id"], seq.length + w) for w in want]
+            entries.append(StepEntry(seq, tokens, want))
         logits = None
         if entries:
             # as generation runs a step: from a recorded graph where the step's shape has come before
@@ -88,6 +95,7 @@ def main(argv=None) -> int:
           file=sys.stderr, flush=True)
 
     session = TraceSession(runner)
+    index = open(os.path.join(args.out, "index.jsonl"), "w")
     while True:
         line = sys.stdin.readline()   # one line at a time: the next step comes only after `done`
         if not line:
@@ -105,6 +113,9 @@ def main(argv=None) -> int:
         if logits is not None and logits.shape[0]:
             host = logits.to("cpu", copy=True).numpy().astype("<f4", copy=False)
             host.tofile(os.path.join(args.out, f"{record['step']}.f32"))
+            rows = [{"row": r, "request": rid, "position": pos} for r, (rid, pos) in enumerate(session.last_rows)]
+            index.write(json.dumps({"step": record["step"], "file": f"{record['step']}.f32", "rows": rows}) + "\n")
+            index.flush()
         else:
             torch.cuda.current_stream().synchronize()
         print(f"done {record['step']}", flush=True)

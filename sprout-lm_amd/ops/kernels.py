@@ -285,7 +285,10 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
             raise KernelError("attention: without a decode list every sequence must bring one query")
         if max_decode_ctx > block_tables.shape[1] * page_size:
             raise KernelError("attention: a decode context is longer than its block table")
-    max_tile_ctx = min(batch.max_ctx, block_tables.shape[1] * page_size) if n_tiles else 0
+    if n_tiles and batch.max_ctx > block_tables.shape[1] * page_size:
+        raise KernelError(f"attention: a context of {batch.max_ctx} tokens is longer than its block table "
+                          f"({block_tables.shape[1]} pages of {page_size})")
+    max_tile_ctx = batch.max_ctx if n_tiles else 0
     if one_query_each:
         n_decode = n_tiles
     need = library().sp_attention_workspace_floats(_code(q, "q"), hd, page_size, nq, nkv, kind, n_decode, max_decode_ctx,
@@ -446,14 +449,6 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> N
         raise KernelError(f"silu_mul: shapes do not fit: gu {tuple(gu.shape)}, out {tuple(out.shape)}")
     check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I,
                                 variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
-
-
-def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
-    _gpu(src, "cast source"); _gpu(dst, "cast destination")
-    if src.numel() != dst.numel():
-        raise KernelError("cast: sizes differ")
-    check(library().sp_cast(_stream(), _code(src, "cast source"), src.data_ptr(), _code(dst, "cast destination"),
-                            dst.data_ptr(), src.numel()))
 
 
 def sample_workspace_floats(rows: int, vocab: int) -> int:

@@ -41,7 +41,6 @@ def _declare(lib):
         "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
         "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
         "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int, c_int],
-        "sp_cast": [c_void, c_int, c_void, c_int, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
         "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],

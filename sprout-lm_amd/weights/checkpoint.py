@@ -36,7 +36,10 @@ class Checkpoint:
                 for name in file.names():
                     if mapping.get(name) == shard:
                         self._infos[name] = (shard, file.info(name))
-            self.missing_in_shards = sorted(n for n in mapping if n not in self._infos)
+            absent = sorted(n for n in mapping if n not in self._infos)
+            if absent:
+                raise SafetensorsError(f"The shard index of {self.folder!r} names {len(absent)} tensors that their shards "
+                                       f"do not hold: " + ", ".join(absent[:8]) + (" ..." if len(absent) > 8 else ""))
         else:
             single = os.path.join(self.folder, "model.safetensors")
             if not os.path.exists(single):
@@ -44,7 +47,6 @@ class Checkpoint:
             file = self._file("model.safetensors")
             for name in file.names():
                 self._infos[name] = ("model.safetensors", file.info(name))
-            self.missing_in_shards = []
 
     def _file(self, shard: str) -> SafetensorsFile:
         file = self._open.get(shard)

@@ -89,8 +89,16 @@ def load_named_tensors(folder: str, expected: dict[str, TensorSpec], ignorable: 
         if unexpected and notes is not None:
             notes.append(f"{len(unexpected)} tensors of the checkpoint are not part of the model and were left "
                          f"unread: " + ", ".join(unexpected[:8]) + (" ..." if len(unexpected) > 8 else ""))
+        stored = {name: ckpt.dtype(name) for name in expected}
+        rounded = sorted(n for n, d in stored.items() if d == torch.float16 and compute == torch.bfloat16
+                         and expected[n].kind != "int_table")
+        if rounded and notes is not None:
+            # float32 compute widens float16 exactly (reference: src/safetensors.ts:91-101); bfloat16 compute keeps
+            # 16-bit tensors in bfloat16, which has three mantissa bits fewer than float16
+            notes.append(f"{len(rounded)} tensors stored in float16 were rounded to bfloat16 for bfloat16 compute: "
+                         + ", ".join(rounded[:8]) + (" ..." if len(rounded) > 8 else ""))
         if before_read is not None:
-            before_read({name: ckpt.dtype(name) for name in expected})
+            before_read(stored)
         out = {}
         for name, spec in expected.items():
             # straight from the file's mapping to the device: no copy on the host in between

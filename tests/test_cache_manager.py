@@ -23,8 +23,8 @@ def invariants(cache: CacheManager):
         for entry in cache._prefixes.values():
             for page in entry.pages[gi] or ():
                 held[page] = held.get(page, 0) + 1
-        free = list(g.pool._free)
-        assert len(free) == len(set(free)), "a page is on the free list twice"
+        free = g.pool.free_list()
+        assert len(free) == len(set(free)) == g.pool.num_free, "a page is on the free list twice"
         for page in range(g.pool.num_pages):
             assert g.pool.refs[page] == held.get(page, 0), f"page {page}: refs {g.pool.refs[page]} held {held.get(page, 0)}"
             assert (page in free) == (g.pool.refs[page] == 0)
@@ -39,6 +39,21 @@ def test_pool_hands_out_page_zero_first_and_reuses_last_freed():
         pool.release(1); pool.release(1)
     with pytest.raises(PageError):
         PagePool(2).retain(0)
+
+
+def test_a_pool_costs_what_it_has_handed_out_not_what_it_could():
+    """A pool of two billion pages (a mistyped option) is built at once and without memory for its pages: the
+    memory budget is what refuses it, and it has to get that far."""
+    import time
+    start = time.time()
+    pool = PagePool(2_000_000_000)
+    assert pool.num_free == 2_000_000_000 and pool.refs[1_999_999_999] == 0 and len(pool.refs) == 2_000_000_000
+    assert [pool.allocate() for _ in range(3)] == [0, 1, 2]
+    pool.release(1)
+    assert pool.num_free == 1_999_999_998 and pool.allocate() == 1 and pool.allocate() == 3
+    cache = CacheManager([FULL, WINDOWED], block_size=16, num_blocks=2_000_000_000, max_sequences=4)
+    assert cache.storage_bytes(2) == CacheManager.pool_bytes([FULL, WINDOWED], 16, 2_000_000_000, 4, 2)
+    assert time.time() - start < 1.0
 
 
 def test_reserve_is_all_or_nothing_over_groups():
@@ -197,6 +212,52 @@ def test_a_short_windowed_pool_takes_cached_pages_back_one_at_a_time():
         seq.release()
     cache.clear_prefixes()
     assert cache.free_pages() == [6]
+
+
+def test_a_prefix_published_again_restores_the_pages_an_entry_gave_back():
+    """An entry that gave a windowed group's page back under pressure stays in its chain.  When a later request
+    computes the same tokens and offers the page again, the entry takes the new page, and the prefix is shared
+    whole again."""
+    cache = CacheManager([WINDOWED], block_size=4, num_blocks=8, max_sequences=3)
+    tokens = list(range(16))
+    a = cache.create()
+    feed(cache, a, tokens, portion=4)
+    a.release()
+    b = cache.create()
+    assert cache.reserve(b, 20)                               # one page more than are free: the oldest entry gives its own
+    b.release()
+    assert sum(e.pages == [None] for e in cache._prefixes.values()) == 1
+    assert cache.reuse_prefix(tokens).length == 0             # a window at key 12 needs page 0, which is gone
+    for seq in list(cache.live):
+        seq.release()
+    again = cache.create()
+    feed(cache, again, tokens, portion=4)                     # computes and offers the same four pages
+    assert all(e.pages != [None] for e in cache._prefixes.values())
+    invariants(cache)
+    again.release()
+    assert cache.reuse_prefix(tokens).length == 12
+    invariants(cache)
+    for seq in list(cache.live):
+        seq.release()
+    cache.clear_prefixes()
+    assert cache.free_pages() == [8]
+
+
+def test_a_prefix_hit_is_believed_only_with_the_same_tokens(monkeypatch):
+    """The index is keyed by a hash; a hit is taken only if the entry holds the very tokens behind the very
+    parent (the reference keys by the tokens themselves, src/kv-cache.ts:103,118).  With a hash that maps
+    everything to one value, other prompts share nothing, and the same prompt still shares."""
+    monkeypatch.setattr(CacheManager, "_chain", staticmethod(lambda parent, tokens: b"same"))
+    cache = CacheManager([FULL], block_size=4, num_blocks=8, max_sequences=4)
+    tokens = [1, 2, 3, 4, 5]
+    a = cache.create()
+    feed(cache, a, tokens, portion=5)
+    assert len(cache._prefixes) == 1
+    assert cache.reuse_prefix([9, 9, 9, 9, 5]).length == 0
+    assert cache.reuse_prefix([1, 2, 3, 4, 9]).length == 4
+    # a second page hashes to the same key: it is not the first page's entry, and is not taken for it
+    assert cache.reuse_prefix([1, 2, 3, 4, 1, 2, 3, 4, 0]).length == 4
+    invariants(cache)
 
 
 def test_lru_eviction_takes_only_pages_no_request_uses():

@@ -152,7 +152,7 @@ def test_rmsnorm(H, out_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_embed_and_silu_mul_and_cast(dtype):
+def test_embed_and_silu_mul(dtype):
     from sprout_lm_amd import ops
     rng = np.random.default_rng(1)
     table = rng.standard_normal((331, 70)).astype(np.float32)
@@ -169,10 +169,6 @@ def test_embed_and_silu_mul_and_cast(dtype):
     want = g / (1 + np.exp(-g)) * u
     tol = 1e-6 if dtype == torch.float32 else 2 ** -8
     assert np.abs(out.float().cpu().numpy() - want).max() <= tol * (1 + np.abs(want).max())
-    src = t(rng.standard_normal(1001).astype(np.float32))
-    dst = torch.empty(1001, dtype=torch.bfloat16, device=DEV)
-    ops.cast(src, dst)
-    assert torch.equal(dst, src.to(torch.bfloat16))
 
 
 def plain_rope(x, pos, hd, rotary, theta):

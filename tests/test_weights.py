@@ -201,6 +201,31 @@ def test_sharded_checkpoint_equals_single_file(tmp_path):
     plan = S.build_model_plan(S.load_config(str(shard_dir)))
     with pytest.raises(WeightError, match=names[0].replace(".", r"\.")):
         load_named_tensors(str(shard_dir), plan.expected_tensors(), set(), torch.float32, "cpu")
+    # a name that the index maps to a shard which does not hold it
+    bad = dict(weight_map)
+    bad[names[0]] = "model-00002-of-00002.safetensors"
+    (shard_dir / "model.safetensors.index.json").write_text(json.dumps({"weight_map": bad}))
+    with pytest.raises(SafetensorsError, match="names 1 tensors that their shards do not hold: " + names[0].replace(".", r"\.")):
+        Checkpoint(str(shard_dir))
     (shard_dir / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"a": "../evil.safetensors"}}))
     with pytest.raises(SafetensorsError, match="shard filename"):
         Checkpoint(str(shard_dir))
+
+
+def test_float16_tensors_widen_exactly_in_float32_and_are_noted_when_rounded_to_bfloat16(tmp_path):
+    """float32 compute widens float16 exactly (reference: src/safetensors.ts:91-101); bfloat16 compute keeps 16-bit
+    tensors in bfloat16, which loses three mantissa bits of a float16: the load says so."""
+    from safetensors.torch import load_file, save_file
+    folder = model_folder(tmp_path, "A")
+    path = os.path.join(folder, "model.safetensors")
+    tensors = {n: t.to(torch.float16) for n, t in load_file(path).items()}
+    name = "model.layers.0.mlp.down_proj.weight"
+    tensors[name][0, 0] = 1.0 + 2.0 ** -10          # a float16 that bfloat16 cannot hold
+    save_file(tensors, path)
+    plan = S.build_model_plan(S.load_config(folder))
+    notes = []
+    exact = load_named_tensors(folder, plan.expected_tensors(), set(), torch.float32, "cpu", notes=notes)
+    assert not notes and exact[name][0, 0].item() == 1.0 + 2.0 ** -10
+    rounded = load_named_tensors(folder, plan.expected_tensors(), set(), torch.bfloat16, "cpu", notes=notes)
+    assert rounded[name].dtype == torch.bfloat16 and rounded[name][0, 0].item() == 1.0
+    assert len(notes) == 1 and "stored in float16 were rounded to bfloat16" in notes[0] and str(len(tensors)) in notes[0]
