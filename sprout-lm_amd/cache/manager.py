@@ -25,7 +25,7 @@ class PagedGroup:
     pool: PagePool
     page_tokens: int = 0          # tokens in one page of this group
     k: object = None              # device tensor [len(slots), pages, kv_heads, page_size, head_dim]
-    v: object = None              # device tensor [len(slots), pages, kv_heads, head_dim, page_size]
+    v: object = None              # device tensor [len(slots), pages, kv_heads, value_dim or head_dim, page_size]
 
 
 @dataclass
@@ -105,9 +105,10 @@ class CacheManager:
                 g = len(groups) - 1
             groups[g].slots.append(slot)
             self.slot_location.append((kind, g, len(groups[g].slots) - 1))
-        # Pages may be shared between requests unless per-request state would have to be rebuilt with them: a
-        # state is no function of pages.  A group with a window shares the pages its window still covers.
-        self.prefix_caching = bool(prefix_caching and self.groups and not self.state_groups)
+        # Whether pages may be shared between requests is the caller's decision (a model whose parts keep per-request
+        # state that is no function of pages says no); there must be pages to share.  A group with a window
+        # shares the pages its window still covers.
+        self.prefix_caching = bool(prefix_caching and self.groups)
         self._prefixes: dict[bytes, _PrefixEntry] = {}
         self._clock = 0
         self.evictions = 0
@@ -121,9 +122,10 @@ class CacheManager:
         for g in self.groups:
             # keys [slot, page, head, token, dim]; values [slot, page, head, dim, token]: the keys of one
             # dimension lie together, which is how the P.V matrix product reads them
-            n, kv, hd = len(g.slots), g.spec.kv_heads, g.spec.head_dim
-            g.k = torch.zeros((n, g.pool.num_pages, kv, g.page_tokens, hd), dtype=dtype, device=device)
-            g.v = torch.zeros((n, g.pool.num_pages, kv, hd, g.page_tokens), dtype=dtype, device=device)
+            n, kv, hd, vd = len(g.slots), g.spec.kv_heads, g.spec.head_dim, g.spec.value_dim or g.spec.head_dim
+            kept = dtype if g.spec.dtype is None else getattr(torch, g.spec.dtype)
+            g.k = torch.zeros((n, g.pool.num_pages, kv, g.page_tokens, hd), dtype=kept, device=device)
+            g.v = torch.zeros((n, g.pool.num_pages, kv, vd, g.page_tokens), dtype=kept, device=device)
         for g in self.state_groups:
             # one slot more than requests can hold: `spare_state_slot`, where the padding rows of a recorded
             # step keep their state, so that no part has to tell them from real rows
@@ -144,7 +146,8 @@ class CacheManager:
         for spec in slot_specs:
             if isinstance(spec, PagedKVSpec):
                 # every pool holds num_blocks * block_size tokens, whatever its page size
-                total += 2 * num_blocks * block_size * spec.kv_heads * spec.head_dim * element_size
+                size = element_size if spec.dtype is None else _DTYPE_BYTES[spec.dtype]
+                total += num_blocks * block_size * spec.kv_heads * (spec.head_dim + (spec.value_dim or spec.head_dim)) * size
             elif isinstance(spec, StateSpec):
                 count = 1
                 for n in spec.shape:

@@ -110,6 +110,12 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 // dst (dst_dtype) = src (src_dtype), n elements
 
 // tokens[i] = previous[source[i]] for every i < n with source[i] >= 0 (others are left as they are):
+// dst[i] = a seeded random value, a function of (key, first + i) alone: the sum of twelve 16-bit fields of three
+// 64-bit hashes, centred, times scale (+ offset if add_offset): near normal with deviation 65536 * scale.
+// weights/random_init.py computes the same numbers on the host.
+int sp_random_fill(void* stream, int dtype, void* dst, int64_t n, uint64_t key, int64_t first, float scale,
+                   float offset, int add_offset);
+
 // feeds tokens sampled by a step that the host has not read yet into the next step.  previous holds at
 // least max(source) + 1 entries; a value outside [0, vocab) is replaced by 0.
 int sp_feed_tokens(void* stream, int32_t* tokens, const int32_t* previous, const int32_t* source, int n, int vocab);

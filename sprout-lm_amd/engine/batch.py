@@ -131,6 +131,7 @@ class StepContext:
         self.attention = None   # ops.AttentionBatch of this step
         self.group_tables: list[torch.Tensor] = []
         self.group_slots: list[torch.Tensor] = []
+        self.extra = {}  # arrays that parts have registered (register_step_array), by name, on the device
         self.host = {}   # the same arrays on the host (numpy), for parts that plan on the CPU
         self.shared = {}   # what a part computes once per step for all layers (key chosen by the part)
 
@@ -173,6 +174,59 @@ class DescriptorStager:
         return [self._dev[i][off:off + n].view(a.shape) for a, off, n in zip(arrays, offsets, sizes)]
 
 
+# The integer arrays of every step, in staging order; each has one entry per token or per sequence.  The recorded
+# decode steps lay their static buffers out from this list too (engine.graphs), so an array is named once.
+STEP_ARRAY_NAMES = ("token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots", "seq_of_token")
+
+# Arrays that parts add to every step: name -> (per, function of a StepLayout, value of padded rows).
+_EXTRA_ARRAYS: dict[str, tuple[str, object, int]] = {}
+
+
+def register_step_array(name: str, per: str, build, pad: int = 0) -> None:
+    """Add an int32 array to every step from now on: `build(layout)` returns one entry per token (`per` "token")
+    or per sequence ("sequence") of the step described by `layout` (a StepLayout).  Parts find its device copy
+    in `ctx.extra[name]`, in eager steps and recorded ones alike; rows that a recorded step adds as padding hold
+    `pad`.  (In a recorded step of single tokens a token id that is still on the device reads 0 in the layout.)
+    Registered once, by the module that defines the part that needs it, before the model is built."""
+    if per not in ("token", "sequence"):
+        raise ValueError("A step array has one entry per 'token' or per 'sequence'.")
+    _EXTRA_ARRAYS[name] = (per, build, int(pad))
+
+
+def unregister_step_array(name: str) -> None:
+    _EXTRA_ARRAYS.pop(name, None)
+
+
+def extra_step_arrays() -> dict:
+    return dict(_EXTRA_ARRAYS)
+
+
+@dataclass
+class StepLayout:
+    """A step as the builders of its arrays see it: per sequence the first position, the number of new tokens,
+    the start of its tokens in the flat order and its state slot; per token its sequence, position and id."""
+
+    entries: list
+    first_pos: np.ndarray
+    q_len: np.ndarray
+    q_start: np.ndarray
+    state_slots: np.ndarray
+    seq_of_token: np.ndarray
+    positions: np.ndarray
+    token_ids: np.ndarray
+
+
+def _extras(layout: StepLayout) -> list:
+    out = []
+    for name, (per, build, _) in _EXTRA_ARRAYS.items():
+        array = np.ascontiguousarray(build(layout), dtype=np.int32).reshape(-1)
+        want = len(layout.token_ids) if per == "token" else len(layout.q_len)
+        if array.size != want:
+            raise ValueError(f"Step array {name!r} has {array.size} entries for {want} {per}s.")
+        out.append(("x:" + name, array))
+    return out
+
+
 @dataclass
 class StepArrays:
     """A step's integer arrays on the host, in the order in which they are staged, and what the step's kernels
@@ -196,8 +250,9 @@ class StepArrays:
 
 def step_arrays(entries: list[StepEntry], cache, table_tokens: int | None = None) -> StepArrays:
     """Lay the entries out flat: token ids, positions, per-sequence start / length / context, the places of
-    wanted logits, state slots, the attention work lists, and per cache group the block tables (a row holds the
-    pages of `table_tokens` tokens, by default as many as the longest table) and the cache slot of every token.
+    wanted logits, state slots, the arrays that parts have registered, the attention work lists, and per cache
+    group the block tables (a row holds the pages of `table_tokens` tokens, by default as many as the longest
+    table) and the cache slot of every token.
 
     Each entry's sequence must already hold pages for its new tokens (CacheManager.reserve).
     """
@@ -216,8 +271,15 @@ def step_arrays(entries: list[StepEntry], cache, table_tokens: int | None = None
     logit_rows = np.asarray(rows, dtype=np.int32)
     state_slots = np.asarray([e.seq.state_slot for e in entries], dtype=np.int32)
 
-    names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots", "seq_of_token"]
-    arrays = [token_ids, positions, starts, q_len, ctx_len, logit_rows, state_slots, seq_of_token]
+    core = {"token_ids": token_ids, "positions": positions, "q_start": starts, "q_len": q_len, "ctx_len": ctx_len,
+            "logit_rows": logit_rows, "state_slots": state_slots, "seq_of_token": seq_of_token}
+    names = list(STEP_ARRAY_NAMES)
+    arrays = [core[name] for name in names]
+    if _EXTRA_ARRAYS:
+        for name, array in _extras(StepLayout(entries, first_pos, q_len, starts, state_slots, seq_of_token, positions,
+                                              token_ids)):
+            names.append(name)
+            arrays.append(array)
     lists = ops.attention_lists(q_lens)
     for name in sorted(lists):
         names.append(name)
@@ -251,6 +313,7 @@ def context_from(step: StepArrays, dev: list, n_groups: int, workspace: Workspac
     ctx.token_ids, ctx.positions, ctx.q_start = by_name["token_ids"], by_name["positions"], by_name["q_start"]
     ctx.q_len, ctx.ctx_len, ctx.logit_rows = by_name["q_len"], by_name["ctx_len"], by_name["logit_rows"]
     ctx.state_slots, ctx.seq_of_token = by_name["state_slots"], by_name["seq_of_token"]
+    ctx.extra = {name[2:]: tensor for name, tensor in by_name.items() if name.startswith("x:")}
     on_device = {name: (by_name[name], len(step.lists[name])) for name in step.lists}
     ctx.attention = ops.AttentionBatch(ctx.q_start, ctx.q_len, ctx.ctx_len, step.n_seqs, on_device,
                                        step.max_decode_ctx if max_decode_ctx is None else max_decode_ctx,

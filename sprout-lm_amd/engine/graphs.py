@@ -27,7 +27,8 @@ import numpy as np
 import torch
 
 from .. import ops
-from .batch import CacheSlotView, KeptWorkspace, OwnedNames, StepContext, Workspace, context_from, step_arrays
+from .batch import (STEP_ARRAY_NAMES, CacheSlotView, KeptWorkspace, OwnedNames, StepContext, StepLayout, Workspace,
+                    context_from, extra_step_arrays, step_arrays)
 
 
 def _bucket(n: int, floor: int = 1) -> int:
@@ -46,9 +47,10 @@ class _DecodeGraph:
         self.max_blocks = [-(-ctx_bucket // g.page_tokens) for g in cache.groups]   # a table row's width, per group
         self.ctx_bucket = ctx_bucket
         S, G = n_seqs, len(cache.groups)
-        # layout of the int32 staging buffer
-        names = ["token_ids", "positions", "q_start", "q_len", "ctx_len", "logit_rows", "state_slots",
-                 "seq_of_token", "counter", "temperature", "feed_source"]
+        # layout of the int32 staging buffer: the arrays of every step (one token a sequence: S entries each), those
+        # that parts have registered, and what sampling and token feeding need
+        self.extras = extra_step_arrays()
+        names = list(STEP_ARRAY_NAMES) + ["x:" + name for name in self.extras] + ["counter", "temperature", "feed_source"]
         self.offsets, total = {}, 0
         for name in names:
             self.offsets[name] = (total, S)
@@ -77,6 +79,7 @@ class _DecodeGraph:
         ctx.token_ids, ctx.positions, ctx.q_start = view("token_ids"), view("positions"), view("q_start")
         ctx.q_len, ctx.ctx_len, ctx.logit_rows = view("q_len"), view("ctx_len"), view("logit_rows")
         ctx.state_slots, ctx.seq_of_token = view("state_slots"), view("seq_of_token")
+        ctx.extra = {name: view("x:" + name) for name in self.extras}
         empty = (self.dev[:0].view(0, 2), 0)
         every = torch.from_numpy(np.stack([arange, np.zeros_like(arange)], axis=1)).to(runner.device)
         lists = {f"tiles_multi_{t}": empty for t in ops.kernels.TILE_SIZES}
@@ -121,6 +124,13 @@ class _DecodeGraph:
         h["counter"][:n] = counters
         h["temperature"].view(np.float32)[:n] = [p.temperature for p in params]
         h["seed"].view(np.int64)[:n] = [p.seed for p in params]
+        if self.extras:
+            first = np.arange(n, dtype=np.int32)
+            layout = StepLayout(entries, lengths, np.ones(n, dtype=np.int32), first, h["state_slots"][:n], first,
+                                lengths, h["token_ids"][:n])
+            for name, (_, build, pad) in self.extras.items():
+                h["x:" + name][:n] = np.asarray(build(layout), dtype=np.int32).reshape(-1)
+                h["x:" + name][n:] = pad
         if n != self._filled:
             for name in ("token_ids", "positions", "temperature"):
                 h[name][n:] = 0

@@ -53,7 +53,9 @@ class ModelRunner:
         self.plan, self.dtype, self.device = plan, dtype, device
         self.parts = parts if parts is not None else plan.instantiate()
         self.budget = budget or MemoryBudget()
-        self.cache = CacheManager(self.parts.cache_slot_specs, block_size, num_blocks, max_sequences, prefix_caching)
+        # whether pages of a common prefix may be shared is the architecture's word (the plan), then the caller's
+        self.cache = CacheManager(self.parts.cache_slot_specs, block_size, num_blocks, max_sequences,
+                                  prefix_caching and self.parts.prefix_sharing)
         if torch.device(device).type == "cuda":
             check_budget(0, self.cache.storage_bytes(dtype.itemsize), free_device_bytes(device), self.budget,
                          "cache pools (the weights are resident already)")
@@ -117,16 +119,24 @@ class ModelRunner:
         return cls(plan, tensors, dtype, device, budget=budget, parts=parts, **cache_options)
 
     # ------------------------------------------------------------------ the step
-    def _slot_view(self, ctx, call) -> CacheSlotView | None:
-        if call.cache_slot is None:
-            return None
-        kind, g, index = self.cache.slot_location[call.cache_slot]
-        if kind == "paged":
-            group = self.cache.groups[g]
-            return CacheSlotView(call.writes, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
-                                 slot_mapping=ctx.group_slots[g], page_size=group.page_tokens)
-        group = self.cache.state_groups[g]
-        return CacheSlotView(call.writes, state=group.data[index])
+    def _slot_views(self, ctx, call_index: int) -> dict:
+        """What the parts of one call of the run order get for their caches: part name -> view, or -> a dict of
+        views where the part asked for several things by name."""
+        views: dict = {}
+        for key, (slot, writes) in self.parts.call_slots[call_index].items():
+            kind, g, index = self.cache.slot_location[slot]
+            if kind == "paged":
+                group = self.cache.groups[g]
+                view = CacheSlotView(writes, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
+                                     slot_mapping=ctx.group_slots[g], page_size=group.page_tokens)
+            else:
+                view = CacheSlotView(writes, state=self.cache.state_groups[g].data[index])
+            name, _, sub = key.partition(".")
+            if sub:
+                views.setdefault(name, {})[sub] = view
+            else:
+                views[name] = view
+        return views
 
     def validate(self, entries: list[StepEntry]) -> None:
         seen = set()
@@ -259,8 +269,8 @@ class ModelRunner:
         with ops.stream_scope():       # one stream lookup for the step's launches
             residual = ctx.buffer("residual", (T, H), torch.float32)
             self.parts.embedding.forward(ctx, ctx.token_ids, residual)
-            for call in self.plan.schedule:
-                self.parts.blocks[call.layer].forward(ctx, residual, self._slot_view(ctx, call))
+            for i, call in enumerate(self.plan.schedule):
+                self.parts.blocks[call.layer].forward(ctx, residual, self._slot_views(ctx, i))
             n = ctx.n_logits
             logits = ctx.buffer("logits", (n, self.vocab_size), torch.float32)
             if n:

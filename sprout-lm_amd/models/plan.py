@@ -34,15 +34,18 @@ class LayerPlan:
 
 @dataclass
 class LayerCall:
-    """One entry of the run order: run `layer` with cache slot `cache_slot`.
+    """One entry of the run order: run `layer`, its parts' caches in the slots `cache_slot` names.
 
-    A layer may be called more than once (its weights are reused; give each call a slot of its
-    own), and a call with writes False reads a slot that another call has written.
+    `cache_slot`: None (the layer keeps nothing), one slot number (for a layer in which exactly one part keeps
+    something), or a mapping from what the layer's parts ask for to slot numbers: `{"mixer": 3}`, and, for a part
+    whose `cache_spec` is itself a dict, `{"mixer.pages": 3, "mixer.tail": 4}`.  A layer may be called more than
+    once (its weights are reused; give each call slots of its own), and a call with `writes` False reads slots
+    that another call has written (`writes` may also be a mapping with the same keys).
     """
 
     layer: int
-    cache_slot: int | None
-    writes: bool = True
+    cache_slot: int | dict | None
+    writes: bool | dict = True
 
 
 @dataclass
@@ -59,6 +62,10 @@ class ModelPlan:
     final_norm: PartPlan
     head: PartPlan
     ignorable_tensors: frozenset = frozenset()
+    # Whether requests may share the pages of a common prefix.  None: yes, unless some part keeps per-request
+    # state of fixed size, which is no function of pages and would have to be rebuilt with them; an architecture
+    # that knows better (a state it can snapshot at page edges, pages that depend on more than the tokens) says so.
+    prefix_sharing: bool | None = None
 
     def instantiate(self) -> "ModelParts":
         return ModelParts(self)
@@ -83,31 +90,67 @@ class ModelParts:
             made = {name: part.make() for name, part in layer.parts.items()}
             self.blocks.append(make_part("block", layer.block, **made))
             self._named.extend((layer.parts[name].prefix, made[name]) for name in layer.parts)
+        # What every call of the run order keeps where: per call {key: (slot, writes)}, key = a part's name in its
+        # block, or "name.sub" where the part's cache_spec is a dict.
+        self.call_slots: list[dict[str, tuple[int, bool]]] = []
         slots: dict[int, object] = {}
         for call in plan.schedule:
             if call.layer < 0 or call.layer >= len(self.blocks):
                 raise ValueError(f"Run order names layer {call.layer}, but the model has {len(self.blocks)} layers.")
-            spec = self.blocks[call.layer].mixer.cache_spec()
+            needs = self.cache_needs(self.blocks[call.layer])
             if call.cache_slot is None:
-                continue
-            if call.writes:
-                if call.cache_slot in slots:
-                    raise ValueError(f"Cache slot {call.cache_slot} is written by two calls of the run order.")
-                slots[call.cache_slot] = spec
-        for call in plan.schedule:
-            if call.cache_slot is not None and not call.writes:
-                spec = self.blocks[call.layer].mixer.cache_spec()
-                if slots.get(call.cache_slot) != spec:
-                    raise ValueError(f"Layer {call.layer} reads cache slot {call.cache_slot}, which no call writes "
-                                     f"with the same shape.")
+                named = {}
+            elif isinstance(call.cache_slot, dict):
+                named = dict(call.cache_slot)
+            else:
+                if len(needs) != 1:
+                    raise ValueError(f"Layer {call.layer} is given one cache slot, but its parts ask for "
+                                     f"{sorted(needs) or 'none'}: name the slots by part.")
+                named = {next(iter(needs)): call.cache_slot}
+            unknown = sorted(set(named) - set(needs))
+            if unknown:
+                raise ValueError(f"Layer {call.layer} has no part that keeps {unknown}; its parts ask for {sorted(needs)}.")
+            mine = {}
+            for key, slot in named.items():
+                writes = call.writes.get(key, True) if isinstance(call.writes, dict) else bool(call.writes)
+                mine[key] = (slot, writes)
+                if writes:
+                    if slot in slots:
+                        raise ValueError(f"Cache slot {slot} is written by two calls of the run order.")
+                    slots[slot] = needs[key]
+            self.call_slots.append(mine)
+        for call, mine in zip(plan.schedule, self.call_slots):
+            needs = self.cache_needs(self.blocks[call.layer])
+            for key, (slot, writes) in mine.items():
+                if not writes and slots.get(slot) != needs[key]:
+                    raise ValueError(f"Layer {call.layer} reads cache slot {slot}, which no call writes with the "
+                                     f"same shape.")
         if sorted(slots) != list(range(len(slots))):
             raise ValueError("Cache slots of the run order must be numbered 0..n-1 without gaps.")
         self.cache_slot_specs = [slots[i] for i in range(len(slots))]
+        if plan.prefix_sharing is None:
+            from ..cache.spec import StateSpec
+            self.prefix_sharing = not any(isinstance(spec, StateSpec) for spec in self.cache_slot_specs)
+        else:
+            self.prefix_sharing = bool(plan.prefix_sharing)
         every = [part for _, part in self._named] + list(self.blocks)
-        every += [getattr(b.mixer, "position", None) for b in self.blocks if hasattr(b, "mixer")]
+        for part in list(every):
+            every += part.subparts()
         self.graph_safe = all(getattr(part, "graph_safe", False) for part in every if part is not None)
         self.graph_safe_portions = self.graph_safe and all(getattr(part, "graph_safe_portions", False)
                                                            for part in every if part is not None)
+
+    @staticmethod
+    def cache_needs(block) -> dict:
+        """What the parts of `block` keep between steps: {"part": spec} and {"part.sub": spec}."""
+        needs = {}
+        for name, part in block.parts().items():
+            spec = part.cache_spec()
+            if isinstance(spec, dict):
+                needs.update({f"{name}.{sub}": one for sub, one in spec.items()})
+            elif spec is not None:
+                needs[name] = spec
+        return needs
 
     # ------------------------------------------------------------------ what a step costs, summed over the parts
     def _calls(self):
@@ -126,7 +169,7 @@ class ModelParts:
 
     def cache_bytes_per_context_token(self, element_size: int) -> int:
         """Cache bytes that one decoded token reads per token of its context, over all calls of the run order."""
-        return sum(block.mixer.cache_elements_per_token() for block in self._calls() if hasattr(block, "mixer")) * element_size
+        return sum(part.cache_elements_per_token() for block in self._calls() for part in block.parts().values()) * element_size
 
     def flops(self, tokens: int, pairs: int, logit_rows: int) -> float:
         """Matrix-product operations of a step of `tokens` tokens with `pairs` (query, key) pairs in every

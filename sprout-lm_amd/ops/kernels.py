@@ -451,6 +451,13 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> N
                                 variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
+def random_fill(dst: torch.Tensor, key: int, scale: float, offset: float | None = None, first: int = 0) -> None:
+    """dst (flat order) = the seeded values of elements first .. of the tensor keyed `key` (see sprout_hip.h)."""
+    _gpu(dst, "random fill destination")
+    check(library().sp_random_fill(_stream(), _code(dst, "random fill destination"), dst.data_ptr(), dst.numel(),
+                                   key & 0xFFFFFFFFFFFFFFFF, first, float(scale), float(offset or 0.0), int(offset is not None)))
+
+
 def sample_workspace_floats(rows: int, vocab: int) -> int:
     return library().sp_sample_workspace_floats(rows, vocab)
 

@@ -44,6 +44,7 @@ def _declare(lib):
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
         "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_random_fill": [c_void, c_int, c_void, c_i64, ctypes.c_uint64, c_i64, c_float, c_float, c_int],
         "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],
         "sp_probe_mfma": [c_void, c_int, c_int, c_void, ctypes.POINTER(ctypes.c_double)],
     }

@@ -9,7 +9,6 @@ from .. import ops
 from ..cache.spec import PagedKVSpec
 from ..config.base import ConfigError
 from ..weights.loader import TensorSpec
-from .norm import RMSNorm
 from .base import Mixer, register_part
 
 
@@ -83,6 +82,9 @@ class Attention(Mixer):
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
+    def subparts(self):
+        return [self.position]
+
     def _fused(self, T: int, cache, norm: bool) -> bool:
         """Whether a projection kernel with bias, rotation and cache write folded in takes this call."""
         return (self.own_kv and cache.writes and self.w_qkv.dtype == torch.bfloat16
@@ -97,16 +99,17 @@ class Attention(Mixer):
 
     def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
         T = residual.shape[0]
-        if not self.fuse_input_norm:
+        fold = norm.fold() if self.fuse_input_norm else None
+        if fold is None or fold.kind != "rms":       # the one prologue the projection kernels have
             return False
-        if ctx.act_dtype != torch.bfloat16 or T > 64 or not isinstance(norm, RMSNorm) or not self._fused(T, cache, True):
+        if ctx.act_dtype != torch.bfloat16 or T > 64 or not self._fused(T, cache, True):
             return False
         if not ops.fused_norm_pays(T, self.w_qkv.shape[0], self.hidden):
             return False
         q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
         ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                            cache.slot_mapping, cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
-                           residual=residual, norm_weight=norm.w["weight"], eps=norm.eps, pairing=self.position.pairing)
+                           residual=residual, norm_weight=fold.weight, eps=fold.eps, pairing=self.position.pairing)
         self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
         return True
 

@@ -63,6 +63,21 @@ class Part:
     def prepare(self, device, dtype) -> None:
         """Build device-side constants (tables of frequencies and the like).  Called once."""
 
+    def subparts(self) -> list:
+        """Parts that this part holds and runs itself (a mixer's position encoding): they are asked for
+        `graph_safe` along with it."""
+        return []
+
+    def cache_spec(self):
+        """What the part keeps between steps: a PagedKVSpec, a StateSpec, a dict of several of them by a name of
+        the part's choosing (pages and a state of fixed size, say), or None.  Any part of a block may keep
+        something; it receives the view of its slot (or a dict of views under the same names) from the block."""
+        return None
+
+    def cache_elements_per_token(self) -> int:
+        """Cache elements that a decoded token reads per token of its context (keys and values)."""
+        return 0
+
     # What a part costs, for measurement: the engine's bench adds these up over the model's parts and
     # knows no architecture.
     def weight_elements(self) -> int:
@@ -86,6 +101,19 @@ class Norm(Part):
         """out = norm(x[rows] or x).  x is the float32 residual stream, out has the activation dtype."""
         raise NotImplementedError
 
+    def fold(self):
+        """How the norm can be computed inside the kernel of the product that follows it, or None if it
+        cannot: a `NormFold` whose `kind` names a prologue that the product kernels have.  A part that
+        folds asks the norm, not its class."""
+        return None
+
+
+class NormFold:
+    """A norm as a product kernel's prologue.  kind "rms": x * rsqrt(mean(x^2) + eps) * weight."""
+
+    def __init__(self, kind: str, weight, eps: float):
+        self.kind, self.weight, self.eps = kind, weight, eps
+
 
 class PositionEncoding(Part):
     """Turns positions into something a mixer applies to its queries and keys.
@@ -101,16 +129,9 @@ class PositionEncoding(Part):
 class Mixer(Part):
     """Mixes information between the tokens of a sequence (attention, or anything with state)."""
 
-    def cache_spec(self):
-        """A PagedKVSpec, a StateSpec, or None if the mixer keeps nothing between steps."""
-        return None
-
-    def cache_elements_per_token(self) -> int:
-        """Cache elements that a decoded token reads per token of its context (keys and values)."""
-        return 0
-
     def forward(self, ctx, h, residual, cache):
-        """residual += mixer(h).  `cache` is this call's cache slot view (engine.batch.CacheSlotView) or None."""
+        """residual += mixer(h).  `cache` is this call's cache slot view (engine.batch.CacheSlotView), a dict of
+        views if `cache_spec` names several, or None."""
         raise NotImplementedError
 
     def forward_from_residual(self, ctx, norm, residual, cache) -> bool:
@@ -130,10 +151,14 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """Arranges a mixer, a feed-forward and their norms around the residual stream."""
+    """Arranges mixers, feed-forwards and their norms around the residual stream."""
 
     def parts(self) -> dict[str, Part]:
+        """The block's parts by the names under which the model plan gave them; everything the engine wants of a
+        block's parts (tensors, cache needs, costs, whether they may be recorded) it asks through this."""
         raise NotImplementedError
 
-    def forward(self, ctx, residual, cache):
+    def forward(self, ctx, residual, caches: dict):
+        """Run the block on the step's tokens.  `caches`: part name -> what that part's `cache_spec` asked for in
+        this call of the run order (a view, or a dict of views); parts that keep nothing are absent."""
         raise NotImplementedError

@@ -18,8 +18,9 @@ class PreNormBlock(Block):
     def parts(self):
         return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ffn_norm": self.ffn_norm, "ffn": self.ffn}
 
-    def forward(self, ctx, residual, cache):
+    def forward(self, ctx, residual, caches):
         T, H = residual.shape
+        cache = caches.get("mixer")
         h = ctx.buffer("normed", (T, H), ctx.act_dtype)
         if not self.mixer.forward_from_residual(ctx, self.mixer_norm, residual, cache):
             self.mixer_norm.forward(ctx, residual, h)

@@ -5,7 +5,6 @@ import torch
 
 from .. import ops
 from ..weights.loader import TensorSpec
-from .norm import RMSNorm
 from .base import FeedForward, register_part
 
 
@@ -44,14 +43,15 @@ class GatedMLP(FeedForward):
 
     def forward_from_residual(self, ctx, norm, residual) -> bool:
         T = residual.shape[0]
-        if not self.fuse_input_norm:
+        fold = norm.fold() if self.fuse_input_norm else None
+        if fold is None or fold.kind != "rms":       # the one prologue the product kernels have
             return False
-        if ctx.act_dtype != torch.bfloat16 or T > 64 or not isinstance(norm, RMSNorm) or not self._fused(T, True):
+        if ctx.act_dtype != torch.bfloat16 or T > 64 or not self._fused(T, True):
             return False
         if not ops.fused_norm_pays(T, 2 * self.inner, self.hidden):
             return False
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=norm.w["weight"], eps=norm.eps,
+        ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=fold.weight, eps=fold.eps,
                          activation=self.activation)
         ops.gemm(act, self.w_down, residual, accumulate=True)
         return True

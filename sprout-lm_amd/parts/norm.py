@@ -3,7 +3,7 @@ from __future__ import annotations
 
 from .. import ops
 from ..weights.loader import TensorSpec
-from .base import Norm, register_part
+from .base import Norm, NormFold, register_part
 
 
 @register_part("norm", "rmsnorm")
@@ -23,3 +23,6 @@ class RMSNorm(Norm):
     def forward(self, ctx, x, out, rows=None):
         ops.rmsnorm(x, self.w["weight"], self.eps, out, rows)
         return out
+
+    def fold(self):
+        return NormFold("rms", self.w["weight"], self.eps)

@@ -281,7 +281,8 @@ def test_lru_eviction_takes_only_pages_no_request_uses():
 
 def test_state_slots_are_per_request_and_come_back():
     cache = CacheManager([FULL, StateSpec((4, 3))], block_size=4, num_blocks=4, max_sequences=2)
-    assert not cache.prefix_caching and cache.slot_location[1] == ("state", 0, 0)
+    # whether a model with state shares prefixes is its plan's word; the manager does what it is told
+    assert cache.prefix_caching and cache.slot_location[1] == ("state", 0, 0)
     a, b = cache.create(), cache.create()
     assert {a.state_slot, b.state_slot} == {0, 1}
     with pytest.raises(PageError):
@@ -350,3 +351,18 @@ def test_groups_with_pages_of_their_own_size():
     assert b.blocks[1][:8] == [FREED] * 8                 # at length 26 keys before 17 are passed: pages up to key 15
     a.release(); b.release(); cache.clear_prefixes()
     assert cache.free_pages() == [6, 24]
+
+
+def test_keys_and_values_of_different_widths_and_a_dtype_of_their_own():
+    """A slot whose values are narrower than its keys, kept in float32 whatever the model computes in: a group
+    of its own, pools of the asked shapes, and the bytes that the memory budget counts."""
+    import torch
+    odd = PagedKVSpec(1, 24, value_dim=8, dtype="float32")
+    cache = CacheManager([FULL, odd, FULL], block_size=4, num_blocks=5, max_sequences=2)
+    assert [g.slots for g in cache.groups] == [[0, 2], [1]]
+    cache.attach_storage(torch.bfloat16, "cpu")
+    full, other = cache.groups
+    assert full.k.shape == (2, 5, 2, 4, 16) and full.v.shape == (2, 5, 2, 16, 4) and full.k.dtype == torch.bfloat16
+    assert other.k.shape == (1, 5, 1, 4, 24) and other.v.shape == (1, 5, 1, 8, 4) and other.v.dtype == torch.float32
+    want = sum(t.numel() * t.element_size() for g in cache.groups for t in (g.k, g.v))
+    assert cache.storage_bytes(2) == want == CacheManager.pool_bytes([FULL, odd, FULL], 4, 5, 2, 2)

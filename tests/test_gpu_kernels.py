@@ -171,6 +171,25 @@ def test_embed_and_silu_mul(dtype):
     assert np.abs(out.float().cpu().numpy() - want).max() <= tol * (1 + np.abs(want).max())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_random_fill_equals_its_host_twin_bit_by_bit(dtype):
+    """Random weights drawn on the device are the numbers that the host draws for the same (seed, name, index):
+    a model folder written on the host and an engine that draws its weights on the GPU hold the same model."""
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.weights.random_init import fill_numpy, key_for, random_tensors
+    from sprout_lm_amd.weights import TensorSpec
+    for name, n, first, offset in (("a", 1, 0, None), ("model.embed_tokens.weight", 100_003, 0, None),
+                                   ("b.norm", 4099, 0, 1.0), ("c", 70_001, 5_000_000_123, None)):
+        key = key_for(17, name)
+        got = torch.empty(n, dtype=dtype, device=DEV)
+        ops.random_fill(got, key, 0.02 / 65536, offset, first)
+        want = torch.from_numpy(fill_numpy(key, n, 0.02 / 65536, offset, first)).to(dtype)
+        assert torch.equal(got.cpu(), want), name
+    expected = {"w": TensorSpec((37, 129)), "n": TensorSpec((129,), "vector", "one_plus_normal")}
+    host, device = random_tensors(expected, 3, dtype, "cpu", 0.05), random_tensors(expected, 3, dtype, DEV, 0.05)
+    assert all(torch.equal(host[k], device[k].cpu()) for k in expected)
+
+
 def plain_rope(x, pos, hd, rotary, theta):
     x = x.astype(np.float64).copy()
     half = rotary // 2

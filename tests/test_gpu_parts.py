@@ -791,3 +791,219 @@ def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype, window_page):
     cache.clear_prefixes()
     assert cache.free_pages() == [40, 40 * per]
     print(f"windowed prefix sharing {dtype}: worst {worst:.2f} of the bound")
+
+
+# A third toy architecture: a layer that holds TWO mixers which both keep something (attention with pages beside a
+# running mean whose state comes as two named pieces), in a block kind of its own, and a per-token array that the
+# engine does not know (the token's segment), registered here and delivered to eager and recorded steps alike.
+
+def register_dual_toy():
+    from dataclasses import dataclass
+    from typing import ClassVar
+
+    import sprout_lm_amd as S
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.cache import StateSpec
+    from sprout_lm_amd.config.base import ModelConfig
+    from sprout_lm_amd.engine.batch import register_step_array
+    from sprout_lm_amd.models.plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+    from sprout_lm_amd.parts import Block, Mixer, register_part, registered_parts
+    from sprout_lm_amd.weights import TensorSpec
+
+    if "toy_segment_mean" in registered_parts("mixer"):
+        return
+
+    register_step_array("toy_segment", "token", lambda layout: layout.positions // 7)
+
+    @register_part("mixer", "toy_segment_mean")
+    class SegmentMean(Mixer):
+        """y_t = W . mean(h_0 .. h_t) + bias[segment(t) % 4].  The state is kept as two named pieces, the running
+        sum and the count; the segment of every token comes from the step array registered above."""
+
+        graph_safe = True
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def cache_spec(self):
+            return {"sum": StateSpec((self.hidden,), "float32"), "count": StateSpec((1,), "float32")}
+
+        def tensors(self):
+            return {"proj.weight": TensorSpec((self.hidden, self.hidden)), "segment_bias.weight": TensorSpec((4, self.hidden))}
+
+        def forward(self, ctx, h, residual, cache):
+            total, count = cache["sum"].state, cache["count"].state
+            if ctx.max_q_len == 1:
+                slots = ctx.state_slots.long()
+                sums = total.index_select(0, slots) + h.float()
+                counts = count.index_select(0, slots) + 1
+                mean = (sums / counts).to(h.dtype).contiguous()
+                ops.gemm(mean, self.w["proj.weight"], residual, accumulate=True)
+                total.index_copy_(0, slots, sums)
+                count.index_copy_(0, slots, counts)
+            else:
+                for start, n, slot in zip(ctx.host["q_start"], ctx.host["q_len"], ctx.host["state_slots"]):
+                    sums = torch.cumsum(h[start:start + n].float(), 0) + total[slot]
+                    counts = count[slot] + torch.arange(1, n + 1, device=h.device, dtype=torch.float32)[:, None]
+                    mean = (sums / counts).to(h.dtype).float()
+                    residual[start:start + n] += mean @ self.w["proj.weight"].float().T
+                    total[slot] = sums[-1]
+                    count[slot] = counts[-1]
+            segment = (ctx.extra["toy_segment"][:h.shape[0]] % 4).long()
+            residual.add_(self.w["segment_bias.weight"].float().index_select(0, segment))
+
+    @register_part("block", "toy_two_mixers")
+    class TwoMixers(Block):
+        """x += attention(norm(x)) + mean(norm(x)); x += feed_forward(norm(x))."""
+
+        graph_safe = True
+
+        def __init__(self, norm, attn, mean, ffn_norm, ffn):
+            self.norm, self.attn, self.mean, self.ffn_norm, self.ffn = norm, attn, mean, ffn_norm, ffn
+
+        def parts(self):
+            return {"norm": self.norm, "attn": self.attn, "mean": self.mean, "ffn_norm": self.ffn_norm, "ffn": self.ffn}
+
+        def forward(self, ctx, residual, caches):
+            T, Hd = residual.shape
+            h = ctx.buffer("normed", (T, Hd), ctx.act_dtype)
+            self.norm.forward(ctx, residual, h)
+            self.attn.forward(ctx, h, residual, caches["attn"])
+            self.mean.forward(ctx, h, residual, caches["mean"])
+            self.ffn_norm.forward(ctx, residual, h)
+            self.ffn.forward(ctx, h, residual)
+
+    @dataclass(frozen=True)
+    class DualConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyDualForCausalLM"
+        model_types: ClassVar[tuple] = ("toy_dual",)
+        hidden: int = 0
+        inner: int = 0
+        vocab: int = 0
+        heads: int = 0
+        kv_heads: int = 0
+        layers: int = 0
+        eps: float = 0.0
+        theta: float = 0.0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "layers", "eps", "theta")})
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "model_type": "toy_dual",
+                    **{k: getattr(self, k) for k in ("hidden", "inner", "vocab", "heads", "kv_heads", "layers", "eps", "theta")}}
+
+    def build(cfg):
+        hd = cfg.hidden // cfg.heads
+        norm = lambda prefix: PartPlan("norm", "rmsnorm", {"size": cfg.hidden, "eps": cfg.eps}, prefix)
+        layers, schedule = [], []
+        for i in range(cfg.layers):
+            layers.append(LayerPlan("toy_two_mixers", {
+                "norm": norm(f"l{i}.n1."),
+                "attn": PartPlan("mixer", "attention", {
+                    "hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.kv_heads, "head_dim": hd,
+                    "position": PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": cfg.theta})}, f"l{i}.attn."),
+                "mean": PartPlan("mixer", "toy_segment_mean", {"hidden": cfg.hidden}, f"l{i}.mean."),
+                "ffn_norm": norm(f"l{i}.n2."),
+                "ffn": PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner}, f"l{i}.mlp.")}))
+            schedule.append(LayerCall(i, {"attn": 3 * i, "mean.sum": 3 * i + 1, "mean.count": 3 * i + 2}))
+        return ModelPlan("ToyDualForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
+                         PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.hidden}, "embed."),
+                         layers, schedule, norm("final."),
+                         PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.hidden, "tied": True}, "head."))
+
+    S.register_architecture("ToyDualForCausalLM", DualConfig, build, model_types=("toy_dual",))
+
+
+DUAL = dict(model_type="toy_dual", hidden=64, inner=112, vocab=113, heads=4, kv_heads=2, layers=2, eps=1e-5, theta=1e4)
+
+
+def plain_dual_logits(w, tokens, store):
+    c = DUAL
+    hd = c["hidden"] // c["heads"]
+    pos = np.arange(len(tokens))
+    x = P.f32(w["embed.weight"][np.asarray(tokens)])
+    for i in range(c["layers"]):
+        n = store(P.rms_norm(x, w[f"l{i}.n1.weight"], c["eps"]))
+        p = f"l{i}.attn."
+        q = store(P.rope_neox(store(P.linear(n, w[p + "q_proj.weight"], w[p + "q_proj.bias"])), pos, hd, c["theta"]))
+        k = store(P.rope_neox(store(P.linear(n, w[p + "k_proj.weight"], w[p + "k_proj.bias"])), pos, hd, c["theta"]))
+        v = store(P.linear(n, w[p + "v_proj.weight"], w[p + "v_proj.bias"]))
+        a = store(P.causal_gqa_attention(q, k, v, c["heads"], c["kv_heads"], hd))
+        x = P.f32(x + P.linear(a, w[p + "o_proj.weight"]))
+        mean = store(np.cumsum(n.astype(np.float64), 0) / np.arange(1, len(tokens) + 1)[:, None])
+        x = P.f32(x + P.linear(mean, w[f"l{i}.mean.proj.weight"]))
+        x = P.f32(x + w[f"l{i}.mean.segment_bias.weight"][(pos // 7) % 4])
+        n = store(P.rms_norm(x, w[f"l{i}.n2.weight"], c["eps"]))
+        gate, up = store(P.linear(n, w[f"l{i}.mlp.gate_proj.weight"])), store(P.linear(n, w[f"l{i}.mlp.up_proj.weight"]))
+        x = P.f32(x + P.linear(store(P.swiglu(gate, up)), w[f"l{i}.mlp.down_proj.weight"]))
+    return P.linear(store(P.rms_norm(x, w["final.weight"], c["eps"])), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_layer_with_two_mixers_that_both_keep_something(tmp_path, dtype):
+    """A block kind, a mixer and a per-token step array defined in this file: every layer holds attention (pages)
+    beside a running mean (two named state tensors), so a call of the run order names three cache slots by part.
+    Replayed whole, with the last tokens one by one, in portions down to two tokens and mixed with so few pages
+    that they are used again, and decoded through recorded graphs: every row against the plain function."""
+    register_dual_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.cache import StateSpec
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    from sprout_lm_amd.engine.trace import TraceSession
+    from sprout_lm_amd.sampling import SamplingParams
+    from sprout_lm_amd.weights import write_model_folder
+    from tests import traces
+    folder = str(tmp_path / "dual")
+    write_model_folder(folder, S.config_from_dict(DUAL), seed=29, dtype=torch.bfloat16, std=0.15)
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    store = P.bf16_round if dtype == "bfloat16" else P.f32
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    requests = {f"r{i}": H.random_tokens(113, n, 40 + i) for i, n in enumerate([37, 9, 70, 44, 25, 61])}
+    want = {k: plain_dual_logits(w, t, store) for k, t in requests.items()}
+    pool = sum(sorted(-(-len(t) // 8) for t in requests.values())[-4:])        # pages of 8: the four longest fit, no more
+    worst = 0.0
+    for family, trace in (("whole", traces.whole(requests)), ("tail", traces.tail_decoded(requests, tail=20)),
+                          ("portions", traces.portions(requests)), ("mixed", traces.mixed(requests, seed=5))):
+        runner = ModelRunner.from_folder(folder, dtype, block_size=8, num_blocks=pool, max_sequences=4, prefix_caching=True)
+        # three slots a layer, named by part: pages for the attention, two state tensors for the mean
+        assert runner.parts.call_slots[1] == {"attn": (3, True), "mean.sum": (4, True), "mean.count": (5, True)}
+        assert [g.slots for g in runner.cache.groups] == [[0, 3]]
+        assert [(g.spec, g.slots) for g in runner.cache.state_groups] == [(StateSpec((64,)), [1, 4]), (StateSpec((1,)), [2, 5])]
+        assert not runner.parts.prefix_sharing and not runner.cache.prefix_caching     # the plan's word, not the manager's
+        session = TraceSession(runner)
+        for record, rows in zip(trace.steps, trace.expected):
+            logits = session.run_step(record)
+            got = logits.cpu().numpy() if rows else None
+            for i, (rid, pos) in enumerate(rows):
+                err = np.abs(got[i] - want[rid][pos]).max() / (tol * (1 + np.abs(want[rid][pos]).max()))
+                worst = max(worst, err)
+                assert err <= 1.0, f"{family} {rid} position {pos}: {err:.2f} of the bound"
+        assert runner.cache.free_pages() == [pool] and not session.live
+    # three requests decoded through recorded graphs (a step of four rows, one of them padding)
+    runner = ModelRunner.from_folder(folder, dtype, block_size=8, num_blocks=40, max_sequences=3)
+    assert runner.parts.graph_safe and not runner.parts.graph_safe_portions
+    names = ["r0", "r2", "r3"]
+    seqs = {k: runner.cache.create() for k in names}
+    fed = {"r0": 20, "r2": 31, "r3": 2}
+    for k, n in fed.items():
+        assert runner.cache.reserve(seqs[k], n)
+        runner.step([StepEntry(seqs[k], requests[k][:n], [])])
+    for _ in range(17):
+        entries = []
+        for k in names:
+            assert runner.cache.reserve(seqs[k], fed[k] + 1)
+            entries.append(StepEntry(seqs[k], [requests[k][fed[k]]], [0]))
+        pending = runner.launch_decode(entries, [SamplingParams()] * 3, [0] * 3)
+        assert pending is not None, "the step did not run from a recorded graph"
+        runner.finish_decode(pending)
+        got = pending.logits[:3].cpu().numpy()
+        for row, k in zip(got, names):
+            err = np.abs(row - want[k][fed[k]]).max() / (tol * (1 + np.abs(want[k][fed[k]]).max()))
+            worst = max(worst, err)
+            assert err <= 1.0, f"recorded decode {k} position {fed[k]}: {err:.2f} of the bound"
+            fed[k] += 1
+    assert runner._graphs.replays == 17
+    print(f"two mixers a layer {dtype}: worst {worst:.2f} of the bound")

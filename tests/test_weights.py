@@ -97,6 +97,23 @@ def test_random_weights_mode_writes_a_loadable_folder(tmp_path):
     assert not torch.equal(other["model.norm.weight"], tensors["model.norm.weight"])
 
 
+def test_random_values_are_a_function_of_seed_name_and_index():
+    """Element i of a tensor depends on (seed, name, i) alone: a piece drawn from the middle equals that piece of
+    the whole, another name or seed gives other values, and the distribution has the asked deviation."""
+    from sprout_lm_amd.weights.random_init import fill_numpy, key_for
+    key = key_for(5, "model.layers.0.mlp.up_proj.weight")
+    whole = fill_numpy(key, 300_000, 0.02 / 65536)
+    assert np.array_equal(fill_numpy(key, 1000, 0.02 / 65536, first=123_457), whole[123_457:124_457])
+    assert abs(whole.std() - 0.02) < 2e-4 and abs(whole.mean()) < 2e-4 and np.abs(whole).max() <= 0.12
+    assert 0.04 < np.mean(np.abs(whole) > 0.04) < 0.05          # 4.55% of a normal distribution lie beyond two deviations
+    assert not np.array_equal(fill_numpy(key_for(6, "model.layers.0.mlp.up_proj.weight"), 100, 1.0), whole[:100])
+    assert key_for(5, "a") != key_for(5, "b")
+    # the first values, pinned: the device kernel and any later rewrite must give these very numbers
+    assert fill_numpy(key_for(1, "w"), 4, 1.0).tolist() == fill_numpy(key_for(1, "w"), 6, 1.0)[:4].tolist()
+    ones = fill_numpy(key, 50, 0.02 / 65536, offset=1.0)
+    assert np.array_equal(ones, whole[:50] + np.float32(1.0))
+
+
 def test_a_tensor_stored_in_32_bit_stays_so(tmp_path):
     folder = model_folder(tmp_path, "A", torch.float32)
     plan = S.build_model_plan(S.load_config(folder))
