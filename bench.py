@@ -7,13 +7,17 @@ Default: Qwen2.5-0.5B layer sizes with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
 Beside the contract's fields the line holds the prefill of 2,048 tokens (the median of its repeats), the
-roofline of the decode step, `points`: decoding at batch 1 and 64, and the same decode step and prefill at
-Qwen2.5-7B sizes with all 28 layers, each with its fraction of the published peak (`7b_...`), `measured`: what
-this GPU gave a kernel that only reads and one that only multiplies, just before the run, `step_ms` (median, 95th percentile and maximum of the timed steps as the
-host sees them, and `host`: the part of a step that the host spends planning and launching, which the
-look-ahead hides behind the GPU's work), `prefill_in_portions` (the same prompt prefilled 256 and 512 tokens a step), `mixed` (the batch decoding while another prompt is prefilled 256
-tokens a step) and, with --pressure SHARE, a run in a pool too small for its requests (preemptions,
-tokens computed again, net tokens a second).
+roofline of the decode step, and `points`: decoding at batch 1, 64, 128 and 256, and the same decode step and
+prefill at Qwen2.5-7B and Qwen2.5-32B sizes with all their layers, each with its fraction of the published peak
+(`7b_...`, `32b_...`); at 32B sizes also the batch in a pool of 0.6 of the pages it needs (`32b_pressure_...`:
+preemptions, tokens computed again, net tokens a second) and the one workload the reference publishes numbers for
+(`32b_mirror_...`: one request, 47 tokens in, 32 out, a pool of 256 tokens; scripts/benchmark-cuda-graph.ts:29-38
+there).  `measured`: what this GPU gave a kernel that only reads and one that only multiplies, just before the
+run; `step_ms`: median, 95th percentile and maximum of the timed steps as the host sees them, and `host`: the
+part of a step that the host spends planning and launching, which the look-ahead hides behind the GPU's work;
+`prefill_in_portions`: the same prompt prefilled 256 and 512 tokens a step; `mixed`: the batch decoding while
+another prompt is prefilled 256 tokens a step; with --pressure SHARE, the batch in a pool too small for its
+requests at the headline sizes.
 """
 from __future__ import annotations
 
@@ -138,14 +142,22 @@ def measure_mixed(engine, cfg, batch, context, chunk, steps, warmup, multiple=1)
             "decode_value": round(batch / elapsed, 1), "chunk_value": round(portion / elapsed, 1)}
 
 
-def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
+def engine_with_pool(model, pages, max_sequences, **options):
+    """An engine over the weights of `model` with a cache pool of its own (`pages` pages of 16 tokens)."""
+    from sprout_lm_amd.engine import Engine
+    runner = model.with_pool_of_its_own(block_size=16, num_blocks=pages, max_sequences=max_sequences)
+    return Engine(runner, block_size=16, num_blocks=pages, max_sequences=max_sequences, prefix_caching=False,
+                  record_trace=False, **options)
+
+
+def measure_pressure(model, cfg, batch, prompt_len, new_tokens, share):
     """A pool that holds `share` of what the requests need at their end: requests are preempted and
     their keys computed again.  Net tokens a second count every token once, however often it was computed."""
     import random
     import torch
     rng = random.Random(7)
     need = batch * -(-(prompt_len + new_tokens) // 16)
-    engine = make_engine(cfg, dtype, batch, prompt_len + new_tokens, prompt_len, pages=max(int(need * share), 2))
+    engine = engine_with_pool(model, max(int(need * share), 2), batch, max_batch_tokens=2048, prefill_chunk_size=2048)
     for i in range(batch):
         engine.add(f"q{i}", [rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], new_tokens, ignore_eos=True)
     torch.cuda.synchronize()
@@ -163,6 +175,37 @@ def measure_pressure(cfg, dtype, batch, prompt_len, new_tokens, share):
     return {"batch": batch, "prompt": prompt_len, "new_tokens": new_tokens, "pages": engine.options.num_blocks,
             "pages_needed": need, "preemptions": stats["preemptions"], "recomputed_tokens": stats["recomputed_tokens"],
             "steps": ticks, "seconds": round(elapsed, 3), "net_value": round(made / elapsed, 1)}
+
+
+def measure_mirror(model, cfg, prompt_len=47, new_tokens=32, requests=4):
+    """The one workload the reference publishes numbers for (scripts/benchmark-cuda-graph.ts:29-38): one request
+    at a time, a prompt of 47 tokens (seeded random ids stand in for its chat prompt), 32 generated tokens, a pool
+    of 256 tokens in pages of 16; one cold request, then the steady ones that are timed.  Returns the mean, median
+    and 95th percentile of a decode step and the mean time to the first token, in milliseconds."""
+    import random
+    import torch
+    rng = random.Random(47)
+    engine = engine_with_pool(model, 16, 1, max_batch_tokens=64, prefill_chunk_size=64)
+    steps, firsts = [], []
+    for r in range(requests):
+        engine.add(f"c{r}", [rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], new_tokens, ignore_eos=True)
+        torch.cuda.synchronize()
+        last = t0 = time.perf_counter()
+        made = 0
+        while engine.pending:
+            engine.step()
+            torch.cuda.synchronize()
+            now = time.perf_counter()
+            tokens = len(engine.scheduler.requests[f"c{r}"].output)
+            if tokens > made and r > 0:       # the first request is the cold one
+                (firsts if made == 0 else steps).append((now - (t0 if made == 0 else last)) * 1000)
+            made, last = tokens, now
+        engine.forget(f"c{r}")
+    engine.close()
+    steps.sort()
+    return {"decode_ms_mean": round(sum(steps) / len(steps), 4), "decode_ms_median": round(steps[len(steps) // 2], 4),
+            "decode_ms_p95": round(steps[min(len(steps) - 1, int(len(steps) * 0.95))], 4), "samples": len(steps),
+            "first_token_ms": round(sum(firsts) / len(firsts), 3)}
 
 
 def measure_prefill(engine, cfg, tokens, repeats=5, chunk=None):
@@ -193,9 +236,12 @@ def measure_prefill(engine, cfg, tokens, repeats=5, chunk=None):
     return sorted(times)[len(times) // 2]      # the median, as for the decode steps
 
 
-def second_model_points(preset, dtype, element, batch, context, prefill_tokens, steps, dtype_name) -> dict:
+def second_model_points(preset, dtype, element, batch, context, prefill_tokens, steps, dtype_name, pressure=0.0,
+                        mirror=False) -> dict:
     """Decode tokens a second and prefill tokens a second of another size of the model, every layer of it, with
-    their fractions of the published peaks: flat numbers for `points`, named by the size."""
+    their fractions of the published peaks: flat numbers for `points`, named by the size.  `pressure`: also the
+    batch from 512-token prompts in a pool of that share of what it needs; `mirror`: also the reference's own
+    workload (see measure_mirror)."""
     import gc
     import torch
     from sprout_lm_amd.cli import PRESETS
@@ -208,14 +254,25 @@ def second_model_points(preset, dtype, element, batch, context, prefill_tokens, 
     parts = engine.model.parts
     step_s, _ = measure_decode(engine, cfg, batch, context, steps, 3)
     prefill_s = measure_prefill(engine, cfg, prefill_tokens, repeats=3)
-    engine.close()
     read = decode_step_bytes(parts, batch, context, element)
-    return {f"{tag}_layers": cfg.num_hidden_layers,
-            f"{tag}_decode_b{batch}": round(batch / step_s, 1), f"{tag}_decode_b{batch}_ms": round(step_s * 1000, 4),
-            f"{tag}_decode_b{batch}_hbm_frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 5),
-            f"{tag}_prefill_{prefill_tokens}": round(prefill_tokens / prefill_s, 1),
-            f"{tag}_prefill_{prefill_tokens}_ms": round(prefill_s * 1000, 3),
-            f"{tag}_prefill_{prefill_tokens}_frac": round(prefill_flops(parts, prefill_tokens) / prefill_s / MFMA_PEAK[dtype_name], 5)}
+    out = {f"{tag}_layers": cfg.num_hidden_layers,
+           f"{tag}_decode_b{batch}": round(batch / step_s, 1), f"{tag}_decode_b{batch}_ms": round(step_s * 1000, 4),
+           f"{tag}_decode_b{batch}_hbm_frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 5),
+           f"{tag}_prefill_{prefill_tokens}": round(prefill_tokens / prefill_s, 1),
+           f"{tag}_prefill_{prefill_tokens}_ms": round(prefill_s * 1000, 3),
+           f"{tag}_prefill_{prefill_tokens}_frac": round(prefill_flops(parts, prefill_tokens) / prefill_s / MFMA_PEAK[dtype_name], 5)}
+    if pressure:
+        run = measure_pressure(engine.model, cfg, batch, 512, 256, pressure)
+        out.update({f"{tag}_pressure_share": pressure, f"{tag}_pressure_preemptions": run["preemptions"],
+                    f"{tag}_pressure_recomputed_tokens": run["recomputed_tokens"], f"{tag}_pressure_net_tok_s": run["net_value"]})
+    if mirror:
+        run = measure_mirror(engine.model, cfg)
+        read1 = decode_step_bytes(parts, 1, 47 + 16, element)
+        out.update({f"{tag}_mirror_decode_ms": run["decode_ms_mean"], f"{tag}_mirror_decode_ms_p95": run["decode_ms_p95"],
+                    f"{tag}_mirror_first_token_ms": run["first_token_ms"],
+                    f"{tag}_mirror_hbm_frac": round(read1 / (run["decode_ms_mean"] / 1000) / 1e9 / HBM_PEAK_GBS, 5)})
+    engine.close()
+    return out
 
 
 def main() -> int:
@@ -232,8 +289,13 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     parser.add_argument("--mixed-chunk", type=int, default=256,
                         help="also time the batch decoding beside a prompt prefilled this many tokens a step (0: skip)")
-    parser.add_argument("--second-preset", default="qwen2.5-7b",
-                        help="sizes of the second model whose decode step and prefill go into `points` ('' or 'none': skip)")
+    parser.add_argument("--second-preset", default="qwen2.5-7b,qwen2.5-32b",
+                        help="sizes of further models whose decode step and prefill go into `points`, every layer of "
+                             "them, where they fit the free device memory ('' or 'none': skip); at 32B sizes also the "
+                             "run under pool pressure and the reference's own workload (47 tokens in, 32 out, alone)")
+    parser.add_argument("--mirror", action="store_true",
+                        help="time nothing but the reference's own workload at --preset sizes (47 random tokens, 32 "
+                             "decoded, one request, a pool of 256 tokens); prints a shorter line")
     parser.add_argument("--prefill-only", action="store_true",
                         help="time nothing but the prefill of --prefill-tokens (for a profile of that step alone); "
                              "prints a shorter line")
@@ -254,6 +316,17 @@ def main() -> int:
     dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
     element = 2 if args.dtype == "bf16" else 4
 
+    if args.mirror:
+        engine = make_engine(cfg, dtype, 1, 256, 64)
+        run = measure_mirror(engine.model, cfg)
+        read1 = decode_step_bytes(engine.model.parts, 1, 47 + 16, element)
+        engine.close()
+        print(json.dumps({"metric": f"ms per decoded token, one request, 47 tokens in and 32 out ({args.preset} sizes)",
+                          "value": run["decode_ms_mean"], "unit": "ms", "n_gpus": 1, "higher_is_better": False,
+                          "dtype": args.dtype, "layers": cfg.num_hidden_layers, **run,
+                          "hbm_frac": round(read1 / (run["decode_ms_mean"] / 1000) / 1e9 / HBM_PEAK_GBS, 5)}))
+        return 0
+
     if args.prefill_only:
         engine = make_engine(cfg, dtype, 1, args.prefill_tokens, args.prefill_tokens)
         seconds = measure_prefill(engine, cfg, args.prefill_tokens)
@@ -268,7 +341,7 @@ def main() -> int:
     from sprout_lm_amd import ops
     measured = ops.probe_machine()
 
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    biggest = max(args.batch, 1 if args.no_points else 256)
     engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
     parts = engine.model.parts
     warmup = max(args.warmup, 1)
@@ -276,9 +349,11 @@ def main() -> int:
     step_s, spread = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
     points = {}
     if not args.no_points:
-        for b in (1, 64):
+        for b in (1, 64, 128, 256):
             s, _ = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
             points[f"decode_b{b}"] = round(b / s, 1)
+            if b > 64:
+                points[f"decode_b{b}_hbm_frac"] = round(decode_step_bytes(parts, b, args.context, element) / s / 1e9 / HBM_PEAK_GBS, 5)
     mixed = measure_mixed(engine, cfg, args.batch, args.context, args.mixed_chunk, min(args.steps, 12), 2) \
         if args.mixed_chunk else None
     # the same with the step cut back to a whole multiple of the chunk (step_token_multiple): 248 + 8 tokens
@@ -287,17 +362,19 @@ def main() -> int:
     prefill_s = measure_prefill(engine, cfg, args.prefill_tokens)
     portions = {str(c): round(args.prefill_tokens / measure_prefill(engine, cfg, args.prefill_tokens, 3, c), 1)
                 for c in (256, 512) if c < args.prefill_tokens and not args.no_points}
-    engine.close()
-    del engine
-    if not args.no_points and args.second_preset not in ("", "none", args.preset):
-        try:
-            points.update(second_model_points(args.second_preset, dtype, element, args.batch, args.context,
-                                              args.prefill_tokens, min(args.steps, 24), args.dtype))
-        except Exception as error:      # the headline above does not depend on the second model: say so and go on
-            print(f"bench.py: the points at {args.second_preset} sizes were not measured: {error}", file=sys.stderr)
     pressure = None
     if args.pressure:
-        pressure = measure_pressure(cfg, dtype, args.batch, 512, 256, args.pressure)
+        pressure = measure_pressure(engine.model, cfg, args.batch, 512, 256, args.pressure)
+    engine.close()
+    del engine
+    for preset in ([] if args.no_points else [p for p in args.second_preset.split(",") if p not in ("", "none", args.preset)]):
+        largest = preset.endswith("32b")
+        try:
+            points.update(second_model_points(preset, dtype, element, args.batch, args.context, args.prefill_tokens,
+                                              min(args.steps, 24), args.dtype, pressure=0.6 if largest else 0.0,
+                                              mirror=largest))
+        except Exception as error:      # the headline above does not depend on the further models: say so and go on
+            print(f"bench.py: the points at {preset} sizes were not measured: {error}", file=sys.stderr)
 
     read = decode_step_bytes(parts, args.batch, args.context, element)
     achieved = read / step_s / 1e9

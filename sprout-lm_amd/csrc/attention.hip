@@ -8,7 +8,8 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
                       float* workspace, bool single);
-size_t attention_generic_workspace_floats(int n_tiles, int nq, int nkv, int hd, int max_tile_ctx, bool single);
+size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
+                                          bool single);
 bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
@@ -59,7 +60,7 @@ static int64_t workspace_floats_of(int hd, int page_size, int nq, int nkv, int n
 extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
                                                  int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx) {
   if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind))   // (n_decode == n_tiles: every sequence brings one query)
-    return (int64_t)attention_generic_workspace_floats(n_tiles, nq, nkv, hd, max_tile_ctx, n_decode > 0 && n_decode == n_tiles);
+    return (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, n_decode > 0 && n_decode == n_tiles);
   return workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, n_tiles, max_tile_ctx);
 }
 
@@ -89,7 +90,7 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
     if (n_tiles == 0) return 0;
     SP_REQUIRE(max_tile_ctx >= 0, "sp_attention: negative context length");
     const bool single = n_decode > 0 && n_decode == n_tiles;
-    const int64_t need = (int64_t)attention_generic_workspace_floats(n_tiles, nq, nkv, hd, max_tile_ctx, single);
+    const int64_t need = (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, single);
     SP_REQUIRE(need == 0 || (workspace && workspace_floats >= need),
                "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
                (long long)need);

@@ -240,6 +240,19 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
   }
 }
 
+bool attention_f32_decode_takes(int hd, int page_size, int nq, int nkv);
+size_t attention_f32_decode_workspace_floats(int n_tiles, int nq, int hd, int max_ctx);
+int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                         const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* ctx_len,
+                         const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd, int page_size,
+                         int num_pages, int window, float scale, int max_ctx, float* workspace);
+
+// A step of one-query sequences in float32 storage goes to the matrix-core kernel of attention_f32.hip where
+// that takes the sizes.
+static bool f32_one_query(int dtype, bool single, int nq, int nkv, int hd, int page_size) {
+  return dtype == kF32 && single && attention_f32_decode_takes(hd, page_size, nq, nkv);
+}
+
 // How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
 // and long contexts; at most 32 chunks of at least 256 keys, whole groups of 32 keys each.
 static void generic_chunks(int n_tiles, int rows_of_blocks, int max_tile_ctx, int* n_chunks, int* chunk) {
@@ -254,7 +267,9 @@ static void generic_chunks(int n_tiles, int rows_of_blocks, int max_tile_ctx, in
 // Whether a step in which every sequence brings one query (`single`) takes the grouped form of the kernel.
 static bool generic_grouped(bool single, int nq, int nkv) { return single && nkv > 0 && nq % nkv == 0 && nq / nkv > 1 && nq / nkv <= AQ; }
 
-size_t attention_generic_workspace_floats(int n_tiles, int nq, int nkv, int hd, int max_tile_ctx, bool single) {
+size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
+                                          bool single) {
+  if (f32_one_query(dtype, single, nq, nkv, hd, page_size)) return attention_f32_decode_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
   int n_chunks, chunk;
   generic_chunks(n_tiles, generic_grouped(single, nq, nkv) ? nkv : nq, max_tile_ctx, &n_chunks, &chunk);
   return n_chunks > 1 ? size_t(n_tiles) * AQ * nq * n_chunks * (hd + 2) : 0;
@@ -300,6 +315,9 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);
+  if (f32_one_query(dtype, single, nq, nkv, hd, page_size))
+    return attention_f32_decode(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, tiles, n_tiles,
+                                out, nq, nkv, hd, page_size, num_pages, window, scale, max_tile_ctx, workspace);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,

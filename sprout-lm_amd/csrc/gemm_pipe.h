@@ -74,11 +74,19 @@ __host__ __device__ inline bool pipe_tile_of(const PipeTiles& tiles, int block, 
 // BN = 32 WN WAVES_N weight rows.  Blocks of up to four waves ask for the registers of two waves a SIMD: with
 // all 512 to itself the compiler keeps the accumulators in one half of them and copies all of them to the
 // other half and back around every turn of the ring.
-template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2 : 1)) void gemm_pipe_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w,
+//
+// TE: the operands' element type.  uint16_t: bfloat16, steps of 64 along K on 32x32x16 MFMA.  float: the same
+// bytes are steps of 32 along K, and a lane's 16-byte LDS read holds four numbers that feed four successive
+// v_mfma_f32_32x32x2_f32 (k-slot l / 32 of MFMA e is element 4 (l / 32) + e of the eight that a 32-byte slice of a
+// row holds, for both operands): true float32 products and sums, no reduced-precision mode, 1/8 of the bfloat16
+// rate per byte, so this form is bound by the matrix cores and not by its fetches.
+template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB, typename TE = uint16_t>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2 : 1)) void gemm_pipe_kernel(const TE* __restrict__ x, const TE* __restrict__ w,
                                                         const TB* __restrict__ bias, void* __restrict__ out, int T,
                                                         int N, int K, int k_per_split, RopeArgs rope) {
   constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int ESZ = sizeof(TE), KSTEP = 128 / ESZ;    // elements of a tile row
+  static_assert(ESZ == 2 || (MODE != kSilu && MODE != kRope && MODE != kStore), "float32 operands store or add float32");
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   constexpr int ROW = 128;                              // bytes of a tile row
   constexpr int STAGE = (BM + BN) * ROW;                // bytes of a stage
@@ -100,7 +108,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   if (!pipe_tile_of(tiles, blockIdx.x, &tile_t, &tile_n)) return;
   const int t0 = tile_t * BM, n0 = tile_n * BN;
   const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
-  const int steps = (k_end - k_begin) / 64;
+  const int steps = (k_end - k_begin) / KSTEP;
   typedef __attribute__((address_space(3))) unsigned char* lds_address_t;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_address_t)pipe_lds;   // the tiles' offset within the LDS
 
@@ -112,7 +120,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   for (int j = 0; j < LX; ++j) {
     const int r = 8 * (NW * j + wave) + (lane >> 3);
     const int piece = (lane & 7) ^ swz(r);
-    xoff[j] = uint32_t(min(r, T - 1 - t0)) * uint32_t(K) * 2u + piece * 16;
+    xoff[j] = uint32_t(min(r, T - 1 - t0)) * uint32_t(K) * uint32_t(ESZ) + piece * 16;
   }
 #pragma unroll
   for (int j = 0; j < LW; ++j) {
@@ -133,7 +141,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
     } else {
       row = min(r, N - 1 - n0);
     }
-    woff[j] = uint32_t(row) * uint32_t(K) * 2u + piece * 16;
+    woff[j] = uint32_t(row) * uint32_t(K) * uint32_t(ESZ) + piece * 16;
   }
   auto fetch = [&](int buf, int step) {
     const unsigned char* xs = xbase + size_t(step) * ROW;
@@ -164,18 +172,30 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
     const unsigned char* stage = pipe_lds + buf * STAGE;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      bf16x8 a[WM], b[WN];
+      uint4 a[WM], b[WN];
       const uint32_t xp = xrow0 + ((ks * 32) ^ xpos0), wp = wrow0 + ((ks * 32) ^ wpos0);
 #pragma unroll
       for (int i = 0; i < WM; ++i)
-        a[i] = as_bf16x8(*reinterpret_cast<const uint4*>(stage + ((i & 1) ? (xp ^ 64) : xp) + i * 32 * ROW));
+        a[i] = *reinterpret_cast<const uint4*>(stage + ((i & 1) ? (xp ^ 64) : xp) + i * 32 * ROW);
 #pragma unroll
       for (int j = 0; j < WN; ++j)
-        b[j] = as_bf16x8(*reinterpret_cast<const uint4*>(stage + ((j & 1) ? (wp ^ 64) : wp) + j * 32 * ROW));
+        b[j] = *reinterpret_cast<const uint4*>(stage + ((j & 1) ? (wp ^ 64) : wp) + j * 32 * ROW);
+      if constexpr (ESZ == 2) {
 #pragma unroll
-      for (int i = 0; i < WM; ++i)
+        for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < WN; ++j) acc[i][j] = mfma32(b[j], a[i], acc[i][j]);
+          for (int j = 0; j < WN; ++j) acc[i][j] = mfma32(as_bf16x8(b[j]), as_bf16x8(a[i]), acc[i][j]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j) {
+            acc[i][j] = mfma32_f32(__uint_as_float(b[j].x), __uint_as_float(a[i].x), acc[i][j]);
+            acc[i][j] = mfma32_f32(__uint_as_float(b[j].y), __uint_as_float(a[i].y), acc[i][j]);
+            acc[i][j] = mfma32_f32(__uint_as_float(b[j].z), __uint_as_float(a[i].z), acc[i][j]);
+            acc[i][j] = mfma32_f32(__uint_as_float(b[j].w), __uint_as_float(a[i].w), acc[i][j]);
+          }
+      }
     }
   };
 
@@ -201,14 +221,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   tile_epilogue<WM, WN, MODE, TB, WAVES_N>(acc, reinterpret_cast<float*>(pipe_lds), bias, out, T, N, t0, n0, rope);
 }
 
-template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB>
-inline int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const uint16_t* w, const TB* bias, void* out,
+template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB, typename TE = uint16_t>
+inline int launch_pipe_mode(hipStream_t s, int splits, const TE* x, const TE* w, const TB* bias, void* out,
                             int T, int N, int K, int k_per_split, const RopeArgs& rope = RopeArgs{}) {
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   constexpr size_t lds = size_t(STAGES) * (BM + BN) * 128;
   static bool raised = false;
   if (lds > 48 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB, TE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     if (e != hipSuccess) {
       set_error("sp_gemm (pipelined): cannot raise the LDS limit: %s", hipGetErrorString(e));
@@ -219,7 +239,7 @@ inline int launch_pipe_mode(hipStream_t s, int splits, const uint16_t* x, const 
   // the kernel's own numbering of tiles
   const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
   dim3 grid(8 * (tiles.own + tiles.run), 1, splits);
-  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope);
+  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB, TE><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope);
   return check_launch("sp_gemm (pipelined)");
 }
 

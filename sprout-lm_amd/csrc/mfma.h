@@ -21,6 +21,12 @@ __device__ __forceinline__ floatx16 mfma32(bf16x8 a, bf16x8 b, floatx16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
+// v_mfma_f32_32x32x2_f32: D[32x32] += A[32x2] . B[2x32] with float32 operands (a true 32-bit product).
+// Lane l holds A[l % 32][l / 32] and B[l / 32][l % 32]; D as above.
+__device__ __forceinline__ floatx16 mfma32_f32(float a, float b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
 __device__ __forceinline__ uint4 ldg128(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 

@@ -87,13 +87,17 @@ class KeptWorkspace(Workspace):
     def release(self, owner) -> None:
         """`owner`'s graph is gone (and the stream has been waited for): free what no other graph uses."""
         for key, kept in list(self._kept.items()):
-            for flat in list(kept):
+            still = []
+            for flat in kept:
                 users = self._users.get(id(flat), set())
                 users.discard(owner)
-                if not users:
-                    kept.remove(flat)
+                if users:
+                    still.append(flat)
+                else:
                     self._users.pop(id(flat), None)
-            if not kept:
+            if still:
+                self._kept[key] = still
+            else:
                 del self._kept[key]
 
     def nbytes(self) -> int:

@@ -49,7 +49,8 @@ class ModelRunner:
                  max_sequences: int, prefix_caching: bool = False, stop_token_ids=None, use_graphs: bool = True,
                  budget: MemoryBudget | None = None, parts=None):
         """`tensors`: the plan's tensors on the device, by checkpoint name (the dict is emptied as parts take
-        them).  The cache pools are counted against the free device memory before they are allocated."""
+        them); None: `parts` hold their tensors already (`with_pool_of_its_own`).  The cache pools are counted
+        against the free device memory before they are allocated."""
         self.plan, self.dtype, self.device = plan, dtype, device
         self.parts = parts if parts is not None else plan.instantiate()
         self.budget = budget or MemoryBudget()
@@ -59,7 +60,8 @@ class ModelRunner:
         if torch.device(device).type == "cuda":
             check_budget(0, self.cache.storage_bytes(dtype.itemsize), free_device_bytes(device), self.budget,
                          "cache pools (the weights are resident already)")
-        self.parts.bind(tensors, device, dtype)
+        if tensors is not None:
+            self.parts.bind(tensors, device, dtype)
         self.cache.attach_storage(dtype, device)
         self.workspace = Workspace(device)
         self.stager = DescriptorStager(device)
@@ -117,6 +119,15 @@ class ModelRunner:
                       **{k: cache_options[k] for k in ("block_size", "num_blocks", "max_sequences")})
         tensors = random_tensors(parts.expected_tensors(), seed, dtype=dtype, device=device)
         return cls(plan, tensors, dtype, device, budget=budget, parts=parts, **cache_options)
+
+    def with_pool_of_its_own(self, block_size: int, num_blocks: int, max_sequences: int, prefix_caching: bool = False,
+                             use_graphs: bool = True) -> "ModelRunner":
+        """A second runner over the same weights with a cache pool, workspace and recorded graphs of its own (a
+        small pool beside a large one, say).  The two must not step at the same time: the parts are shared."""
+        other = ModelRunner(self.plan, None, self.dtype, self.device, block_size, num_blocks, max_sequences,
+                            prefix_caching, self.stop_token_ids, use_graphs, self.budget, parts=self.parts)
+        other.load_notes = list(self.load_notes)
+        return other
 
     # ------------------------------------------------------------------ the step
     def _slot_views(self, ctx, call_index: int) -> dict:

@@ -255,8 +255,12 @@ def plain_attention(q, keys, values, nq, nkv, hd, first_pos, window, scale):
     return out
 
 
-def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=None, seed=0, hidden=None):
+def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=None, seed=0, hidden=None, exact_table=False,
+                  poison=None):
     """seqs: list of (ctx_len, q_len).  Pages are scattered over the pool in random order.
+
+    exact_table: a table row holds the longest sequence's pages and no entry more.  poison: a sequence whose pages
+    are filled with NaN after the expected values have been taken (its own rows of the result mean nothing).
 
     hidden: an output projection [hidden, nq * hd] is given along, which the kernels must fold in; what is
     compared is then what was added to a float32 residual."""
@@ -270,7 +274,7 @@ def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=Non
         kp, vp = bf16(kp), bf16(vp)
     T = sum(q for _, q in seqs)
     q = rng.standard_normal((T, nq * hd)).astype(np.float32)
-    max_blocks = max(-(-c // page) for c, _ in seqs) + 1
+    max_blocks = max(-(-c // page) for c, _ in seqs) + (0 if exact_table else 1)
     tables = np.full((len(seqs), max_blocks), -1, np.int32)
     keys, values, starts = [], [], []
     t0 = 0
@@ -293,6 +297,8 @@ def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=Non
             k, v = bf16(k), bf16(v)
         keys.append(k); values.append(v); starts.append(t0)
         t0 += qlen
+        if poison == s:
+            kp[blocks], vp[blocks] = np.nan, np.nan
     if dtype == torch.bfloat16:
         q, kp = bf16(q), bf16(kp)
     out = torch.full((T, nq * hd), float("nan"), dtype=dtype, device=DEV)
@@ -347,6 +353,21 @@ def test_attention_one_query_each_on_the_float32_kernel(dtype, nq, nkv, hd, page
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     assert not np.isnan(got).any()
     assert np.abs(got - want).max() <= tol * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
+@pytest.mark.parametrize("nq,nkv,hd,page", [(14, 2, 64, 16), (16, 1, 32, 8), (6, 3, 80, 12), (4, 4, 48, 4)])
+def test_attention_never_reads_past_a_sequence_s_table_row(dtype, kind, nq, nkv, hd, page):
+    """One-query sequences whose contexts fill the last page of their table row, the rows no wider than that: the
+    entry after a row's end is the next sequence's first page, here full of NaN.  A kernel that walks even one key
+    past its context multiplies that NaN by a zero probability and spoils the row."""
+    ctx = 8 * page
+    seqs = [(ctx, 1), (3, 1), (ctx, 1), (ctx - 1, 1), (5, 1)]
+    got, want = run_attention(dtype, nq, nkv, hd, page, seqs, kind=kind, seed=hd, exact_table=True, poison=1)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    keep = [0, 2, 3, 4]
+    assert not np.isnan(got[keep]).any()           # the poisoned sequence's own row may hold anything
+    assert np.abs(got[keep] - want[keep]).max() <= tol * (1 + np.abs(want[keep]).max())
 
 
 @pytest.mark.parametrize("dtype,kind", [(torch.float32, 1), (torch.bfloat16, 1), (torch.bfloat16, 0)])
