@@ -10,6 +10,7 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       float* workspace, bool single);
 size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
                                           bool single);
+int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size);
 bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
@@ -44,7 +45,7 @@ extern "C" int sp_attention_plan(int dtype, int hd, int page_size, int nq, int n
     plan[0] = attention_mfma_tile_q(hd);
     plan[1] = attention_mfma_decode_supports(nq, nkv) ? 0 : 1;
   } else {
-    plan[0] = 16;
+    plan[0] = attention_generic_tile_q(dtype, nq, nkv, hd, page_size);
     plan[1] = 1;
   }
   return 0;

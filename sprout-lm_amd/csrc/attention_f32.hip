@@ -228,6 +228,171 @@ __global__ __launch_bounds__(64) void attention_f32_merge_kernel(const float* __
   }
 }
 
+// ------------------------------------------------------------------------------------------------ several queries
+// Steps with portions of prompts: one block per (tile of 32 queries of a sequence, key/value head), one wave per
+// query head of the group, so the waves of a block walk the same keys at the same time and fetch them once between
+// them (the second wave on finds them in the CU's cache).  A wave holds two tiles of 16 queries as the B operands
+//   S^T[key, query] = K[key, :] . Q[query, :]       O^T[dim, query] += V^T[dim, key] . P^T[key, query]
+// and walks the keys 16 at a time from a multiple of 16, the next step's keys and values requested while the
+// current ones are multiplied (head sizes up to 64; above that the registers do not hold two steps).  Causal
+// mask and window by position; softmax statistics float32.  A sequence with one query is a tile with one row.
+// MAXW: the most waves (query heads of a group) a block may have; it sets the registers a wave may use.
+template <int DT, bool AHEAD, int MAXW>
+__global__ __launch_bounds__(64 * MAXW) void attention_f32_tiles_kernel(
+    const float* __restrict__ q, int q_stride, const float* __restrict__ k_pool, const float* __restrict__ v_pool,
+    const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
+    const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
+    float* __restrict__ out, int nq, int nkv, int page_size, int num_pages, int window, float scale2) {
+  constexpr int HD = 16 * DT;
+  const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
+  const int g = blockIdx.y, G = nq / nkv;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const int head = g * G + wave;
+  const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
+  const int nvalid = min(32, qlen - q_off);
+  if (nvalid <= 0) return;
+  const int pos0 = ctx - qlen + q_off;                 // position of the tile's first query
+  const int last_pos = pos0 + nvalid - 1;
+  const int32_t* table = block_tables + size_t(seq) * max_blocks;
+  PageDivider by_page;
+  by_page.d = page_size;
+  by_page.inv = 1.0f / float(page_size);
+  const size_t page_stride = size_t(nkv) * page_size * HD;
+  const float* kbase = k_pool + size_t(g) * page_size * HD;
+  const float* vbase = v_pool + size_t(g) * page_size * HD;
+
+  float4 qv[2][DT];
+  int qpos[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const int row = 16 * qt + lr;
+    qpos[qt] = row < nvalid ? pos0 + row : -1;
+#pragma unroll
+    for (int c = 0; c < DT; ++c)
+      qv[qt][c] = row < nvalid ? *reinterpret_cast<const float4*>(q + size_t(qs + q_off + row) * q_stride + head * HD + 16 * c + 4 * lj)
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  floatx4 o[2][DT];
+  float m[2] = {kNoKey, kNoKey}, lsum[2] = {0.f, 0.f};
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;     // the oldest key any query of the tile sees
+  const int first_key = (k_lo / kStep) * kStep;
+
+  auto load = [&](int key0, float4 (&kr)[DT], float4 (&vr)[DT]) {
+    int logical, slot;
+    by_page.divmod(min(max(key0 + lr, k_lo), last_pos), logical, slot);
+    int page = min(max(table[min(logical, max_blocks - 1)], 0), num_pages - 1);
+    const float* krow = kbase + size_t(page) * page_stride + size_t(slot) * HD + 4 * lj;
+#pragma unroll
+    for (int c = 0; c < DT; ++c) kr[c] = *reinterpret_cast<const float4*>(krow + 16 * c);
+    by_page.divmod(min(max(key0 + 4 * lj, (k_lo >> 2) << 2), (last_pos >> 2) << 2), logical, slot);
+    page = min(max(table[min(logical, max_blocks - 1)], 0), num_pages - 1);
+    const float* vcol = vbase + size_t(page) * page_stride + slot + size_t(lr) * page_size;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vr[dt] = *reinterpret_cast<const float4*>(vcol + size_t(16 * dt) * page_size);
+  };
+  auto attend = [&](int key0, const float4 (&kr)[DT], const float4 (&vr)[DT]) {
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      if (qt == 1 && nvalid <= 16) break;              // the same in every lane
+      floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DT; ++c) {
+        s = mfma4(kr[c].x, qv[qt][c].x, s);
+        s = mfma4(kr[c].y, qv[qt][c].y, s);
+        s = mfma4(kr[c].z, qv[qt][c].z, s);
+        s = mfma4(kr[c].w, qv[qt][c].w, s);
+      }
+      const int hi = qpos[qt], lo = window > 0 ? max(0, hi - window + 1) : 0;
+      float sv[4], top = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + 4 * lj + e;
+        sv[e] = (key >= lo && key <= hi) ? s[e] * scale2 : -INFINITY;      // hi = -1: a row that does not exist
+        top = fmaxf(top, sv[e]);
+      }
+      top = max_over_quarters(top);
+      const float m_new = fmaxf(m[qt], top);
+      const float alpha = exp2f(m[qt] - m_new);
+      m[qt] = m_new;
+      lsum[qt] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[qt][dt] *= alpha;
+      float p[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        p[e] = exp2f(sv[e] - m_new);
+        lsum[qt] += p[e];
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        o[qt][dt] = mfma4(vr[dt].x, p[0], o[qt][dt]);
+        o[qt][dt] = mfma4(vr[dt].y, p[1], o[qt][dt]);
+        o[qt][dt] = mfma4(vr[dt].z, p[2], o[qt][dt]);
+        o[qt][dt] = mfma4(vr[dt].w, p[3], o[qt][dt]);
+      }
+    }
+  };
+
+  if (AHEAD) {
+    float4 ka[DT], va[DT], kb[DT], vb[DT];
+    load(first_key, ka, va);
+    for (int key0 = first_key; key0 <= last_pos; key0 += 2 * kStep) {
+      const bool second = key0 + kStep <= last_pos;
+      if (second) load(key0 + kStep, kb, vb);
+      attend(key0, ka, va);
+      if (!second) break;
+      if (key0 + 2 * kStep <= last_pos) load(key0 + 2 * kStep, ka, va);
+      attend(key0 + kStep, kb, vb);
+    }
+  } else {
+    float4 ka[DT], va[DT];
+    for (int key0 = first_key; key0 <= last_pos; key0 += kStep) {
+      load(key0, ka, va);
+      attend(key0, ka, va);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    float l = lsum[qt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int row = 16 * qt + lr;
+    if (row >= nvalid) continue;
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* dst = out + size_t(qs + q_off + row) * (size_t(nq) * HD) + head * HD + 4 * lj;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+      *reinterpret_cast<float4*>(dst + 16 * dt) = make_float4(o[qt][dt][0] * inv, o[qt][dt][1] * inv, o[qt][dt][2] * inv, o[qt][dt][3] * inv);
+  }
+}
+
+template <int DT>
+int launch_tiles(hipStream_t s, const float* q, int q_stride, const float* k_pool, const float* v_pool,
+                 const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                 const int32_t* ctx_len, const int32_t* tiles, int n_tiles, float* out, int nq, int nkv, int page_size,
+                 int num_pages, int window, float scale) {
+  const int G = nq / nkv;
+  const dim3 grid(n_tiles, nkv);
+  if (G <= 4)
+    attention_f32_tiles_kernel<DT, (DT <= 8), 4><<<grid, 64 * G, 0, s>>>(
+        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
+        num_pages, window, scale * kLog2e);
+  else if (G <= 8)
+    attention_f32_tiles_kernel<DT, (DT <= 4), 8><<<grid, 64 * G, 0, s>>>(
+        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
+        num_pages, window, scale * kLog2e);
+  else
+    attention_f32_tiles_kernel<DT, false, 16><<<grid, 64 * G, 0, s>>>(
+        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
+        num_pages, window, scale * kLog2e);
+  return check_launch("sp_attention (float32, tiles)");
+}
+
 size_t decode_lds_bytes(int hd) { return sizeof(float) * (size_t(4) * 16 * (hd + 1) + 128) + sizeof(int32_t) * (kChunk / 4 + 4); }
 
 template <int DT, int SB>
@@ -308,6 +473,30 @@ int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void*
     default: SP_F32_DECODE(16, 1);
   }
 #undef SP_F32_DECODE
+}
+
+int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                        const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                        const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd,
+                        int page_size, int num_pages, int window, float scale) {
+  SP_REQUIRE(attention_f32_decode_takes(hd, page_size, nq, nkv), "sp_attention (float32, tiles): sizes not taken");
+  SP_REQUIRE((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool) |
+              reinterpret_cast<uintptr_t>(out)) % 16 == 0 && q_stride % 4 == 0,
+             "sp_attention (float32, tiles): operands must be 16-byte aligned");
+#define SP_F32_TILES(DT)                                                                                          \
+  case DT:                                                                                                        \
+    return launch_tiles<DT>(s, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool, block_tables, \
+                            max_blocks, q_start, q_len, ctx_len, tiles, n_tiles, (float*)out, nq, nkv, page_size,  \
+                            num_pages, window, scale)
+  switch (hd / 16) {
+    SP_F32_TILES(1); SP_F32_TILES(2); SP_F32_TILES(3); SP_F32_TILES(4); SP_F32_TILES(5); SP_F32_TILES(6);
+    SP_F32_TILES(7); SP_F32_TILES(8); SP_F32_TILES(9); SP_F32_TILES(10); SP_F32_TILES(11); SP_F32_TILES(12);
+    SP_F32_TILES(13); SP_F32_TILES(14); SP_F32_TILES(15);
+    default: return launch_tiles<16>(s, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,
+                                     block_tables, max_blocks, q_start, q_len, ctx_len, tiles, n_tiles, (float*)out, nq,
+                                     nkv, page_size, num_pages, window, scale);
+  }
+#undef SP_F32_TILES
 }
 
 }  // namespace sprout

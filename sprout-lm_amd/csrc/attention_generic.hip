@@ -247,10 +247,23 @@ int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void*
                          const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd, int page_size,
                          int num_pages, int window, float scale, int max_ctx, float* workspace);
 
-// A step of one-query sequences in float32 storage goes to the matrix-core kernel of attention_f32.hip where
-// that takes the sizes.
+int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                        const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
+                        const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd,
+                        int page_size, int num_pages, int window, float scale);
+
+// Float32 storage goes to the matrix-core kernels of attention_f32.hip where they take the sizes: a step of
+// one-query sequences to the one that shares a sequence's keys out over blocks, any other to the one that walks
+// tiles of 32 queries.
+bool attention_generic_on_matrix_cores(int dtype, int nq, int nkv, int hd, int page_size) {
+  return dtype == kF32 && attention_f32_decode_takes(hd, page_size, nq, nkv);
+}
 static bool f32_one_query(int dtype, bool single, int nq, int nkv, int hd, int page_size) {
-  return dtype == kF32 && single && attention_f32_decode_takes(hd, page_size, nq, nkv);
+  return single && attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size);
+}
+// Queries in a tile of the tile list that the kernels of this path expect.
+int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size) {
+  return attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size) ? 32 : AQ;
 }
 
 // How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
@@ -270,6 +283,7 @@ static bool generic_grouped(bool single, int nq, int nkv) { return single && nkv
 size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
                                           bool single) {
   if (f32_one_query(dtype, single, nq, nkv, hd, page_size)) return attention_f32_decode_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
+  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size)) return 0;
   int n_chunks, chunk;
   generic_chunks(n_tiles, generic_grouped(single, nq, nkv) ? nkv : nq, max_tile_ctx, &n_chunks, &chunk);
   return n_chunks > 1 ? size_t(n_tiles) * AQ * nq * n_chunks * (hd + 2) : 0;
@@ -318,6 +332,9 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
   if (f32_one_query(dtype, single, nq, nkv, hd, page_size))
     return attention_f32_decode(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, tiles, n_tiles,
                                 out, nq, nkv, hd, page_size, num_pages, window, scale, max_tile_ctx, workspace);
+  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size))
+    return attention_f32_tiles(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
+                               n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,

@@ -8,6 +8,9 @@ int gemm_generic(hipStream_t s, int a_dtype, const void* a, int w_dtype, const v
 int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode,
               int out_dtype, void* out, int T, int N, int K, bool* handled);
 bool gemm_f32_takes(int T, int N, int K, const void* a, const void* w, const void* out);
+bool gemm_f32_skinny_takes(int T, int N, int K, const void* a, const void* w);
+int gemm_f32_skinny(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
+                    int T, int N, int K);
 int gemm_f32(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out, int T,
              int N, int K);
 }  // namespace sprout
@@ -31,7 +34,9 @@ extern "C" int sp_gemm(void* stream, int a_dtype, const void* a, int w_dtype, co
     if (handled) return rc;
   }
   // float32 operands and a float32 result, more than a handful of tokens: the matrix cores' true 32-bit products
-  if (a_dtype == kF32 && w_dtype == kF32 && (mode != 0 || out_dtype == kF32) && gemm_f32_takes(T, N, K, a, w, out))
-    return gemm_f32(s, a, w, bias_dtype, bias, mode, out, T, N, K);
+  if (a_dtype == kF32 && w_dtype == kF32 && (mode != 0 || out_dtype == kF32)) {
+    if (gemm_f32_skinny_takes(T, N, K, a, w)) return gemm_f32_skinny(s, a, w, bias_dtype, bias, mode, out, T, N, K);
+    if (gemm_f32_takes(T, N, K, a, w, out)) return gemm_f32(s, a, w, bias_dtype, bias, mode, out, T, N, K);
+  }
   return gemm_generic(s, a_dtype, a, w_dtype, w, bias_dtype, bias, mode, out_dtype, out, T, N, K);
 }

@@ -107,22 +107,6 @@ def test_replay_with_pages_of_odd_sizes(folders, name, dtype, page):
     results = replay_in_process(folders[name], name, dtype, trace, None, page=page, num_blocks=pages, reused=reused)
     assert len(reused) >= 2, "no page of the pool served two requests"
     check(folders[name], dtype, requests, trace, results)
-    # the index names the request and position of every row, as the trace's builder knows them
-    index = [json.loads(line) for line in open(out / "index.jsonl")]
-    assert [r["step"] for r in index] == [s["step"] for s, rows in zip(trace.steps, trace.expected) if rows]
-    for record in index:
-        assert [(r["request"], r["position"]) for r in record["rows"]] == trace.expected[record["step"]]
-        assert [r["row"] for r in record["rows"]] == list(range(len(record["rows"])))
-    # the plain side of the same trace, file by file
-    from tests.plain import trace_plain
-    cfg, weights = H.plain_model(folders[name], dtype)
-    trace_plain.replay(cfg, weights, dtype, trace.steps[:12], str(tmp_path / "plain"))
-    plain_index = [json.loads(line) for line in open(tmp_path / "plain" / "index.jsonl")]
-    assert plain_index == index[:len(plain_index)] and plain_index
-    for record in plain_index:
-        want = np.fromfile(tmp_path / "plain" / record["file"], dtype="<f4")
-        got = np.fromfile(out / record["file"], dtype="<f4")
-        assert want.shape == got.shape and np.abs(want - got).max() <= H.tolerance(dtype, want)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -176,3 +160,19 @@ def test_trace_run_program(folders, tmp_path):
             assert not path.exists()
             results.append(None)
     check(folders[name], dtype, requests, trace, results)
+    # the index names the request and position of every row, as the trace's builder knows them
+    index = [json.loads(line) for line in open(out / "index.jsonl")]
+    assert [r["step"] for r in index] == [s["step"] for s, rows in zip(trace.steps, trace.expected) if rows]
+    for record in index:
+        assert [(r["request"], r["position"]) for r in record["rows"]] == trace.expected[record["step"]]
+        assert [r["row"] for r in record["rows"]] == list(range(len(record["rows"])))
+    # the plain side of the same trace, file by file
+    from tests.plain import trace_plain
+    cfg, weights = H.plain_model(folders[name], dtype)
+    trace_plain.replay(cfg, weights, dtype, trace.steps[:12], str(tmp_path / "plain"))
+    plain_index = [json.loads(line) for line in open(tmp_path / "plain" / "index.jsonl")]
+    assert plain_index == index[:len(plain_index)] and plain_index
+    for record in plain_index:
+        want = np.fromfile(tmp_path / "plain" / record["file"], dtype="<f4")
+        got = np.fromfile(out / record["file"], dtype="<f4")
+        assert want.shape == got.shape and np.abs(want - got).max() <= H.tolerance(dtype, want)
