@@ -229,9 +229,11 @@ __global__ __launch_bounds__(64) void attention_f32_merge_kernel(const float* __
 }
 
 // ------------------------------------------------------------------------------------------------ several queries
-// Steps with portions of prompts: one block per (tile of 32 queries of a sequence, key/value head), one wave per
-// query head of the group, so the waves of a block walk the same keys at the same time and fetch them once between
-// them (the second wave on finds them in the CU's cache).  A wave holds two tiles of 16 queries as the B operands
+// Steps with portions of prompts: one block per (tile of 32 queries of a sequence, up to four query heads of one
+// key/value head), one wave per head, so the waves of a block walk the same keys at the same time and fetch them
+// once between them (the second wave on finds them in the CU's cache) and every wave has a SIMD of its own: the
+// matrix cores bound this kernel, and a prompt's last tile, which walks every key, bounds the launch.  Tiles are
+// taken from the end of the list, the longest walks first.  A wave holds two tiles of 16 queries as the B operands
 //   S^T[key, query] = K[key, :] . Q[query, :]       O^T[dim, query] += V^T[dim, key] . P^T[key, query]
 // and walks the keys 16 at a time from a multiple of 16, the next step's keys and values requested while the
 // current ones are multiplied (head sizes up to 64; above that the registers do not hold two steps).  Causal
@@ -244,10 +246,13 @@ __global__ __launch_bounds__(64 * MAXW) void attention_f32_tiles_kernel(
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
     float* __restrict__ out, int nq, int nkv, int page_size, int num_pages, int window, float scale2) {
   constexpr int HD = 16 * DT;
-  const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
-  const int g = blockIdx.y, G = nq / nkv;
+  const int tile = gridDim.x - 1 - blockIdx.x;
+  const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
+  const int G = nq / nkv, parts = (G + MAXW - 1) / MAXW;      // a group's heads in `parts` blocks of up to MAXW
+  const int g = blockIdx.y / parts, part = blockIdx.y % parts;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
-  const int head = g * G + wave;
+  if (part * MAXW + wave >= G) return;
+  const int head = g * G + part * MAXW + wave;
   const int qlen = q_len[seq], ctx = ctx_len[seq], qs = q_start[seq];
   const int nvalid = min(32, qlen - q_off);
   if (nvalid <= 0) return;
@@ -376,20 +381,10 @@ int launch_tiles(hipStream_t s, const float* q, int q_stride, const float* k_poo
                  const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                  const int32_t* ctx_len, const int32_t* tiles, int n_tiles, float* out, int nq, int nkv, int page_size,
                  int num_pages, int window, float scale) {
-  const int G = nq / nkv;
-  const dim3 grid(n_tiles, nkv);
-  if (G <= 4)
-    attention_f32_tiles_kernel<DT, (DT <= 8), 4><<<grid, 64 * G, 0, s>>>(
-        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
-        num_pages, window, scale * kLog2e);
-  else if (G <= 8)
-    attention_f32_tiles_kernel<DT, (DT <= 4), 8><<<grid, 64 * G, 0, s>>>(
-        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
-        num_pages, window, scale * kLog2e);
-  else
-    attention_f32_tiles_kernel<DT, false, 16><<<grid, 64 * G, 0, s>>>(
-        q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
-        num_pages, window, scale * kLog2e);
+  const int G = nq / nkv, parts = (G + 3) / 4;
+  attention_f32_tiles_kernel<DT, (DT <= 8), 4><<<dim3(n_tiles, nkv * parts), 64 * min(G, 4), 0, s>>>(
+      q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
+      num_pages, window, scale * kLog2e);
   return check_launch("sp_attention (float32, tiles)");
 }
 

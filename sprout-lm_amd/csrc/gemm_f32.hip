@@ -72,13 +72,15 @@ namespace {
 
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-template <int RT, int MODE, typename TB>   // MODE: kStoreF32 or kAccumulate
+// MODE kSilu: w holds N gate rows, then N up rows; the block's RT tiles are RT / 2 tiles of gate rows and the
+// matching tiles of up rows, and out[t, n] = silu(gate) * up (float32 [T, N]).
+template <int RT, int MODE, typename TB>   // MODE: kStoreF32, kAccumulate or kSilu
 __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const TB* __restrict__ bias, float* __restrict__ out,
                                                               int T, int N, int K, int steps_per_block) {
   __shared__ float sums[4][RT][64][4];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
-  const int n0 = blockIdx.x * 16 * RT;
+  const int n0 = blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
   const int total_steps = (K + 15) / 16;
   const int first = blockIdx.y * steps_per_block, last = min(total_steps, first + steps_per_block);
   // this wave's steps of the block's: a contiguous quarter
@@ -87,7 +89,10 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
 
   const float* wrow[RT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) wrow[rt] = w + size_t(min(n0 + 16 * rt + lr, N - 1)) * K + 4 * lj;
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = MODE == kSilu ? min(n0 + 16 * (rt / 2) + lr, N - 1) + (rt & 1) * N : min(n0 + 16 * rt + lr, N - 1);
+    wrow[rt] = w + size_t(row) * K + 4 * lj;
+  }
   const float* xrow = x + size_t(min(lr, T - 1)) * K + 4 * lj;
   const bool token = lr < T;
 
@@ -123,6 +128,21 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
   __syncthreads();
   // thread (rt, lane) of the first RT waves' worth of threads joins the four waves: element e is
   // out[token lane % 16][n0 + 16 rt + 4 (lane / 16) + e]
+  if (MODE == kSilu) {
+    for (int i = threadIdx.x; i < RT / 2 * 64; i += 256) {
+      const int pair = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * pair + 4 * (l >> 4);
+      if (t >= T || n >= N) continue;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (n + e >= N) break;
+        const int a = 2 * pair, b = 2 * pair + 1;
+        const float gate = ((sums[0][a][l][e] + sums[1][a][l][e]) + sums[2][a][l][e]) + sums[3][a][l][e];
+        const float up = ((sums[0][b][l][e] + sums[1][b][l][e]) + sums[2][b][l][e]) + sums[3][b][l][e];
+        out[size_t(t) * N + n + e] = gate / (1.0f + expf(-gate)) * up;
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < RT * 64; i += 256) {
     const int rt = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * rt + 4 * (l >> 4);
     if (t >= T || n >= N) continue;
@@ -173,6 +193,17 @@ int skinny_shape(hipStream_t s, const float* x, const float* w, const void* bias
 
 }  // namespace
 
+// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for up to 16 tokens, float32 throughout.
+int gemm_f32_gated(hipStream_t s, const float* x, const float* w, float* out, int T, int I, int K) {
+  const int pairs = (I + 15) / 16;
+  if (pairs >= 2048) {
+    gemm_f32_skinny_kernel<4, kSilu, float><<<dim3((pairs + 1) / 2, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, (K + 15) / 16);
+  } else {
+    gemm_f32_skinny_kernel<2, kSilu, float><<<dim3(pairs, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, (K + 15) / 16);
+  }
+  return check_launch("sp_gate_up_silu (float32, few tokens)");
+}
+
 bool gemm_f32_skinny_takes(int T, int N, int K, const void* a, const void* w) {
   return T >= 1 && T <= 16 && K % 4 == 0 && K >= 64 &&
          (reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) % 16 == 0;
@@ -186,3 +217,19 @@ int gemm_f32_skinny(hipStream_t s, const void* a, const void* w, int bias_dtype,
 }
 
 }  // namespace sprout
+
+using namespace sprout;
+
+// Whether sp_gate_up_silu_f32 takes T tokens by 2 I rows of K.
+extern "C" int sp_gate_up_silu_f32_takes(int T, int I, int K) { return T >= 1 && T <= 16 && I >= 1 && K % 4 == 0 && K >= 64; }
+
+// out[T, I] (float32) = act(x . w[:I]^T) * (x . w[I:]^T), x float32 [T, K], w float32 [2 I, K], up to 16 tokens:
+// the gated product of a decode step on the float32 path, in one kernel.
+extern "C" int sp_gate_up_silu_f32(void* stream, const float* x, const float* w, float* out, int T, int I, int K,
+                                   int activation) {
+  SP_REQUIRE(activation == 0, "sp_gate_up_silu_f32: no kernel for activation %d (0 = SiLU)", activation);
+  SP_REQUIRE(sp_gate_up_silu_f32_takes(T, I, K), "sp_gate_up_silu_f32: shape T=%d I=%d K=%d is not taken", T, I, K);
+  SP_REQUIRE(x && w && out && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
+             "sp_gate_up_silu_f32: operands must be given and 16-byte aligned");
+  return gemm_f32_gated((hipStream_t)stream, x, w, out, T, I, K);
+}

@@ -110,6 +110,10 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 // dst (dst_dtype) = src (src_dtype), n elements
 
 // tokens[i] = previous[source[i]] for every i < n with source[i] >= 0 (others are left as they are):
+// The gated product of up to 16 tokens on the float32 path: out[T, I] = act(x . w[:I]^T) * (x . w[I:]^T), all float32.
+int sp_gate_up_silu_f32_takes(int T, int I, int K);
+int sp_gate_up_silu_f32(void* stream, const float* x, const float* w, float* out, int T, int I, int K, int activation);
+
 // dst[i] = a seeded random value, a function of (key, first + i) alone: the sum of twelve 16-bit fields of three
 // 64-bit hashes, centred, times scale (+ offset if add_offset): near normal with deviation 65536 * scale.
 // weights/random_init.py computes the same numbers on the host.

@@ -441,6 +441,20 @@ def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm
                                     variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
+def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> bool:
+    """out = act(x . w[:I]^T) * (x . w[I:]^T), everything float32, for the few tokens of a decode step.  Returns
+    False (and does nothing) where the kernel does not take the shape: the caller then multiplies and gates in turn."""
+    N, K = w.shape
+    T, I = out.shape
+    if (w.dtype != torch.float32 or x.dtype != torch.float32 or out.dtype != torch.float32 or N != 2 * I
+            or tuple(x.shape) != (T, K) or not library().sp_gate_up_silu_f32_takes(T, I, K)):
+        return False
+    _gpu(w, "gate/up weight"); _gpu(x, "activations"); _gpu(out, "gated output")
+    check(library().sp_gate_up_silu_f32(_stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), T, I, K,
+                                        variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+    return True
+
+
 def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
     """out[t, i] = act(gu[t, i]) * gu[t, I + i]."""
     _gpu(gu, "gate/up"); _gpu(out, "gated output")

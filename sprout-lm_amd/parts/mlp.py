@@ -61,6 +61,8 @@ class GatedMLP(FeedForward):
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
         if ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
             ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation)
+        elif ctx.act_dtype == torch.float32 and ops.gate_up_silu_f32(self.w_gate_up, h, act, activation=self.activation):
+            pass
         else:
             gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
             ops.gemm(h, self.w_gate_up, gu)

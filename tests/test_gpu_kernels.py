@@ -112,6 +112,20 @@ def test_gemm_float32_sums_for_few_tokens(T, N, K, a_dtype, w_dtype):
     assert np.abs(acc.cpu().numpy() - (base + want)).max() <= tol
 
 
+@pytest.mark.parametrize("T,I,K", [(1, 16, 64), (8, 4864, 896), (16, 37, 132), (5, 40000, 64), (3, 100, 4864)])
+def test_gated_product_of_few_tokens_in_float32(T, I, K):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T + I + K)
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    w = (rng.standard_normal((2 * I, K)) * 2 / math.sqrt(K)).astype(np.float32)
+    gate, up = x.astype(np.float64) @ w[:I].astype(np.float64).T, x.astype(np.float64) @ w[I:].astype(np.float64).T
+    want = gate / (1 + np.exp(-gate)) * up
+    out = torch.full((T, I), float("nan"), dtype=torch.float32, device=DEV)
+    assert ops.gate_up_silu_f32(t(w), t(x), out)
+    assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
+    assert not ops.gate_up_silu_f32(t(w), t(np.zeros((17, K), np.float32)), torch.empty(17, I, device=DEV))    # more tokens: not taken
+
+
 def test_gemm_mixed_operand_dtypes_and_refusals():
     from sprout_lm_amd import ops
     rng = np.random.default_rng(0)
