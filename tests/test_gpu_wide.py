@@ -46,7 +46,7 @@ def wide(request, tmp_path_factory):
     from sprout_lm_amd.cli import PRESETS
     from sprout_lm_amd.weights import write_model_folder
     preset, layers = WIDE[request.param]
-    raw = dict(PRESETS[preset], num_hidden_layers=layers, max_position_embeddings=1024)
+    raw = dict(PRESETS[preset], num_hidden_layers=layers, max_position_embeddings=2048)
     folder = str(tmp_path_factory.mktemp(f"wide_{request.param}"))
     write_model_folder(folder, S.config_from_dict(raw), seed=31, dtype=torch.bfloat16, std=0.02)
     return folder, raw, Plain(folder)
@@ -121,4 +121,23 @@ def test_mixed_replay_and_recorded_decode_at_the_widths_of_the_larger_models(wid
             err = np.abs(row - ref)
             worst = max(worst, float((err / bound(dtype, ref)).max()))
             assert np.all(err <= bound(dtype, ref)), f"recorded decode {k} position {first + i}: {err.max():.3e}"
+    del runner
+    torch.cuda.empty_cache()
+
+    if dtype == "bfloat16" and raw["hidden_size"] == 3584:
+        # one prompt of 2,048 tokens in one step, the size whose throughput is measured: the products' largest block
+        # shapes (q/k/v on blocks of 256 x 160 followed by the rotation kernel, the gated product on 256 x 256) and
+        # the prompt attention's long walks, tiles taken in pairs
+        tokens = H.random_tokens(vocab, 2048, 900)
+        places = [0, 255, 256, 1500, 2047]
+        runner = ModelRunner.from_folder(folder, dtype, block_size=16, num_blocks=130, max_sequences=1)
+        seq = runner.cache.create()
+        assert runner.cache.reserve(seq, len(tokens))
+        got = runner.step([StepEntry(seq, tokens, places)]).cpu().numpy()
+        want = plain.logits(dtype, tokens, places)
+        for row, ref, pos in zip(got, want, places):
+            err = np.abs(row - ref)
+            worst = max(worst, float((err / bound(dtype, ref)).max()))
+            assert np.all(err <= bound(dtype, ref)), f"long prompt position {pos}: {err.max():.3e}"
+        seq.release()
     print(f"wide {raw['hidden_size']} {dtype}: worst {worst:.2f} of the bound")
