@@ -57,8 +57,10 @@ class TraceSession:
             entries.append(StepEntry(seq, tokens, want))
         logits = None
         if entries:
-            # as generation runs a step: from a recorded graph where the step's shape has come before
-            logits = self.runner.step_recorded(entries)
+            logits = self._decode(entries)
+            if logits is None:
+                # as generation runs a step: from a recorded graph where the step's shape has come before
+                logits = self.runner.step_recorded(entries)
             if logits is None:
                 logits = self.runner.step(entries)
         for name in record.get("end", []):
@@ -66,6 +68,27 @@ class TraceSession:
             if seq is not None:
                 seq.release()
         return logits
+
+
+    def _decode(self, entries):
+        """A step in which every request brings one token runs as generation runs it: through the recorded decode
+        step (`ModelRunner.launch_decode`: its own descriptors, padded rows, the sampler inside).  What the sampler
+        draws is dropped; the logits of the wanted rows are returned.  None where that path does not take the step."""
+        from ..sampling.params import SamplingParams
+        from .batch import StepEntry
+        if any(len(e.tokens) != 1 or len(e.want) > 1 for e in entries):
+            return None
+        asked = [StepEntry(e.seq, e.tokens, [0]) for e in entries]
+        greedy = [SamplingParams(0.0, 0, None, True)] * len(asked)
+        pending = self.runner.launch_decode(asked, greedy, [0] * len(asked))
+        if pending is None:
+            return None
+        pending.result()
+        rows = [i for i, e in enumerate(entries) if e.want]
+        if len(rows) == len(entries):
+            return pending.logits[:len(rows)]
+        import torch
+        return pending.logits.index_select(0, torch.tensor(rows, dtype=torch.int64, device=pending.logits.device))
 
 
 def main(argv=None) -> int:
