@@ -76,7 +76,7 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   SP_REQUIRE(scores == 0, "sp_attention: no kernel for score stage %d (0 = the scaled product alone)", scores);
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
-  SP_REQUIRE(hd > 0 && hd <= 256, "sp_attention: head size %d is outside 1..256", hd);
+  SP_REQUIRE(hd > 0 && hd <= 512, "sp_attention: head size %d is outside 1..512", hd);
   SP_REQUIRE(page_size > 0 && num_pages > 0 && max_blocks > 0, "sp_attention: bad cache geometry");
   SP_REQUIRE(q_stride >= nq * hd, "sp_attention: q row stride %d is smaller than %d", q_stride, nq * hd);
   int plan[2];

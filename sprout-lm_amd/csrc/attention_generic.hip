@@ -1,5 +1,5 @@
 // Causal grouped-query attention of a mixed batch over paged keys and values, float32 arithmetic.
-// Any head size up to 256, any page size, any number of heads and groups, optional window.
+// Any head size up to 512, any page size, any number of heads and groups, optional window.
 // One block works on 16 queries of one sequence and one head, walking the keys 32 at a time with a
 // running maximum and sum (all float32).  Keys are always walked from a multiple of 32, so the order
 // of the sums at a position does not depend on how the tokens were cut into steps.
@@ -312,7 +312,24 @@ int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const v
         ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk)
   if (hd <= 64) { SP_ATT(4); }
   else if (hd <= 128) { SP_ATT(8); }
-  else { SP_ATT(16); }
+  else if (hd <= 256) { SP_ATT(16); }
+  else {
+    // head sizes up to 512: the tiles of queries, keys and probabilities need more LDS than a kernel gets unasked
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_generic_kernel<T, 32, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024);
+      if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_generic_kernel<T, 32, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024);
+      if (e != hipSuccess) {
+        set_error("sp_attention (generic): cannot raise the LDS limit: %s", hipGetErrorString(e));
+        return 1;
+      }
+      raised = true;
+    }
+    SP_ATT(32);
+  }
 #undef SP_ATT
   if (check_launch("sp_attention (generic)")) return 1;
   if (n_chunks == 1) return 0;

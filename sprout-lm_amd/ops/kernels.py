@@ -64,7 +64,7 @@ def _ptr(t):
 ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox")
 GATE_ACTIVATIONS = {"silu": 0}
 SCORE_STAGES = {"scaled_dot": 0}         # what stands between q . k and the softmax: the scale and nothing else
-MAX_HEAD_DIM = 256                       # the largest head size any attention kernel takes
+MAX_HEAD_DIM = 512                       # the largest head size any attention kernel takes
 
 
 def variant_code(table: dict, name: str, what: str) -> int:
@@ -76,8 +76,8 @@ def variant_code(table: dict, name: str, what: str) -> int:
 
 def check_attention_sizes(heads: int, kv_heads: int, head_dim: int) -> None:
     """Raises KernelError unless some attention kernel takes these sizes (any page size goes with them).
-    Head sizes of 16 ... 96 in steps of 16 and 128 run on the matrix cores in bfloat16, every other size up to
-    256, and everything in float32, on the general kernel."""
+    Head sizes of 16 ... 96 in steps of 16 and 128 run on the matrix cores in bfloat16, float32 in steps of 16 up
+    to 256 on the matrix cores' float32 instructions, every other size up to 512 on the general kernel."""
     if kv_heads <= 0 or heads <= 0 or heads % kv_heads:
         raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key/value heads")
     if not 0 < head_dim <= MAX_HEAD_DIM:

@@ -84,8 +84,10 @@ def test_sizes_that_no_kernel_takes_are_refused_when_the_parts_are_built():
     from sprout_lm_amd.config.base import ConfigError
     from sprout_lm_amd.models.plan import PartPlan
     from sprout_lm_amd import ops
-    raw = dict(H.TINY_A, hidden_size=1024, num_attention_heads=2, num_key_value_heads=1)     # head size 512
-    with pytest.raises(ConfigError, match="head size 512 is outside 1..256"):
+    raw = dict(H.TINY_A, hidden_size=1024, num_attention_heads=2, num_key_value_heads=1)     # head size 512: taken
+    S.build_model_plan(S.config_from_dict(raw)).instantiate()
+    raw = dict(H.TINY_A, hidden_size=1056, num_attention_heads=2, num_key_value_heads=1)     # head size 528
+    with pytest.raises(ConfigError, match="head size 528 is outside 1..512"):
         S.build_model_plan(S.config_from_dict(raw)).instantiate()
     with pytest.raises(ValueError, match="'gelu' has no kernel"):
         PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "gelu"}).make()

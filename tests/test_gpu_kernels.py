@@ -337,10 +337,11 @@ def run_attention(dtype, nq, nkv, hd, page, seqs, window=None, kind=0, spike=Non
     return got, want
 
 
-# the last two: pages whose size is no power of two (the kernel that walks pages without LDS staging), and one
-# that is no multiple of 4 either (the float32-arithmetic kernel takes it, whatever the storage type)
+# (4, 2, 64, 12) and (5, 1, 48, 6): pages whose size is no power of two (the kernel that walks pages without LDS
+# staging), and one that is no multiple of 4 either (the float32-arithmetic kernel takes it, whatever the storage
+# type); then head sizes above 256 (the general kernel with a larger tile) and one that is no multiple of 16
 ATT_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 8), (5, 5, 48, 16), (14, 2, 64, 16), (8, 2, 128, 32), (6, 3, 80, 4), (2, 1, 256, 16),
-              (4, 2, 64, 12), (5, 1, 48, 6)]
+              (4, 2, 64, 12), (5, 1, 48, 6), (2, 1, 320, 16), (1, 1, 512, 8), (3, 1, 40, 16)]
 ATT_BATCHES = [[(1, 1)], [(17, 17)], [(70, 1), (33, 33), (9, 2), (130, 5)], [(300, 300)], [(513, 1), (64, 64), (257, 2)]]
 
 
@@ -477,10 +478,10 @@ def test_attention_refuses_what_it_cannot_take():
     table = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
     with pytest.raises(ops.KernelError, match="groups"):
         ops.attention(q, 64, pool, pool, table, batch, torch.empty_like(q), 4, 3, 16, None, 0.25, kind=1)
-    big = torch.zeros(1, 512, device=DEV)
-    pool = torch.zeros(2, 1, 16, 512, device=DEV)
-    with pytest.raises(ops.KernelError, match="head size"):
-        ops.attention(big, 512, pool, pool.transpose(2, 3).contiguous(), table, batch, torch.empty_like(big), 1, 1, 512, None, 0.1, kind=1)
+    big = torch.zeros(1, 528, device=DEV)
+    pool = torch.zeros(2, 1, 16, 528, device=DEV)
+    with pytest.raises(ops.KernelError, match="head size 528 is outside 1..512"):
+        ops.attention(big, 528, pool, pool.transpose(2, 3).contiguous(), table, batch, torch.empty_like(big), 1, 1, 528, None, 0.1, kind=1)
 
 
 @pytest.mark.parametrize("dtype,kind", [(torch.bfloat16, 0), (torch.float32, 1)])
