@@ -197,27 +197,46 @@ __global__ __launch_bounds__(256) void attention_f32_decode_kernel(
   }
 }
 
-// Joins the chunks of one (sequence, head), in the order of the chunks: grid (sequences, heads), one wave.
+// Joins the chunks of one (sequence, head), in the order of the chunks: grid (sequences, heads), one wave.  What a
+// lane reads depends on its indices alone (empty chunks say so themselves), so it asks for 16 chunks at a time.
 __global__ __launch_bounds__(64) void attention_f32_merge_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml,
                                                                  const int32_t* __restrict__ q_start,
                                                                  const int32_t* __restrict__ tiles,
                                                                  float* __restrict__ out, int n_splits, int nq, int hd) {
+  constexpr int GROUP = 16;
   const int ti = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int seq = tiles[2 * ti];
   const size_t base = (size_t(ti) * nq + head) * n_splits;
-  float mx = kNoKey;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, part_ml[2 * (base + s)]);
-  float den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < n_splits; ++s) {
-    const float l = part_ml[2 * (base + s) + 1];
-    if (l > 0.f) {                                  // an empty chunk left nothing to read
-      const float f = exp2f(part_ml[2 * (base + s)] - mx);
-      den = fmaf(f, l, den);
+  float mx = kNoKey, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0; s0 < n_splits; s0 += GROUP) {
+    float ms[GROUP], ls[GROUP], os[GROUP][4];
+#pragma unroll
+    for (int i = 0; i < GROUP; ++i) {
+      const bool in = s0 + i < n_splits;
+      ms[i] = in ? part_ml[2 * (base + s0 + i)] : kNoKey;
+      ls[i] = in ? part_ml[2 * (base + s0 + i) + 1] : 0.f;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int d = lane + 64 * j;
-        if (d < hd) num[j] = fmaf(f, part_o[(base + s) * hd + d], num[j]);
+        os[i][j] = (in && d < hd) ? part_o[(base + s0 + i) * hd + d] : 0.f;
+      }
+    }
+    float top = mx;
+#pragma unroll
+    for (int i = 0; i < GROUP; ++i) top = fmaxf(top, ms[i]);
+    const float keep = exp2f(mx - top);
+    mx = top;
+    den *= keep;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) num[j] *= keep;
+#pragma unroll
+    for (int i = 0; i < GROUP; ++i) {
+      if (ls[i] > 0.f) {                      // an empty chunk left nothing to read in part_o
+        const float f = exp2f(ms[i] - mx);
+        den = fmaf(f, ls[i], den);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) num[j] = fmaf(f, os[i][j], num[j]);
       }
     }
   }

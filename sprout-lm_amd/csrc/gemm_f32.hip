@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  constexpr int U = 4;      // steps requested together
+  constexpr int U = RT <= 2 ? 8 : 4;      // steps requested together: what a wave has on its way
   for (int s = s0; s < s1; s += U) {
     float4 wv[U][RT], xv[U];
 #pragma unroll
