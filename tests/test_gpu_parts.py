@@ -1007,3 +1007,177 @@ def test_a_layer_with_two_mixers_that_both_keep_something(tmp_path, dtype):
             fed[k] += 1
     assert runner._graphs.replays == 17
     print(f"two mixers a layer {dtype}: worst {worst:.2f} of the bound")
+
+
+# A fourth toy: a mixer whose cached keys and values differ in width and are kept in float32 whatever the model
+# computes in (`PagedKVSpec.value_dim`, `.dtype`).  No attention kernel of the engine takes such a cache; the toy
+# gathers its pages itself.  What is shown is that the cache manager, the step's block tables and slot mapping and
+# the runner serve a cache of that description without a change to the engine's files.
+
+def register_latent_toy():
+    from dataclasses import dataclass
+    from typing import ClassVar
+
+    import sprout_lm_amd as S
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.cache import PagedKVSpec
+    from sprout_lm_amd.config.base import ModelConfig
+    from sprout_lm_amd.models.plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+    from sprout_lm_amd.parts import Mixer, register_part, registered_parts
+    from sprout_lm_amd.weights import TensorSpec
+
+    if "toy_narrow_values" in registered_parts("mixer"):
+        return
+
+    @register_part("mixer", "toy_narrow_values")
+    class NarrowValues(Mixer):
+        """Causal attention of `heads` query heads over ONE cached key of width key_dim and ONE cached value of
+        width value_dim per token (no position encoding): y = W_o . concat_h softmax(q_h . k / sqrt(key_dim)) . v."""
+
+        def __init__(self, hidden, heads, key_dim, value_dim):
+            self.hidden, self.heads, self.key_dim, self.value_dim = hidden, heads, key_dim, value_dim
+
+        def cache_spec(self):
+            return PagedKVSpec(1, self.key_dim, value_dim=self.value_dim, dtype="float32")
+
+        def cache_elements_per_token(self):
+            return self.key_dim + self.value_dim
+
+        def tensors(self):
+            return {"q.weight": TensorSpec((self.heads * self.key_dim, self.hidden)), "k.weight": TensorSpec((self.key_dim, self.hidden)),
+                    "v.weight": TensorSpec((self.value_dim, self.hidden)), "o.weight": TensorSpec((self.hidden, self.heads * self.value_dim))}
+
+        def forward(self, ctx, h, residual, cache):
+            T = h.shape[0]
+            out = {}
+            for name, width in (("q", self.heads * self.key_dim), ("k", self.key_dim), ("v", self.value_dim)):
+                out[name] = torch.empty(T, width, dtype=h.dtype, device=h.device)
+                ops.gemm(h, self.w[f"{name}.weight"], out[name])
+            pages, page = cache.k.shape[0], cache.page_size
+            assert cache.k.shape == (pages, 1, page, self.key_dim) and cache.v.shape == (pages, 1, self.value_dim, page)
+            assert cache.k.dtype == cache.v.dtype == torch.float32
+            slots = cache.slot_mapping[:T].long()
+            cache.k.view(pages * page, self.key_dim)[slots] = out["k"].float()
+            cache.v[slots // page, 0, :, slots % page] = out["v"].float()
+            mixed = torch.empty(T, self.heads * self.value_dim, dtype=torch.float32, device=h.device)
+            for s, (start, n, length) in enumerate(zip(ctx.host["q_start"], ctx.host["q_len"], ctx.host["ctx_len"])):
+                table = cache.block_tables[s, :-(-int(length) // page)].long()
+                keys = cache.k[table, 0].reshape(-1, self.key_dim)[:length]
+                values = cache.v[table, 0].permute(0, 2, 1).reshape(-1, self.value_dim)[:length]
+                q = out["q"][start:start + n].float().view(n, self.heads, self.key_dim)
+                scores = torch.einsum("nhd,kd->nhk", q, keys) / math.sqrt(self.key_dim)
+                position = (length - n + torch.arange(n, device=h.device))[:, None, None]
+                scores = scores.masked_fill(torch.arange(length, device=h.device)[None, None, :] > position, float("-inf"))
+                mixed[start:start + n] = torch.einsum("nhk,kv->nhv", torch.softmax(scores, -1), values).reshape(n, -1)
+            ops.gemm(mixed.to(h.dtype), self.w["o.weight"], residual, accumulate=True)
+
+    @dataclass(frozen=True)
+    class LatentConfig(ModelConfig):
+        architecture: ClassVar[str] = "ToyLatentForCausalLM"
+        model_types: ClassVar[tuple] = ("toy_latent",)
+        hidden: int = 0
+        inner: int = 0
+        vocab: int = 0
+        heads: int = 0
+        key_dim: int = 0
+        value_dim: int = 0
+        eps: float = 0.0
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(**{k: raw[k] for k in ("hidden", "inner", "vocab", "heads", "key_dim", "value_dim", "eps")})
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "model_type": "toy_latent",
+                    **{k: getattr(self, k) for k in ("hidden", "inner", "vocab", "heads", "key_dim", "value_dim", "eps")}}
+
+    def build(cfg):
+        norm = lambda prefix: PartPlan("norm", "rmsnorm", {"size": cfg.hidden, "eps": cfg.eps}, prefix)
+        mlp = lambda prefix: PartPlan("feed_forward", "gated_mlp", {"hidden": cfg.hidden, "inner": cfg.inner}, prefix)
+        hd = cfg.hidden // cfg.heads
+        mixers = [PartPlan("mixer", "attention", {"hidden": cfg.hidden, "heads": cfg.heads, "kv_heads": cfg.heads, "head_dim": hd,
+                                                  "position": PartPlan("position", "rotary_neox", {"head_dim": hd, "theta": 1e4})}, "l0.attn."),
+                  PartPlan("mixer", "toy_narrow_values", {"hidden": cfg.hidden, "heads": cfg.heads, "key_dim": cfg.key_dim,
+                                                          "value_dim": cfg.value_dim}, "l1.mix.")]
+        layers = [LayerPlan("pre_norm", {"mixer_norm": norm(f"l{i}.n1."), "mixer": m, "ffn_norm": norm(f"l{i}.n2."),
+                                         "ffn": mlp(f"l{i}.mlp.")}) for i, m in enumerate(mixers)]
+        return ModelPlan("ToyLatentForCausalLM", cfg, cfg.hidden, cfg.vocab, 512, (0,),
+                         PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.hidden}, "embed."),
+                         layers, [LayerCall(0, 0), LayerCall(1, 1)], norm("final."),
+                         PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.hidden, "tied": True}, "head."))
+
+    S.register_architecture("ToyLatentForCausalLM", LatentConfig, build, model_types=("toy_latent",))
+
+
+LATENT = dict(model_type="toy_latent", hidden=64, inner=96, vocab=103, heads=2, key_dim=24, value_dim=8, eps=1e-6)
+
+
+def plain_latent_logits(w, tokens, store):
+    c = LATENT
+    hd = c["hidden"] // c["heads"]
+    pos = np.arange(len(tokens))
+    x = P.f32(w["embed.weight"][np.asarray(tokens)])
+
+    def mlp(x, i):
+        n = store(P.rms_norm(x, w[f"l{i}.n2.weight"], c["eps"]))
+        gate, up = store(P.linear(n, w[f"l{i}.mlp.gate_proj.weight"])), store(P.linear(n, w[f"l{i}.mlp.up_proj.weight"]))
+        return P.f32(x + P.linear(store(P.swiglu(gate, up)), w[f"l{i}.mlp.down_proj.weight"]))
+
+    n = store(P.rms_norm(x, w["l0.n1.weight"], c["eps"]))
+    p = "l0.attn."
+    q = store(P.rope_neox(store(P.linear(n, w[p + "q_proj.weight"], w[p + "q_proj.bias"])), pos, hd, 1e4))
+    k = store(P.rope_neox(store(P.linear(n, w[p + "k_proj.weight"], w[p + "k_proj.bias"])), pos, hd, 1e4))
+    v = store(P.linear(n, w[p + "v_proj.weight"], w[p + "v_proj.bias"]))
+    a = store(P.causal_gqa_attention(q, k, v, c["heads"], c["heads"], hd))
+    x = mlp(P.f32(x + P.linear(a, w[p + "o_proj.weight"])), 0)
+    n = store(P.rms_norm(x, w["l1.n1.weight"], c["eps"]))
+    q = store(P.linear(n, w["l1.mix.q.weight"])).astype(np.float64).reshape(len(tokens), c["heads"], c["key_dim"])
+    k = store(P.linear(n, w["l1.mix.k.weight"])).astype(np.float64)
+    v = store(P.linear(n, w["l1.mix.v.weight"])).astype(np.float64)
+    mixed = np.zeros((len(tokens), c["heads"] * c["value_dim"]))
+    for t in range(len(tokens)):
+        for h in range(c["heads"]):
+            s = k[:t + 1] @ q[t, h] / math.sqrt(c["key_dim"])
+            e = np.exp(s - s.max())
+            mixed[t, h * c["value_dim"]:(h + 1) * c["value_dim"]] = (e / e.sum()) @ v[:t + 1]
+    x = mlp(P.f32(x + P.linear(store(P.f32(mixed)), w["l1.mix.o.weight"])), 1)
+    return P.linear(store(P.rms_norm(x, w["final.weight"], c["eps"])), w["embed.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_cache_whose_keys_and_values_differ_in_width(tmp_path, dtype):
+    """Keys of 24 numbers, values of 8, both kept in float32 under either compute dtype, beside an ordinary
+    attention layer: two cache groups, the toy's pools of the shapes and dtype it asked for; mixed replay with so
+    few pages that they are used again, against the plain function."""
+    register_latent_toy()
+    import sprout_lm_amd as S
+    from sprout_lm_amd.engine import ModelRunner
+    from sprout_lm_amd.engine.trace import TraceSession
+    from sprout_lm_amd.weights import write_model_folder
+    from tests import traces
+    folder = str(tmp_path / "latent")
+    write_model_folder(folder, S.config_from_dict(LATENT), seed=41, dtype=torch.bfloat16, std=0.15)
+    from safetensors.torch import load_file
+    w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    store = P.bf16_round if dtype == "bfloat16" else P.f32
+    tol = 3e-5 if dtype == "float32" else 5e-2
+    requests = {f"r{i}": H.random_tokens(103, n, 60 + i) for i, n in enumerate([37, 12, 58, 41, 26])}
+    want = {k: plain_latent_logits(w, t, store) for k, t in requests.items()}
+    pool = sum(sorted(-(-len(t) // 8) for t in requests.values())[-4:])
+    runner = ModelRunner.from_folder(folder, dtype, block_size=8, num_blocks=pool, max_sequences=4)
+    ordinary, narrow = runner.cache.groups
+    assert narrow.k.shape == (1, pool, 1, 8, 24) and narrow.v.shape == (1, pool, 1, 8, 8) and narrow.v.dtype == torch.float32
+    assert ordinary.k.dtype == (torch.float32 if dtype == "float32" else torch.bfloat16) and ordinary.k.shape[-1] == 32
+    assert not runner.parts.graph_safe
+    worst = 0.0
+    for trace in (traces.mixed(requests, seed=9), traces.portions(requests)):
+        session = TraceSession(runner)
+        for record, rows in zip(trace.steps, trace.expected):
+            logits = session.run_step(record)
+            got = logits.cpu().numpy() if rows else None
+            for i, (rid, pos) in enumerate(rows):
+                err = np.abs(got[i] - want[rid][pos]).max() / (tol * (1 + np.abs(want[rid][pos]).max()))
+                worst = max(worst, err)
+                assert err <= 1.0, f"{rid} position {pos}: {err:.2f} of the bound"
+        assert runner.cache.free_pages() == [pool, pool] and not session.live
+    print(f"narrow values {dtype}: worst {worst:.2f} of the bound")
