@@ -66,54 +66,109 @@ int gemm_f32(hipStream_t s, const void* a, const void* w, int bias_dtype, const 
 // A lane loads 16 bytes of a weight row (4 numbers that feed 4 successive MFMAs) and 16 bytes of a token's
 // activations, which serve every row tile of the wave; no sum crosses lanes.  The four waves' sums meet in LDS
 // in a fixed order.  K must be a multiple of 4.
+// NORM: the activations are rmsnorm(x) * norm_w of the float32 residual x, computed here ((x * scale) * w, the
+// very numbers the norm kernel stores): every block sums the squares of its tokens' rows first.
+// MODE kSilu: w holds N gate rows, then N up rows; the block's RT tiles are RT / 2 tiles of gate rows and the
+// matching tiles of up rows, and out[t, n] = silu(gate) * up (float32 [T, N]).
+// MODE kRope: the rows of w are q, k and v heads of size hd (a multiple of 16); a block's tile is 8 dimensions of
+// a head's first half (tile rows 0-7) and their rotation partners half a head further on (rows 8-15): twice the
+// blocks of whole tiles of 16, and these products live on how many blocks stream.  Bias, rotation of q and k
+// heads by positions * inv_freq (angle, sine and cosine in float64 where inv_freq_tail is given), q to out
+// [T, nq * hd], k and v into the paged pools.
 namespace sprout {
 
 namespace {
 
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-// MODE kSilu: w holds N gate rows, then N up rows; the block's RT tiles are RT / 2 tiles of gate rows and the
-// matching tiles of up rows, and out[t, n] = silu(gate) * up (float32 [T, N]).
-template <int RT, int MODE, typename TB>   // MODE: kStoreF32, kAccumulate or kSilu
+struct SkinnyExtra {
+  const float* norm_w;          // NORM
+  float eps;
+  // kRope
+  const int32_t* positions;
+  const float* inv_freq;
+  const float* inv_freq_tail;   // may be null
+  const int32_t* slot_mapping;
+  float* k_pool;                // [page][kv head][slot][dim]
+  float* v_pool;                // [page][kv head][dim][slot]
+  int nq, nkv, hd, page_size, num_pages;
+};
+
+template <int RT, int MODE, typename TB, bool NORM>   // MODE: kStoreF32, kAccumulate, kSilu or kRope
 __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const TB* __restrict__ bias, float* __restrict__ out,
-                                                              int T, int N, int K, int steps_per_block) {
+                                                              int T, int N, int K, int steps_per_block, SkinnyExtra extra) {
   __shared__ float sums[4][RT][64][4];
+  __shared__ float row_scale[16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
-  const int n0 = blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
   const int total_steps = (K + 15) / 16;
   const int first = blockIdx.y * steps_per_block, last = min(total_steps, first + steps_per_block);
   // this wave's steps of the block's: a contiguous quarter
   const int mine = (last - first + 3) / 4;
   const int s0 = first + wave * mine, s1 = min(last, s0 + mine);
 
+  int n0 = blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
   const float* wrow[RT];
+  if (MODE == kRope) {
+    static_assert(MODE != kRope || RT == 1, "a block of the rotating product is one tile: 8 dimensions and their partners");
+    const int per_head = extra.hd / 16, head = blockIdx.x / per_head, u = blockIdx.x % per_head;
+    n0 = head * extra.hd + 8 * u;
+    wrow[0] = w + size_t(n0 + (lr & 7) + (lr >> 3) * (extra.hd / 2)) * K + 4 * lj;
+  } else {
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int row = MODE == kSilu ? min(n0 + 16 * (rt / 2) + lr, N - 1) + (rt & 1) * N : min(n0 + 16 * rt + lr, N - 1);
-    wrow[rt] = w + size_t(row) * K + 4 * lj;
+    for (int rt = 0; rt < RT; ++rt) {
+      const int row = MODE == kSilu ? min(n0 + 16 * (rt / 2) + lr, N - 1) + (rt & 1) * N : min(n0 + 16 * rt + lr, N - 1);
+      wrow[rt] = w + size_t(row) * K + 4 * lj;
+    }
   }
   const float* xrow = x + size_t(min(lr, T - 1)) * K + 4 * lj;
   const bool token = lr < T;
 
-  floatx4_t acc[RT];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-
   constexpr int U = RT <= 2 ? 8 : 4;      // steps requested together: what a wave has on its way
-  for (int s = s0; s < s1; s += U) {
-    float4 wv[U][RT], xv[U];
+  float4 wv[U][RT], xv[U], nv[U];
+  auto request = [&](int s) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = 16 * (s + u);
       const bool in = s + u < s1 && k + 4 * lj < K;
       xv[u] = (in && token) ? *reinterpret_cast<const float4*>(xrow + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (NORM) nv[u] = in ? *reinterpret_cast<const float4*>(extra.norm_w + k + 4 * lj) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
         wv[u][rt] = in ? *reinterpret_cast<const float4*>(wrow[rt] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
+  };
+  // the first steps' weights are asked for before the norm is worked out: they do not depend on it
+  request(s0);
+
+  float scale = 1.f;
+  if (NORM) {
+    // thread (token threadIdx.x / 16, part threadIdx.x % 16) sums its sixteenth of the row's squares
+    const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
+    float sum = 0.f;
+    if (t < T)
+      for (int k = 4 * part; k < K; k += 64) {
+        const float4 v = *reinterpret_cast<const float4*>(x + size_t(t) * K + k);
+        sum = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sum))));
+      }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    if (part == 0) row_scale[t] = 1.0f / sqrtf(sum / float(K) + extra.eps);
+    __syncthreads();
+    scale = row_scale[lr];
+  }
+
+  floatx4_t acc[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int s = s0; s < s1; s += U) {
+    if (s != s0) request(s);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (NORM)
+        xv[u] = make_float4((xv[u].x * scale) * nv[u].x, (xv[u].y * scale) * nv[u].y, (xv[u].z * scale) * nv[u].z,
+                            (xv[u].w * scale) * nv[u].w);
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         acc[rt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[u][rt].x, xv[u].x, acc[rt], 0, 0, 0);
@@ -121,13 +176,61 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
         acc[rt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[u][rt].z, xv[u].z, acc[rt], 0, 0, 0);
         acc[rt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wv[u][rt].w, xv[u].w, acc[rt], 0, 0, 0);
       }
+    }
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
     *reinterpret_cast<float4*>(&sums[wave][rt][lane][0]) = make_float4(acc[rt][0], acc[rt][1], acc[rt][2], acc[rt][3]);
   __syncthreads();
-  // thread (rt, lane) of the first RT waves' worth of threads joins the four waves: element e is
-  // out[token lane % 16][n0 + 16 rt + 4 (lane / 16) + e]
+  // Element e of lane l of tile rt is out[token l % 16][tile row 4 (l / 16) + e]; the four waves are joined in order.
+  auto joined = [&](int rt, int l, int e) {
+    return ((sums[0][rt][l][e] + sums[1][rt][l][e]) + sums[2][rt][l][e]) + sums[3][rt][l][e];
+  };
+  if (MODE == kRope) {
+    // thread (token t, row r < 8): tile row r is element r % 4 of lane t + 16 (r / 4), its partner row r + 8 lies
+    // two quarters of the wave further on
+    if (threadIdx.x >= 128) return;
+    const int t = threadIdx.x & 15, r = threadIdx.x >> 4;
+    if (t >= T) return;
+    const int hd = extra.hd, half = hd / 2;
+    const int head = n0 / hd, d = n0 % hd + r;                       // the dimension of the first half
+    float a = joined(0, t + 16 * (r >> 2), r & 3), b = joined(0, t + 16 * (r >> 2) + 32, r & 3);
+    if (bias) { a += to_float(bias[head * hd + d]); b += to_float(bias[head * hd + d + half]); }
+    if (head < extra.nq + extra.nkv) {
+      float sn, cs;
+      if (extra.inv_freq_tail) {
+        double sn64, cs64;
+        sincos(double(extra.positions[t]) * (double(extra.inv_freq[d]) + double(extra.inv_freq_tail[d])), &sn64, &cs64);
+        sn = float(sn64);
+        cs = float(cs64);
+      } else {
+        sincosf(float(extra.positions[t]) * extra.inv_freq[d], &sn, &cs);
+      }
+      const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+      a = ra;
+      b = rb;
+    }
+    if (head < extra.nq) {
+      float* q = out + size_t(t) * (size_t(extra.nq) * hd) + head * hd + d;
+      q[0] = a;
+      q[half] = b;
+      return;
+    }
+    const int slot = extra.slot_mapping[t];
+    if (slot < 0) return;
+    const int page = slot / extra.page_size, off = slot % extra.page_size;
+    if (page >= extra.num_pages) return;                       // a bad slot must not become a wild address
+    if (head < extra.nq + extra.nkv) {
+      float* k = extra.k_pool + ((size_t(page) * extra.nkv + (head - extra.nq)) * extra.page_size + off) * hd + d;
+      k[0] = a;
+      k[half] = b;
+    } else {
+      float* v = extra.v_pool + ((size_t(page) * extra.nkv + (head - extra.nq - extra.nkv)) * hd + d) * extra.page_size + off;
+      v[0] = a;
+      v[size_t(half) * extra.page_size] = b;
+    }
+    return;
+  }
   if (MODE == kSilu) {
     for (int i = threadIdx.x; i < RT / 2 * 64; i += 256) {
       const int pair = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * pair + 4 * (l >> 4);
@@ -135,9 +238,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (n + e >= N) break;
-        const int a = 2 * pair, b = 2 * pair + 1;
-        const float gate = ((sums[0][a][l][e] + sums[1][a][l][e]) + sums[2][a][l][e]) + sums[3][a][l][e];
-        const float up = ((sums[0][b][l][e] + sums[1][b][l][e]) + sums[2][b][l][e]) + sums[3][b][l][e];
+        const float gate = joined(2 * pair, l, e), up = joined(2 * pair + 1, l, e);
         out[size_t(t) * N + n + e] = gate / (1.0f + expf(-gate)) * up;
       }
     }
@@ -146,14 +247,11 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
   for (int i = threadIdx.x; i < RT * 64; i += 256) {
     const int rt = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * rt + 4 * (l >> 4);
     if (t >= T || n >= N) continue;
-    float v[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = ((sums[0][rt][l][e] + sums[1][rt][l][e]) + sums[2][rt][l][e]) + sums[3][rt][l][e];
     float* dst = out + size_t(t) * N + n;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (n + e >= N) break;
-      float r = v[e];
+      float r = joined(rt, l, e);
       if (bias && blockIdx.y == 0) r += to_float(bias[n + e]);
       if (MODE == kAccumulate) {
         if (gridDim.y > 1) unsafeAtomicAdd(dst + e, r);
@@ -177,9 +275,9 @@ int launch_skinny(hipStream_t s, const float* x, const float* w, const void* bia
   splits = (steps + per_block - 1) / per_block;
   dim3 grid(blocks_n, splits);
   if (mode == kAccumulate)
-    gemm_f32_skinny_kernel<RT, kAccumulate, TB><<<grid, 256, 0, s>>>(x, w, (const TB*)bias, out, T, N, K, per_block);
+    gemm_f32_skinny_kernel<RT, kAccumulate, TB, false><<<grid, 256, 0, s>>>(x, w, (const TB*)bias, out, T, N, K, per_block, SkinnyExtra{});
   else
-    gemm_f32_skinny_kernel<RT, kStoreF32, TB><<<grid, 256, 0, s>>>(x, w, (const TB*)bias, out, T, N, K, per_block);
+    gemm_f32_skinny_kernel<RT, kStoreF32, TB, false><<<grid, 256, 0, s>>>(x, w, (const TB*)bias, out, T, N, K, per_block, SkinnyExtra{});
   return check_launch("sp_gemm (float32, few tokens)");
 }
 
@@ -193,15 +291,34 @@ int skinny_shape(hipStream_t s, const float* x, const float* w, const void* bias
 
 }  // namespace
 
-// out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T) for up to 16 tokens, float32 throughout.
-int gemm_f32_gated(hipStream_t s, const float* x, const float* w, float* out, int T, int I, int K) {
-  const int pairs = (I + 15) / 16;
+// out[T, I] = silu(a . w[:I]^T) * (a . w[I:]^T) for up to 16 tokens, float32 throughout; a = x, or
+// rmsnorm(x) * norm_w where norm_w is given.
+int gemm_f32_gated(hipStream_t s, const float* x, const float* norm_w, float eps, const float* w, float* out, int T, int I, int K) {
+  const int pairs = (I + 15) / 16, steps = (K + 15) / 16;
+  SkinnyExtra extra = {};
+  extra.norm_w = norm_w;
+  extra.eps = eps;
+#define SP_GATED(RT, NORM, BLOCKS) \
+  gemm_f32_skinny_kernel<RT, kSilu, float, NORM><<<dim3(BLOCKS, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, steps, extra)
   if (pairs >= 2048) {
-    gemm_f32_skinny_kernel<4, kSilu, float><<<dim3((pairs + 1) / 2, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, (K + 15) / 16);
+    if (norm_w) SP_GATED(4, true, (pairs + 1) / 2); else SP_GATED(4, false, (pairs + 1) / 2);
   } else {
-    gemm_f32_skinny_kernel<2, kSilu, float><<<dim3(pairs, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, (K + 15) / 16);
+    if (norm_w) SP_GATED(2, true, pairs); else SP_GATED(2, false, pairs);
   }
-  return check_launch("sp_gate_up_silu (float32, few tokens)");
+#undef SP_GATED
+  return check_launch("sp_gate_up_silu_f32");
+}
+
+template <typename TB>
+static int launch_qkv(hipStream_t s, const float* x, const float* w, const void* bias, float* q_out, int T, int K,
+                      const SkinnyExtra& extra) {
+  const int N = (extra.nq + 2 * extra.nkv) * extra.hd, blocks = (extra.nq + 2 * extra.nkv) * (extra.hd / 16);
+  const int steps = (K + 15) / 16;
+  if (extra.norm_w)
+    gemm_f32_skinny_kernel<1, kRope, TB, true><<<dim3(blocks, 1), 256, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
+  else
+    gemm_f32_skinny_kernel<1, kRope, TB, false><<<dim3(blocks, 1), 256, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
+  return check_launch("sp_qkv_rope_cache_f32");
 }
 
 bool gemm_f32_skinny_takes(int T, int N, int K, const void* a, const void* w) {
@@ -223,13 +340,43 @@ using namespace sprout;
 // Whether sp_gate_up_silu_f32 takes T tokens by 2 I rows of K.
 extern "C" int sp_gate_up_silu_f32_takes(int T, int I, int K) { return T >= 1 && T <= 16 && I >= 1 && K % 4 == 0 && K >= 64; }
 
-// out[T, I] (float32) = act(x . w[:I]^T) * (x . w[I:]^T), x float32 [T, K], w float32 [2 I, K], up to 16 tokens:
-// the gated product of a decode step on the float32 path, in one kernel.
-extern "C" int sp_gate_up_silu_f32(void* stream, const float* x, const float* w, float* out, int T, int I, int K,
-                                   int activation) {
+// out[T, I] (float32) = act(a . w[:I]^T) * (a . w[I:]^T), w float32 [2 I, K], up to 16 tokens: the gated product of
+// a decode step on the float32 path, in one kernel.  a = x (float32 [T, K]), or rmsnorm(x) * norm_w (float32 [K],
+// eps) where norm_w is given: the norm before the feed-forward folded in.
+extern "C" int sp_gate_up_silu_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, float* out,
+                                   int T, int I, int K, int activation) {
   SP_REQUIRE(activation == 0, "sp_gate_up_silu_f32: no kernel for activation %d (0 = SiLU)", activation);
   SP_REQUIRE(sp_gate_up_silu_f32_takes(T, I, K), "sp_gate_up_silu_f32: shape T=%d I=%d K=%d is not taken", T, I, K);
-  SP_REQUIRE(x && w && out && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
+  SP_REQUIRE(x && w && out && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(norm_w)) % 16 == 0,
              "sp_gate_up_silu_f32: operands must be given and 16-byte aligned");
-  return gemm_f32_gated((hipStream_t)stream, x, w, out, T, I, K);
+  return gemm_f32_gated((hipStream_t)stream, x, norm_w, eps, w, out, T, I, K);
+}
+
+// Whether sp_qkv_rope_cache_f32 takes the shape: up to 16 tokens, head sizes in 16s turned whole, pairing "halves".
+extern "C" int sp_qkv_rope_cache_f32_takes(int T, int K, int nq, int nkv, int hd, int rotary_dim, int pairing) {
+  return T >= 1 && T <= 16 && K % 4 == 0 && K >= 64 && nq > 0 && nkv > 0 && hd > 0 && hd % 16 == 0 && rotary_dim == hd && pairing == 0;
+}
+
+// q, k, v = a . w^T + bias for up to 16 tokens, all float32; q and k heads turned by positions * inv_freq (angles in
+// float64 where inv_freq_tail, the float64 table minus inv_freq, is given); q to q_out [T, nq * hd], k and v into the
+// paged pools at slot_mapping.  a = x [T, K], or rmsnorm(x) * norm_w where norm_w is given.
+extern "C" int sp_qkv_rope_cache_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w,
+                                     int bias_dtype, const void* bias, float* q_out, const int32_t* positions,
+                                     const float* inv_freq, const float* inv_freq_tail, int rotary_dim,
+                                     const int32_t* slot_mapping, float* k_pool, float* v_pool, int T, int K, int nq,
+                                     int nkv, int hd, int page_size, int num_pages, int pairing) {
+  SP_REQUIRE(sp_qkv_rope_cache_f32_takes(T, K, nq, nkv, hd, rotary_dim, pairing),
+             "sp_qkv_rope_cache_f32: T=%d K=%d heads=%d/%d hd=%d rotary=%d pairing=%d is not taken", T, K, nq, nkv, hd,
+             rotary_dim, pairing);
+  SP_REQUIRE(x && w && q_out && positions && inv_freq && slot_mapping && k_pool && v_pool && page_size > 0 && num_pages > 0,
+             "sp_qkv_rope_cache_f32: null operand or bad cache geometry");
+  SP_REQUIRE((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(norm_w)) % 16 == 0,
+             "sp_qkv_rope_cache_f32: operands must be 16-byte aligned");
+  SP_REQUIRE(!bias || bias_dtype == kF32 || bias_dtype == kBF16, "sp_qkv_rope_cache_f32: unsupported bias dtype %d", bias_dtype);
+  SkinnyExtra extra = {};
+  extra.norm_w = norm_w; extra.eps = eps; extra.positions = positions; extra.inv_freq = inv_freq;
+  extra.inv_freq_tail = inv_freq_tail; extra.slot_mapping = slot_mapping; extra.k_pool = k_pool; extra.v_pool = v_pool;
+  extra.nq = nq; extra.nkv = nkv; extra.hd = hd; extra.page_size = page_size; extra.num_pages = num_pages;
+  if (bias && bias_dtype == kBF16) return launch_qkv<bf16_t>((hipStream_t)stream, x, w, bias, q_out, T, K, extra);
+  return launch_qkv<float>((hipStream_t)stream, x, w, bias, q_out, T, K, extra);
 }

@@ -110,9 +110,20 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 // dst (dst_dtype) = src (src_dtype), n elements
 
 // tokens[i] = previous[source[i]] for every i < n with source[i] >= 0 (others are left as they are):
-// The gated product of up to 16 tokens on the float32 path: out[T, I] = act(x . w[:I]^T) * (x . w[I:]^T), all float32.
+// The float32 path's decode-sized products (up to 16 tokens, everything float32) with neighbouring work folded in.
+// Activations are x [T, K], or rmsnorm(x) * norm_w computed inside the kernel where norm_w [K] is given.
+//   sp_gate_up_silu_f32:   out[T, I] = act(a . w[:I]^T) * (a . w[I:]^T)
+//   sp_qkv_rope_cache_f32: q, k, v = a . w^T + bias; q and k heads turned whole by positions * inv_freq (angles
+//                          in float64 where inv_freq_tail, the float64 table minus inv_freq, is given); q to
+//                          q_out [T, nq * hd], k and v into the paged pools at slot_mapping.  Head sizes in 16s.
 int sp_gate_up_silu_f32_takes(int T, int I, int K);
-int sp_gate_up_silu_f32(void* stream, const float* x, const float* w, float* out, int T, int I, int K, int activation);
+int sp_gate_up_silu_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, float* out,
+                        int T, int I, int K, int activation);
+int sp_qkv_rope_cache_f32_takes(int T, int K, int nq, int nkv, int hd, int rotary_dim, int pairing);
+int sp_qkv_rope_cache_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, int bias_dtype,
+                          const void* bias, float* q_out, const int32_t* positions, const float* inv_freq,
+                          const float* inv_freq_tail, int rotary_dim, const int32_t* slot_mapping, float* k_pool,
+                          float* v_pool, int T, int K, int nq, int nkv, int hd, int page_size, int num_pages, int pairing);
 
 // dst[i] = a seeded random value, a function of (key, first + i) alone: the sum of twelve 16-bit fields of three
 // 64-bit hashes, centred, times scale (+ offset if add_offset): near normal with deviation 65536 * scale.

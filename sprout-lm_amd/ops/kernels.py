@@ -441,17 +441,55 @@ def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm
                                     variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
-def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> bool:
-    """out = act(x . w[:I]^T) * (x . w[I:]^T), everything float32, for the few tokens of a decode step.  Returns
+def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activation: str = "silu", norm_weight=None,
+                     eps: float = 0.0) -> bool:
+    """out = act(a . w[:I]^T) * (a . w[I:]^T), everything float32, for the few tokens of a decode step; a = x, or
+    rmsnorm(x) * norm_weight computed inside the kernel where norm_weight is given (x is then the residual).  Returns
     False (and does nothing) where the kernel does not take the shape: the caller then multiplies and gates in turn."""
     N, K = w.shape
     T, I = out.shape
     if (w.dtype != torch.float32 or x.dtype != torch.float32 or out.dtype != torch.float32 or N != 2 * I
             or tuple(x.shape) != (T, K) or not library().sp_gate_up_silu_f32_takes(T, I, K)):
         return False
+    if norm_weight is not None and (norm_weight.dtype != torch.float32 or norm_weight.numel() != K):
+        return False
     _gpu(w, "gate/up weight"); _gpu(x, "activations"); _gpu(out, "gated output")
-    check(library().sp_gate_up_silu_f32(_stream(), x.data_ptr(), w.data_ptr(), out.data_ptr(), T, I, K,
-                                        variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+    check(library().sp_gate_up_silu_f32(_stream(), x.data_ptr(), _ptr(norm_weight), float(eps), w.data_ptr(), out.data_ptr(),
+                                        T, I, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+    return True
+
+
+def qkv_rope_cache_f32(w: torch.Tensor, bias, x: torch.Tensor, q_out: torch.Tensor, positions, inv_freq, inv_freq_tail,
+                       rotary_dim: int, slot_mapping, k_pool, v_pool, nq: int, nkv: int, hd: int, norm_weight=None,
+                       eps: float = 0.0, pairing: str = "halves") -> bool:
+    """The float32 path's q/k/v product of a decode step with bias, rotation and cache write folded in (and the norm
+    before it, where norm_weight is given and x is the residual); see sprout_hip.h.  Returns False, and does
+    nothing, where the kernel does not take the shape."""
+    N, K = w.shape
+    T = x.shape[0]
+    code = ROTARY_PAIRINGS.get(pairing, -1)
+    if (w.dtype != torch.float32 or x.dtype != torch.float32 or q_out.dtype != torch.float32 or N != (nq + 2 * nkv) * hd
+            or tuple(x.shape) != (T, K) or tuple(q_out.shape) != (T, nq * hd) or k_pool is None or k_pool.dtype != torch.float32
+            or not library().sp_qkv_rope_cache_f32_takes(T, K, nq, nkv, hd, rotary_dim, code)):
+        return False
+    if norm_weight is not None and (norm_weight.dtype != torch.float32 or norm_weight.numel() != K):
+        return False
+    for t_, what in ((w, "qkv weight"), (x, "activations"), (q_out, "q output"), (inv_freq, "inv_freq")):
+        _gpu(t_, what)
+    if bias is not None:
+        _gpu(bias, "qkv bias")
+        if bias.numel() != N:
+            raise KernelError("qkv_rope_cache_f32: bias size")
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() < hd // 2 or (inv_freq_tail is not None and (
+            inv_freq_tail.dtype != torch.float32 or inv_freq_tail.numel() != inv_freq.numel())):
+        raise KernelError("qkv_rope_cache_f32: inv_freq (and its tail) must hold hd / 2 float32 values")
+    _ints(positions, T, "positions"); _ints(slot_mapping, T, "slot_mapping")
+    num_pages, page_size = _check_pools(k_pool, v_pool, nkv, hd, torch.float32, "qkv_rope_cache_f32")
+    check(library().sp_qkv_rope_cache_f32(_stream(), x.data_ptr(), _ptr(norm_weight), float(eps), w.data_ptr(),
+                                          _code(bias, "bias") if bias is not None else 0, _ptr(bias), q_out.data_ptr(),
+                                          positions.data_ptr(), inv_freq.data_ptr(), _ptr(inv_freq_tail), rotary_dim,
+                                          slot_mapping.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), T, K, nq, nkv, hd,
+                                          page_size, num_pages, code))
     return True
 
 

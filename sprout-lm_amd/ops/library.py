@@ -41,7 +41,10 @@ def _declare(lib):
         "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
         "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
         "sp_gate_up_silu_f32_takes": [c_int, c_int, c_int],
-        "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int],
+        "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
+        "sp_qkv_rope_cache_f32_takes": [c_int] * 7,
+        "sp_qkv_rope_cache_f32": [c_void, c_void, c_void, c_float, c_void, c_int, c_void, c_void, c_void, c_void, c_void,
+                                  c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int],
         "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int, c_int],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],

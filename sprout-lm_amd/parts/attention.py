@@ -102,6 +102,8 @@ class Attention(Mixer):
         fold = norm.fold() if self.fuse_input_norm else None
         if fold is None or fold.kind != "rms":       # the one prologue the projection kernels have
             return False
+        if ctx.act_dtype == torch.float32:
+            return self._fused_f32(ctx, residual, residual, cache, fold)
         if ctx.act_dtype != torch.bfloat16 or T > 64 or not self._fused(T, cache, True):
             return False
         if not ops.fused_norm_pays(T, self.w_qkv.shape[0], self.hidden):
@@ -110,6 +112,22 @@ class Attention(Mixer):
         ops.qkv_rope_cache(self.w_qkv, self.b_qkv, q, ctx.positions, self.position.inv_freq, self.position.rotary_dim,
                            cache.slot_mapping, cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
                            residual=residual, norm_weight=fold.weight, eps=fold.eps, pairing=self.position.pairing)
+        self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
+        return True
+
+    def _fused_f32(self, ctx, x, residual, cache, fold=None) -> bool:
+        """The float32 path's decode step: projections, bias, rotation and cache write in one kernel (and the norm,
+        where `fold` is given and x is the residual).  False where that kernel does not take the call."""
+        T = x.shape[0]
+        if not (self.own_kv and cache.writes) or T > 16:
+            return False
+        q = ctx.buffer("q", (T, self.heads * self.head_dim), ctx.act_dtype)
+        if not ops.qkv_rope_cache_f32(self.w_qkv, self.b_qkv, x, q, ctx.positions, self.position.inv_freq,
+                                      getattr(self.position, "inv_freq_tail", None), self.position.rotary_dim,
+                                      cache.slot_mapping, cache.k, cache.v, self.heads, self.kv_heads, self.head_dim,
+                                      norm_weight=None if fold is None else fold.weight,
+                                      eps=0.0 if fold is None else fold.eps, pairing=self.position.pairing):
+            return False
         self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
         return True
 
@@ -135,6 +153,8 @@ class Attention(Mixer):
                                self.position.rotary_dim, cache.slot_mapping, cache.k, cache.v, self.heads,
                                self.kv_heads, self.head_dim, x=h, table=table, pairing=self.position.pairing)
             self._attend(ctx, q, self.heads * self.head_dim, residual, cache)
+            return
+        if ctx.act_dtype == torch.float32 and self._fused_f32(ctx, h, residual, cache):
             return
         nkv = self.kv_heads if (self.own_kv and cache.writes) else 0
         width = (self.heads + 2 * nkv) * self.head_dim

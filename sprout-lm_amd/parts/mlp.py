@@ -40,12 +40,20 @@ class GatedMLP(FeedForward):
                                                                                self.hidden, norm=norm, variant=self.activation)
 
     fuse_input_norm = True    # see Attention.fuse_input_norm
+    fuse_input_norm_f32 = True
 
     def forward_from_residual(self, ctx, norm, residual) -> bool:
         T = residual.shape[0]
         fold = norm.fold() if self.fuse_input_norm else None
         if fold is None or fold.kind != "rms":       # the one prologue the product kernels have
             return False
+        if ctx.act_dtype == torch.float32 and self.fuse_input_norm_f32:
+            act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
+            if not ops.gate_up_silu_f32(self.w_gate_up, residual, act, activation=self.activation, norm_weight=fold.weight,
+                                        eps=fold.eps):
+                return False
+            ops.gemm(act, self.w_down, residual, accumulate=True)
+            return True
         if ctx.act_dtype != torch.bfloat16 or T > 64 or not self._fused(T, True):
             return False
         if not ops.fused_norm_pays(T, 2 * self.inner, self.hidden):

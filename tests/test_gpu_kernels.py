@@ -742,3 +742,69 @@ def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
     g, u = gu[:, :I], gu[:, I:]
     want = g / (1 + np.exp(-g)) * u
     assert np.abs(out.float().cpu().numpy() - want).max() <= 2 ** -6 * (1 + np.abs(want).max())
+
+
+@pytest.mark.parametrize("T", [1, 8, 16])
+@pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (2, 1, 96, 64, 4),
+                                              (4, 2, 16, 64, 16), (5, 5, 48, 240, 16)])
+@pytest.mark.parametrize("norm", [False, True])
+def test_float32_qkv_with_norm_rotation_and_cache_write_folded_in(T, nq, nkv, hd, K, page, norm):
+    """The float32 path's q/k/v product of a decode step: bias, rotation with float64 angles at far positions and
+    the cache write in its epilogue, the norm before it as its prologue; against float64 arithmetic."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T * 11 + hd)
+    N, pages, theta, eps = (nq + 2 * nkv) * hd, 40, 1e6, 1e-5
+    w = (rng.standard_normal((N, K)) / math.sqrt(K)).astype(np.float32)
+    b = (rng.standard_normal(N) * 0.3).astype(np.float32)
+    res = (rng.standard_normal((T, K)) * 2).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    x = res.astype(np.float64)
+    if norm:
+        x = x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * nw
+    pos = rng.integers(0, 30000, T)
+    slots = rng.permutation(pages * page)[:T].astype(np.int32)
+    if T > 2:
+        slots[2] = -1
+    exact = theta ** (-2.0 * np.arange(hd // 2) / hd)
+    inv = torch.tensor(exact, dtype=torch.float32, device=DEV)
+    tail = torch.tensor(exact - inv.cpu().double().numpy(), dtype=torch.float32, device=DEV)
+    kp = torch.zeros(pages, nkv, page, hd, device=DEV)
+    vp = torch.zeros(pages, nkv, hd, page, device=DEV)
+    q_out = torch.full((T, nq * hd), float("nan"), device=DEV)
+    assert ops.qkv_rope_cache_f32(t(w), t(b), t(res), q_out, t(pos, torch.int32), inv, tail, hd, t(slots, torch.int32), kp, vp,
+                                  nq, nkv, hd, norm_weight=t(nw) if norm else None, eps=eps)
+    qkv = x @ w.astype(np.float64).T + b
+    want = plain_rope(qkv[:, :(nq + nkv) * hd], pos, hd, hd, theta)
+    tol = 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(qkv).max())
+    assert np.abs(q_out.cpu().numpy() - want[:, :nq * hd]).max() <= tol
+    kp, vp = kp.cpu().numpy(), vp.cpu().numpy().transpose(0, 1, 3, 2)
+    for i in range(T):
+        if slots[i] < 0:
+            continue
+        pg, off = divmod(int(slots[i]), page)
+        assert np.abs(kp[pg, :, off].reshape(-1) - want[i, nq * hd:]).max() <= tol
+        assert np.abs(vp[pg, :, off].reshape(-1) - qkv[i, (nq + nkv) * hd:]).max() <= tol
+    written = np.zeros((pages, page), bool)
+    written[[s // page for s in slots if s >= 0], [s % page for s in slots if s >= 0]] = True
+    assert np.all((kp == 0) | written[:, None, :, None]) and np.all((vp == 0) | written[:, None, :, None])
+    # shapes it does not take are declined, nothing is written
+    assert not ops.qkv_rope_cache_f32(t(w[:(nq + 2 * nkv) * 24]), None, t(res), torch.empty(T, nq * 24, device=DEV),
+                                      t(pos, torch.int32), inv, None, 24, t(slots, torch.int32),
+                                      torch.zeros(pages, nkv, page, 24, device=DEV), torch.zeros(pages, nkv, 24, page, device=DEV),
+                                      nq, nkv, 24)
+
+
+@pytest.mark.parametrize("T,I,K", [(8, 4864, 896), (16, 37, 132), (3, 100, 4864)])
+def test_gated_product_of_few_tokens_in_float32_with_the_norm_folded_in(T, I, K):
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T + I + K + 1)
+    res = (rng.standard_normal((T, K)) * 3).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, K).astype(np.float32)
+    w = (rng.standard_normal((2 * I, K)) * 2 / math.sqrt(K)).astype(np.float32)
+    x = res.astype(np.float64)
+    x = x / np.sqrt((x * x).mean(-1, keepdims=True) + 1e-6) * nw
+    gate, up = x @ w[:I].astype(np.float64).T, x @ w[I:].astype(np.float64).T
+    want = gate / (1 + np.exp(-gate)) * up
+    out = torch.full((T, I), float("nan"), dtype=torch.float32, device=DEV)
+    assert ops.gate_up_silu_f32(t(w), t(res), out, norm_weight=t(nw), eps=1e-6)
+    assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * max(1, math.sqrt(K) / 8) * (1 + np.abs(want).max())
