@@ -69,7 +69,8 @@ int gemm_f32(hipStream_t s, const void* a, const void* w, int bias_dtype, const 
 // NORM: the activations are rmsnorm(x) * norm_w of the float32 residual x, computed here ((x * scale) * w, the
 // very numbers the norm kernel stores): every block sums the squares of its tokens' rows first.
 // MODE kSilu: w holds N gate rows, then N up rows; the block's RT tiles are RT / 2 tiles of gate rows and the
-// matching tiles of up rows, and out[t, n] = silu(gate) * up (float32 [T, N]).
+// matching tiles of up rows (RT = 1: one tile of 8 gate rows, tile rows 0-7, and the matching 8 up rows, 8-15), and
+// out[t, n] = silu(gate) * up (float32 [T, N]).
 // MODE kRope: the rows of w are q, k and v heads of size hd (a multiple of 16); a block's tile is 8 dimensions of
 // a head's first half (tile rows 0-7) and their rotation partners half a head further on (rows 8-15): twice the
 // blocks of whole tiles of 16, and these products live on how many blocks stream.  Bias, rotation of q and k
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
   const int mine = (last - first + 3) / 4;
   const int s0 = first + wave * mine, s1 = min(last, s0 + mine);
 
-  int n0 = blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
+  int n0 = MODE == kSilu && RT == 1 ? blockIdx.x * 8 : blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
   const float* wrow[RT];
   if (MODE == kRope) {
     static_assert(MODE != kRope || RT == 1, "a block of the rotating product is one tile: 8 dimensions and their partners");
@@ -117,7 +118,10 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
   } else {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      const int row = MODE == kSilu ? min(n0 + 16 * (rt / 2) + lr, N - 1) + (rt & 1) * N : min(n0 + 16 * rt + lr, N - 1);
+      int row;
+      if (MODE == kSilu && RT == 1) row = min(n0 + (lr & 7), N - 1) + (lr >> 3) * N;
+      else if (MODE == kSilu) row = min(n0 + 16 * (rt / 2) + lr, N - 1) + (rt & 1) * N;
+      else row = min(n0 + 16 * rt + lr, N - 1);
       wrow[rt] = w + size_t(row) * K + 4 * lj;
     }
   }
@@ -231,6 +235,14 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     }
     return;
   }
+  if (MODE == kSilu && RT == 1) {
+    if (threadIdx.x >= 128) return;
+    const int t = threadIdx.x & 15, r = threadIdx.x >> 4, n = n0 + r;
+    if (t >= T || n >= N) return;
+    const float gate = joined(0, t + 16 * (r >> 2), r & 3), up = joined(0, t + 16 * (r >> 2) + 32, r & 3);
+    out[size_t(t) * N + n] = gate / (1.0f + expf(-gate)) * up;
+    return;
+  }
   if (MODE == kSilu) {
     for (int i = threadIdx.x; i < RT / 2 * 64; i += 256) {
       const int pair = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * pair + 4 * (l >> 4);
@@ -302,8 +314,11 @@ int gemm_f32_gated(hipStream_t s, const float* x, const float* norm_w, float eps
   gemm_f32_skinny_kernel<RT, kSilu, float, NORM><<<dim3(BLOCKS, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, steps, extra)
   if (pairs >= 2048) {
     if (norm_w) SP_GATED(4, true, (pairs + 1) / 2); else SP_GATED(4, false, (pairs + 1) / 2);
-  } else {
+  } else if (pairs >= 512) {
     if (norm_w) SP_GATED(2, true, pairs); else SP_GATED(2, false, pairs);
+  } else {
+    // few rows: tiles of 8 gate rows and their 8 up rows, twice the blocks
+    if (norm_w) SP_GATED(1, true, (I + 7) / 8); else SP_GATED(1, false, (I + 7) / 8);
   }
 #undef SP_GATED
   return check_launch("sp_gate_up_silu_f32");
