@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
     if (part == 0) row_scale[t] = 1.0f / sqrtf(sum / float(K) + extra.eps);
     __syncthreads();
-    scale = row_scale[lr];
+    scale = token ? row_scale[lr] : 0.f;      // lanes past the last token multiply zeros
   }
 
   floatx4_t acc[RT];

@@ -29,7 +29,9 @@ def bf16(x):
                                    # many tokens by few rows; the second with K in four
                                    (1100, 900, 1088), (2000, 130, 2432),
                                    # few tiles and a long K
-                                   (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432)])
+                                   (256, 896, 896), (130, 100, 1088), (200, 1152, 576), (300, 896, 2432),
+                                   # one and two steps of the float32 tiles (K of 32 and 64), and every float32 block shape
+                                   (40, 70, 32), (300, 100, 64), (2048, 9728, 96), (2048, 896, 160), (700, 300, 32)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gemm_all_modes_odd_sizes(T, N, K, dtype):
     from sprout_lm_amd import ops
