@@ -95,3 +95,33 @@ def test_a_registered_step_array_is_laid_out_with_every_step():
         unregister_step_array("plan_test_parity")
         unregister_step_array("plan_test_first")
     assert not any(name.startswith("x:") for name in step_arrays(entries, cache).names)
+
+
+def test_scratch_of_recorded_steps_is_freed_with_the_last_graph_that_used_it():
+    """Recorded steps share scratch tensors that must never move while a graph holds their addresses; a tensor goes
+    when the last graph that was handed it is given up, so shapes that come and go do not pile memory up."""
+    import torch
+    from sprout_lm_amd.engine.batch import KeptWorkspace, OwnedNames
+    kept = KeptWorkspace("cpu")
+    kept.owner = 1
+    small = kept.get("residual", (4, 8), torch.float32)
+    kept.owner = 2
+    again = kept.get("residual", (2, 8), torch.float32)          # fits the tensor that graph 1 made: shared
+    assert again.data_ptr() == small.data_ptr()
+    large = kept.get("residual", (16, 8), torch.float32)         # a further tensor; the first one stays where it is
+    assert large.data_ptr() != small.data_ptr() and kept.nbytes() == (32 + 128) * 4
+    kept.release(1)                                              # graph 2 still uses both
+    assert kept.nbytes() == (32 + 128) * 4
+    kept.release(2)
+    assert kept.nbytes() == 0
+    # what a recorded step hands its caller is kept apart from the shared scratch
+    own = OwnedNames(kept, ("logits",), "cpu")
+    kept.owner = 3
+    logits, scratch = own.get("logits", (2, 5), torch.float32), own.get("normed", (2, 5), torch.float32)
+    assert kept.nbytes() == 40 and logits.data_ptr() != scratch.data_ptr()
+    own.frozen = True
+    with pytest.raises(RuntimeError, match="would grow while a graph is recorded"):
+        own.get("logits", (3, 5), torch.float32)
+    with pytest.raises(RuntimeError, match="would grow while a graph is recorded"):
+        own.get("normed", (3, 5), torch.float32)
+    own.frozen = False
