@@ -334,7 +334,7 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
     store = P.bf16_round if dtype == "bfloat16" else P.f32
     requests = {"a": H.random_tokens(97, 41, 1), "b": H.random_tokens(97, 23, 2), "c": H.random_tokens(97, 30, 3)}
     want = {k: plain_toy_logits(w, t, store) for k, t in requests.items()}
-    tol = 3e-5 if dtype == "float32" else 5e-2
+    tol = 3e-5 if dtype == "float32" else 4e-2
     # a and b run beside each other in uneven portions; c starts when b has ended, in b's state slot and pages
     seqs = {"a": runner.cache.create(), "b": runner.cache.create()}
     fed = {k: 0 for k in requests}
@@ -384,7 +384,7 @@ def test_toy_architecture_decodes_through_recorded_graphs(tmp_path):
         store = P.bf16_round if dtype == "bfloat16" else P.f32
         requests = {"a": H.random_tokens(97, 30, 11), "b": H.random_tokens(97, 19, 12), "c": H.random_tokens(97, 25, 13)}
         want = {k: plain_toy_logits(w, t, store) for k, t in requests.items()}
-        tol = 3e-5 if dtype == "float32" else 5e-2
+        tol = 3e-5 if dtype == "float32" else 4e-2
         seqs = {k: runner.cache.create() for k in requests}
         fed = {"a": 9, "b": 2, "c": 14}
         for k, n in fed.items():                                # the prompts' first portions, eagerly
@@ -609,7 +609,7 @@ def test_toy_routed_feed_forward_and_another_position_encoding(tmp_path, dtype):
     store = P.bf16_round if dtype == "bfloat16" else P.f32
     requests = {"a": H.random_tokens(101, 37, 7), "b": H.random_tokens(101, 20, 8)}
     want = {k: plain_routed_logits(w, t, store) for k, t in requests.items()}
-    tol = 3e-5 if dtype == "float32" else 5e-2
+    tol = 3e-5 if dtype == "float32" else 4e-2
     seqs = {k: runner.cache.create() for k in requests}
     fed = {k: 0 for k in requests}
     used = set()
@@ -737,7 +737,7 @@ def test_a_windowed_layer_shares_prefix_pages(tmp_path, dtype, window_page):
     from safetensors.torch import load_file
     w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
     store = P.bf16_round if dtype == "bfloat16" else P.f32
-    tol = 3e-5 if dtype == "float32" else 5e-2
+    tol = 3e-5 if dtype == "float32" else 4e-2
     shared = H.random_tokens(89, 30, 5)
     requests = {"a": shared + H.random_tokens(89, 9, 6), "b": shared[:26] + H.random_tokens(89, 15, 7),
                 "c": shared[:22] + H.random_tokens(89, 11, 8)}
@@ -960,7 +960,7 @@ def test_a_layer_with_two_mixers_that_both_keep_something(tmp_path, dtype):
     from safetensors.torch import load_file
     w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
     store = P.bf16_round if dtype == "bfloat16" else P.f32
-    tol = 3e-5 if dtype == "float32" else 5e-2
+    tol = 3e-5 if dtype == "float32" else 4e-2
     requests = {f"r{i}": H.random_tokens(113, n, 40 + i) for i, n in enumerate([37, 9, 70, 44, 25, 61])}
     want = {k: plain_dual_logits(w, t, store) for k, t in requests.items()}
     pool = sum(sorted(-(-len(t) // 8) for t in requests.values())[-4:])        # pages of 8: the four longest fit, no more
@@ -1160,7 +1160,7 @@ def test_a_cache_whose_keys_and_values_differ_in_width(tmp_path, dtype):
     from safetensors.torch import load_file
     w = {k: v.float().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
     store = P.bf16_round if dtype == "bfloat16" else P.f32
-    tol = 3e-5 if dtype == "float32" else 5e-2
+    tol = 3e-5 if dtype == "float32" else 4e-2
     requests = {f"r{i}": H.random_tokens(103, n, 60 + i) for i, n in enumerate([37, 12, 58, 41, 26])}
     want = {k: plain_latent_logits(w, t, store) for k, t in requests.items()}
     pool = sum(sorted(-(-len(t) // 8) for t in requests.values())[-4:])
