@@ -341,15 +341,26 @@ def main() -> int:
     from sprout_lm_amd import ops
     measured = ops.probe_machine()
 
-    biggest = max(args.batch, 1 if args.no_points else 256)
-    engine = make_engine(cfg, dtype, biggest, args.context, args.prefill_tokens)
+    # the further batch sizes share the engine's pool: the largest ones are left out where that pool does not fit
+    # beside the weights (the check runs before anything is allocated)
+    from sprout_lm_amd.engine.memory import MemoryBudgetError
+    point_batches = [] if args.no_points else [1, 64, 128, 256]
+    while True:
+        try:
+            engine = make_engine(cfg, dtype, max([args.batch] + point_batches), args.context, args.prefill_tokens)
+            break
+        except MemoryBudgetError:
+            if not point_batches or point_batches[-1] <= args.batch:
+                raise
+            print(f"bench.py: no room for the pool of batch {point_batches.pop()} beside the weights: point left out",
+                  file=sys.stderr)
     parts = engine.model.parts
     warmup = max(args.warmup, 1)
 
     step_s, spread = measure_decode(engine, cfg, args.batch, args.context, args.steps, warmup)
     points = {}
-    if not args.no_points:
-        for b in (1, 64, 128, 256):
+    if point_batches:
+        for b in point_batches:
             s, _ = measure_decode(engine, cfg, b, args.context, max(8, args.steps // 2), min(warmup, 4))
             points[f"decode_b{b}"] = round(b / s, 1)
             if b > 64:
