@@ -95,17 +95,18 @@ struct SkinnyExtra {
   int nq, nkv, hd, page_size, num_pages;
 };
 
-template <int RT, int MODE, typename TB, bool NORM>   // MODE: kStoreF32, kAccumulate, kSilu or kRope
-__global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w,
+template <int RT, int MODE, typename TB, bool NORM, int WAVES = 4>   // MODE: kStoreF32, kAccumulate, kSilu or kRope
+__global__ __launch_bounds__(64 * WAVES) void gemm_f32_skinny_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                               const TB* __restrict__ bias, float* __restrict__ out,
                                                               int T, int N, int K, int steps_per_block, SkinnyExtra extra) {
-  __shared__ float sums[4][RT][64][4];
+  static_assert(WAVES == 4 || WAVES == 8, "four or eight waves share K");
+  __shared__ float sums[WAVES][RT][64][4];
   __shared__ float row_scale[16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
   const int total_steps = (K + 15) / 16;
   const int first = blockIdx.y * steps_per_block, last = min(total_steps, first + steps_per_block);
-  // this wave's steps of the block's: a contiguous quarter
-  const int mine = (last - first + 3) / 4;
+  // this wave's steps of the block's: a contiguous share
+  const int mine = (last - first + WAVES - 1) / WAVES;
   const int s0 = first + wave * mine, s1 = min(last, s0 + mine);
 
   int n0 = MODE == kSilu && RT == 1 ? blockIdx.x * 8 : blockIdx.x * 16 * (MODE == kSilu ? RT / 2 : RT);
@@ -142,24 +143,45 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
         wv[u][rt] = in ? *reinterpret_cast<const float4*>(wrow[rt] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   };
-  // the first steps' weights are asked for before the norm is worked out: they do not depend on it
-  request(s0);
-
+  // NORM: thread (token threadIdx.x / P, part threadIdx.x % P) sums its share of the squares of the token's row,
+  // 8 loads at a time.  The first 8 are asked for before the weights (they come from the
+  // caches, and what returns from memory returns in the order asked for), the weights before anything is summed:
+  // they are on their way meanwhile, and the rest of a longer row queues behind them.
   float scale = 1.f;
   if (NORM) {
-    // thread (token threadIdx.x / 16, part threadIdx.x % 16) sums its sixteenth of the row's squares
-    const int t = threadIdx.x >> 4, part = threadIdx.x & 15;
+    constexpr int P = 4 * WAVES, NB = 8;
+    const int t = threadIdx.x / P, part = threadIdx.x % P;
+    const float* row = x + size_t(min(t, T - 1)) * K;
+    float4 part_x[NB];
+    auto ask = [&](int k0) {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const int k = k0 + j * 4 * P;
+        part_x[j] = (t < T && k < K) ? *reinterpret_cast<const float4*>(row + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    };
     float sum = 0.f;
-    if (t < T)
-      for (int k = 4 * part; k < K; k += 64) {
-        const float4 v = *reinterpret_cast<const float4*>(x + size_t(t) * K + k);
+    auto add = [&]() {
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const float4 v = part_x[j];
         sum = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, sum))));
       }
+    };
+    ask(4 * part);
+    request(s0);
+    add();
+    for (int k0 = 4 * part + NB * 4 * P; k0 < K; k0 += NB * 4 * P) {
+      ask(k0);
+      add();
+    }
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    for (int o = P / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
     if (part == 0) row_scale[t] = 1.0f / sqrtf(sum / float(K) + extra.eps);
     __syncthreads();
     scale = token ? row_scale[lr] : 0.f;      // lanes past the last token multiply zeros
+  } else {
+    request(s0);
   }
 
   floatx4_t acc[RT];
@@ -170,6 +192,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     if (s != s0) request(s);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      if (s + u >= s1) break;      // the same for the whole wave
       if (NORM)
         xv[u] = make_float4((xv[u].x * scale) * nv[u].x, (xv[u].y * scale) * nv[u].y, (xv[u].z * scale) * nv[u].z,
                             (xv[u].w * scale) * nv[u].w);
@@ -186,9 +209,12 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
   for (int rt = 0; rt < RT; ++rt)
     *reinterpret_cast<float4*>(&sums[wave][rt][lane][0]) = make_float4(acc[rt][0], acc[rt][1], acc[rt][2], acc[rt][3]);
   __syncthreads();
-  // Element e of lane l of tile rt is out[token l % 16][tile row 4 (l / 16) + e]; the four waves are joined in order.
+  // Element e of lane l of tile rt is out[token l % 16][tile row 4 (l / 16) + e]; the waves are joined in order.
   auto joined = [&](int rt, int l, int e) {
-    return ((sums[0][rt][l][e] + sums[1][rt][l][e]) + sums[2][rt][l][e]) + sums[3][rt][l][e];
+    float sum = sums[0][rt][l][e];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) sum += sums[w][rt][l][e];
+    return sum;
   };
   if (MODE == kRope) {
     // thread (token t, row r < 8): tile row r is element r % 4 of lane t + 16 (r / 4), its partner row r + 8 lies
@@ -244,7 +270,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     return;
   }
   if (MODE == kSilu) {
-    for (int i = threadIdx.x; i < RT / 2 * 64; i += 256) {
+    for (int i = threadIdx.x; i < RT / 2 * 64; i += 64 * WAVES) {
       const int pair = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * pair + 4 * (l >> 4);
       if (t >= T || n >= N) continue;
 #pragma unroll
@@ -256,7 +282,7 @@ __global__ __launch_bounds__(256) void gemm_f32_skinny_kernel(const float* __res
     }
     return;
   }
-  for (int i = threadIdx.x; i < RT * 64; i += 256) {
+  for (int i = threadIdx.x; i < RT * 64; i += 64 * WAVES) {
     const int rt = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * rt + 4 * (l >> 4);
     if (t >= T || n >= N) continue;
     float* dst = out + size_t(t) * N + n;
@@ -324,16 +350,26 @@ int gemm_f32_gated(hipStream_t s, const float* x, const float* norm_w, float eps
   return check_launch("sp_gate_up_silu_f32");
 }
 
+template <typename TB, int WAVES>
+static int launch_qkv_waves(hipStream_t s, const float* x, const float* w, const void* bias, float* q_out, int T, int K,
+                            const SkinnyExtra& extra, int N, int blocks, int steps) {
+  if (extra.norm_w)
+    gemm_f32_skinny_kernel<1, kRope, TB, true, WAVES><<<dim3(blocks, 1), 64 * WAVES, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
+  else
+    gemm_f32_skinny_kernel<1, kRope, TB, false, WAVES><<<dim3(blocks, 1), 64 * WAVES, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
+  return check_launch("sp_qkv_rope_cache_f32");
+}
+
 template <typename TB>
 static int launch_qkv(hipStream_t s, const float* x, const float* w, const void* bias, float* q_out, int T, int K,
                       const SkinnyExtra& extra) {
   const int N = (extra.nq + 2 * extra.nkv) * extra.hd, blocks = (extra.nq + 2 * extra.nkv) * (extra.hd / 16);
   const int steps = (K + 15) / 16;
-  if (extra.norm_w)
-    gemm_f32_skinny_kernel<1, kRope, TB, true><<<dim3(blocks, 1), 256, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
-  else
-    gemm_f32_skinny_kernel<1, kRope, TB, false><<<dim3(blocks, 1), 256, 0, s>>>(x, w, (const TB*)bias, q_out, T, N, K, steps, extra);
-  return check_launch("sp_qkv_rope_cache_f32");
+  // Few blocks (these rows cannot be split along K: the rotation needs whole sums): eight waves a block share K, so
+  // that half as many trips to memory follow each other in a wave (14 heads of 64 at a width of 896, 72 blocks:
+  // 7.8 against 8.8 us; 16 heads of 128 at 1,536, 128 blocks: 11.8 against 13.3).
+  if (blocks <= 128 && steps > 32) return launch_qkv_waves<TB, 8>(s, x, w, bias, q_out, T, K, extra, N, blocks, steps);
+  return launch_qkv_waves<TB, 4>(s, x, w, bias, q_out, T, K, extra, N, blocks, steps);
 }
 
 bool gemm_f32_skinny_takes(int T, int N, int K, const void* a, const void* w) {

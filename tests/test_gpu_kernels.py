@@ -748,7 +748,7 @@ def test_fused_gate_up_silu_and_normed_product(T, I, K, norm):
 
 @pytest.mark.parametrize("T", [1, 8, 16])
 @pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (2, 1, 96, 64, 4),
-                                              (4, 2, 16, 64, 16), (5, 5, 48, 240, 16)])
+                                              (4, 2, 16, 64, 16), (5, 5, 48, 240, 16), (2, 1, 32, 2116, 8)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_float32_qkv_with_norm_rotation_and_cache_write_folded_in(T, nq, nkv, hd, K, page, norm):
     """The float32 path's q/k/v product of a decode step: bias, rotation with float64 angles at far positions and
