@@ -787,11 +787,12 @@ __global__ __launch_bounds__(64 * WAVES) void attention_merge_kernel(const float
 
 // Merge of the chunks of one head, folded into that head's share of the output projection (decode steps):
 //   residual[row(di), n] += sum_d merged[di, head, d] * w_o[n, head * HD + d]
-// grid (heads, blocks of 64 TPW rows of w_o).  A block merges its head's chunks for every decode sequence
-// (as attention_merge_kernel does, rounded to bfloat16 as the attention output is) into LDS, while its rows
-// of w_o, requested first, are on their way; each wave then multiplies TPW tiles of 16 rows and adds them
-// into the float32 residual.  Against merge kernel + projection kernel this saves a launch and the trip of
-// the attention output through memory.
+// grid (heads, blocks of 64 TPW rows of w_o, tiles of 16 TN decode sequences).  A block merges its head's chunks
+// for its sequences (as attention_merge_kernel does, rounded to bfloat16 as the attention output is) into LDS,
+// while its rows of w_o, requested first, are on their way; each wave then multiplies TPW tiles of 16 rows and
+// adds them into the float32 residual.  Against merge kernel + projection kernel this saves a launch and the
+// trip of the attention output through memory; every block of a head and a tile of sequences merges the same
+// chunks again, so with many sequences a block takes more rows (TPW) and the head fewer blocks.
 template <int DT, int TN, int TPW>
 __global__ __launch_bounds__(256) void attention_merge_project_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int32_t* __restrict__ q_start,
@@ -799,9 +800,12 @@ __global__ __launch_bounds__(256) void attention_merge_project_kernel(
     int n_decode, int n_splits, int nq, int hidden) {
   // GROUP chunks are requested together: the 16 chunks of a context of 4,096 keys in one trip to memory
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2, XP = HD + 8, GROUP = 16;
+  static_assert(TN == 1, "a block merges one tile of 16 sequences");
   __shared__ __attribute__((aligned(16))) uint16_t xs[16 * TN][XP];
+  __shared__ __attribute__((aligned(16))) float sums[16][64 * TPW + 4];
   __shared__ int32_t s_row[16 * TN];
   const int head = blockIdx.x, n_begin = blockIdx.y * (64 * TPW);
+  const int di0 = blockIdx.z * (16 * TN);       // the block's first decode sequence
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
 
   uint4 wa[TPW][HC];
@@ -820,8 +824,9 @@ __global__ __launch_bounds__(256) void attention_merge_project_kernel(
   // merge: HD / 4 threads per decode sequence, four dimensions each
   constexpr int TPR = HD / 4, ROWS = 256 / TPR;
   for (int r0 = 0; r0 < 16 * TN; r0 += ROWS) {
-    const int di = r0 + int(threadIdx.x) / TPR, d = 4 * (int(threadIdx.x) % TPR);
-    if (int(threadIdx.x) >= ROWS * TPR || di >= 16 * TN) continue;
+    const int row = r0 + int(threadIdx.x) / TPR, d = 4 * (int(threadIdx.x) % TPR);   // row of the block's tile
+    if (int(threadIdx.x) >= ROWS * TPR || row >= 16 * TN) continue;
+    const int di = di0 + row;
     float mx = kNoKeyYet, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
     if (di < n_decode) {
       const size_t base = (size_t(di) * nq + head) * n_splits;
@@ -855,34 +860,33 @@ __global__ __launch_bounds__(256) void attention_merge_project_kernel(
           }
         }
       }
-      if (d == 0) s_row[di] = q_start[decode_seqs ? decode_seqs[di] : di];
+      if (d == 0) s_row[row] = q_start[decode_seqs ? decode_seqs[di] : di];
     }
     const float inv = den > 0.f ? 1.0f / den : 0.f;
-    *reinterpret_cast<uint2*>(&xs[di][d]) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
+    *reinterpret_cast<uint2*>(&xs[row][d]) = make_uint2(pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv));
   }
   __syncthreads();
 
+  // The sums go through LDS so that a wave adds 64 neighbouring numbers of one sequence's row of the residual at a
+  // time: heads add into the same rows, and atomics scattered over 16 rows a wave take many times longer.
 #pragma unroll
   for (int i = 0; i < TPW; ++i) {
-    const int n0 = n_begin + 16 * (wave + 4 * i);
-    if (n0 >= hidden) continue;
+    const int tile = wave + 4 * i;
+    if (n_begin + 16 * tile >= hidden || di0 >= n_decode) continue;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      if (16 * tn >= n_decode) continue;
-      floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < HC; ++c) {
-        const int d0 = 32 * c + 8 * lj;
-        const uint4 b = d0 < HD ? *reinterpret_cast<const uint4*>(&xs[16 * tn + lr][d0]) : make_uint4(0, 0, 0, 0);
-        acc = mfma16(as_bf16x8(wa[i][c]), as_bf16x8(b), acc);
-      }
-      const int t = 16 * tn + lr;                 // lane holds rows n0 + 4 lj + 0..3 of w_o for token t
-      if (t >= n_decode) continue;
-      float* dst = residual + size_t(s_row[t]) * hidden + n0 + 4 * lj;
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (n0 + 4 * lj + r < hidden) unsafeAtomicAdd(dst + r, acc[r]);
+    for (int c = 0; c < HC; ++c) {
+      const int d0 = 32 * c + 8 * lj;
+      const uint4 b = d0 < HD ? *reinterpret_cast<const uint4*>(&xs[lr][d0]) : make_uint4(0, 0, 0, 0);
+      acc = mfma16(as_bf16x8(wa[i][c]), as_bf16x8(b), acc);
     }
+    // lane holds rows 16 tile + 4 lj + 0..3 of the block's rows of w_o for sequence di0 + lr
+    *reinterpret_cast<float4*>(&sums[lr][16 * tile + 4 * lj]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 16 * 64 * TPW; i += 256) {
+    const int t = i / (64 * TPW), n = n_begin + i % (64 * TPW);
+    if (di0 + t < n_decode && n < hidden) unsafeAtomicAdd(residual + size_t(s_row[t]) * hidden + n, sums[t][i % (64 * TPW)]);
   }
 }
 
@@ -1060,13 +1064,27 @@ int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_poo
 }
 
 // Decode steps whose chunks' merge is folded into the output projection.  Worth it where the merged partial
-// results, which every block of a head reads again, stay small beside the rows of w_o.
+// results, which every block of a head and a tile of 16 sequences reads again, stay small beside the rows of w_o
+// (measured at 14 heads of 64, a width of 896, contexts of 4,096, tokens a second with the fold against merge and
+// projection kernels of their own: 8 sequences 8,250 against 7,930, 24 sequences 21,870 against 21,260, 32
+// sequences 27,400 against 26,660, 64 sequences 39,840 against 40,350).
 bool attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx, int hidden) {
   if (!attention_mfma_supports(hd, page_size, nq, nkv) || !attention_mfma_decode_supports(nq, nkv)) return false;
   const int n_splits = (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk;
-  // (measured at 14 heads of 64, a width of 896, contexts of 4,096: 8 sequences 7,930 -> 8,250 tokens/s, 64
-  // sequences 31,700 -> 27,800: every block of a head reads all its sequences' chunks)
-  return n_decode >= 1 && n_decode <= 64 && n_splits > 1 && n_decode * n_splits <= 256 && hidden >= 16 && hidden <= 2048;
+  return n_decode >= 1 && n_decode <= 32 && n_splits > 1 && min(n_decode, 16) * n_splits <= 256 && hidden >= 16 &&
+         hidden <= 2048;
+}
+
+// Tiles of 16 rows of w_o a wave takes in the folded kernel: one up to 16 sequences; with more, every tile of 16
+// sequences is a block of its own and merges the head's chunks again, so a block takes as many rows as still
+// leaves about 200 blocks (24 and 32 sequences, 14 heads, a width of 896: two tiles a wave 21,870 and 27,400
+// tokens a second, one 21,600 and 27,100, four 21,400 and 26,990).
+static int project_tiles_per_wave(int n_decode, int nq, int hidden) {
+  if (n_decode <= 16) return 1;
+  const int seq_tiles = (n_decode + 15) / 16;
+  for (int tpw = 4; tpw > 1; tpw /= 2)
+    if (nq * ((hidden + 64 * tpw - 1) / (64 * tpw)) * seq_tiles >= 192) return tpw;
+  return 1;
 }
 
 template <int DT>
@@ -1088,13 +1106,14 @@ static int launch_decode_project(hipStream_t s, const void* q, int q_stride, con
         (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
         ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
   if (check_launch("sp_attention_decode_project (decode)")) return 1;
-  const dim3 grid(nq, (hidden + 63) / 64);
-#define SP_PROJECT(TN)                                                                                          \
-  attention_merge_project_kernel<DT, TN, 1><<<grid, 256, 0, s>>>(part_o, part_ml, q_start, decode_seqs,         \
-                                                                  (const uint16_t*)w_o, residual, n_decode,       \
-                                                                  n_splits, nq, hidden)
-  if (n_decode <= 16) SP_PROJECT(1);
-  else if (n_decode <= 32) SP_PROJECT(2);
+  const int tpw = project_tiles_per_wave(n_decode, nq, hidden);
+  const dim3 grid(nq, (hidden + 64 * tpw - 1) / (64 * tpw), (n_decode + 15) / 16);
+#define SP_PROJECT(TPW)                                                                                         \
+  attention_merge_project_kernel<DT, 1, TPW><<<grid, 256, 0, s>>>(part_o, part_ml, q_start, decode_seqs,        \
+                                                                   (const uint16_t*)w_o, residual, n_decode,     \
+                                                                   n_splits, nq, hidden)
+  if (tpw == 1) SP_PROJECT(1);
+  else if (tpw == 2) SP_PROJECT(2);
   else SP_PROJECT(4);
 #undef SP_PROJECT
   return check_launch("sp_attention_decode_project (merge and projection)");

@@ -282,21 +282,19 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_f32_skinny_kernel(const float
     }
     return;
   }
-  for (int i = threadIdx.x; i < RT * 64; i += 64 * WAVES) {
-    const int rt = i >> 6, l = i & 63, t = l & 15, n = n0 + 16 * rt + 4 * (l >> 4);
+  // thread -> (token, row of the block): neighbouring threads take neighbouring rows of one token, so that a wave
+  // writes or adds runs of 16 RT numbers (atomics scattered one number at a time take several times longer)
+  for (int i = threadIdx.x; i < RT * 256; i += 64 * WAVES) {
+    const int t = i / (16 * RT), row = i % (16 * RT), n = n0 + row;
     if (t >= T || n >= N) continue;
+    float r = joined(row >> 4, t + 16 * ((row & 15) >> 2), row & 3);
+    if (bias && blockIdx.y == 0) r += to_float(bias[n]);
     float* dst = out + size_t(t) * N + n;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (n + e >= N) break;
-      float r = joined(rt, l, e);
-      if (bias && blockIdx.y == 0) r += to_float(bias[n + e]);
-      if (MODE == kAccumulate) {
-        if (gridDim.y > 1) unsafeAtomicAdd(dst + e, r);
-        else dst[e] += r;
-      } else {
-        dst[e] = r;
-      }
+    if (MODE == kAccumulate) {
+      if (gridDim.y > 1) unsafeAtomicAdd(dst, r);
+      else *dst += r;
+    } else {
+      *dst = r;
     }
   }
 }
