@@ -247,8 +247,15 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   // the output rows this thread finishes: kEpiRope dimension er of the block and its partner; kEpiSilu the
   // block's inner columns ei and 16 + ei; otherwise row ei of either tile
   constexpr int OUTS = EPI == kEpiSilu ? (NT + 1) / 2 : 2;
+  // the plain epilogues: thread -> (row pr of the block's 32, tokens pt and pt + 8 of a tile of 16), so that a
+  // wave stores or adds runs of 32 neighbouring numbers of a token's row
+  constexpr bool PLAIN = EPI == kEpiStore || EPI == kEpiAccumulate || EPI == kEpiStoreF32;
+  const int pr = threadIdx.x & 31, pt = threadIdx.x >> 5;
   uint32_t bias_bits[2] = {0u, 0u};   // zero bits are zero in either dtype
-  if (EPI != kEpiSilu && a.bias && blockIdx.y == 0) {
+  if (PLAIN) {
+    if (a.bias && blockIdx.y == 0 && 32 * int(blockIdx.x) + pr < a.N)
+      bias_bits[0] = load_param_bits(a.bias, a.bias_bf16, 32 * blockIdx.x + pr);
+  } else if (EPI != kEpiSilu && a.bias && blockIdx.y == 0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int n = EPI == kEpiRope ? weight_row<EPI, NT>(a, blockIdx.x, NT == 1 ? 0 : i, NT == 1 ? er + 8 * i : er)
@@ -351,13 +358,14 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 
   // The sum of the four waves for (tile, row of the tile, token tile tn, token et): row r of a tile lies in
   // MFMA lane (r / 4) * 16 + token, element r % 4.
-  auto summed = [&](int tile, int row, int tn) {
+  auto summed_at = [&](int tile, int row, int tn, int token) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w)
-      sum += reinterpret_cast<const float*>(&red[((w * NT + tile) * TN + tn) * 64 + (row >> 2) * 16 + et])[row & 3];
+      sum += reinterpret_cast<const float*>(&red[((w * NT + tile) * TN + tn) * 64 + (row >> 2) * 16 + token])[row & 3];
     return sum;
   };
+  auto summed = [&](int tile, int row, int tn) { return summed_at(tile, row, tn, et); };
 #pragma unroll
   for (int tn = 0; tn < TN; ++tn) {
     const int t = t0 + tn * 16 + et;
@@ -375,6 +383,22 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       }
       continue;
     }
+    if (PLAIN) {
+      static_assert(!PLAIN || NT == 2, "the plain epilogues take blocks of two tiles");
+      const int n = 32 * blockIdx.x + pr;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int token = pt + 8 * j, tp = t0 + tn * 16 + token;
+        if (tp >= a.T || n >= a.N) continue;
+        const float v = summed_at(pr >> 4, pr & 15, tn, token) + param_value(bias_bits[0], a.bias_bf16);
+        const size_t o = size_t(tp) * a.N + n;
+        if (EPI == kEpiStore) reinterpret_cast<uint16_t*>(a.out)[o] = f32_to_bf16_bits(v);
+        else if (EPI == kEpiStoreF32) reinterpret_cast<float*>(a.out)[o] = v;
+        else if (gridDim.y == 1) reinterpret_cast<float*>(a.out)[o] += v;
+        else unsafeAtomicAdd(reinterpret_cast<float*>(a.out) + o, v);
+      }
+      continue;
+    }
     float v[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -382,18 +406,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       v[i] = sum + param_value(bias_bits[i], a.bias_bf16);
     }
     if (t >= a.T || (EPI == kEpiRope && NT == 1 && ei >= 8)) continue;
-    if (EPI == kEpiStore || EPI == kEpiStoreF32 || EPI == kEpiAccumulate) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int n = 16 * (NT * blockIdx.x + i) + ei;
-        if (n >= a.N) continue;
-        const size_t o = size_t(t) * a.N + n;
-        if (EPI == kEpiStore) reinterpret_cast<uint16_t*>(a.out)[o] = f32_to_bf16_bits(v[i]);
-        else if (EPI == kEpiStoreF32) reinterpret_cast<float*>(a.out)[o] = v[i];
-        else if (gridDim.y == 1) reinterpret_cast<float*>(a.out)[o] += v[i];
-        else unsafeAtomicAdd(reinterpret_cast<float*>(a.out) + o, v[i]);
-      }
-    } else {  // kEpiRope
+    {  // kEpiRope
       const int head = rope_head, d = rope_dim;      // d < hd / 2; partner dim d + hd / 2
       // projections are kept as bfloat16 before the rotation, as in the unfused path
       float lo = to_float(bf16_t{f32_to_bf16_bits(v[0])}), hi = to_float(bf16_t{f32_to_bf16_bits(v[1])});
