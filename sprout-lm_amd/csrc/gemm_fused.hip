@@ -152,7 +152,8 @@ struct NormInputs {
 };
 
 // The weight row that lane-row `lr` of tile `i` of block `b` multiplies (an existing row also where the tile
-// has no row for the lane: what it computes there is not used).
+// has no row for the lane: what it computes there is not used, and in the gated product's last tile, which the
+// block's rows fill only in part, such a lane asks for nothing).
 template <int EPI, int NT>
 __device__ __forceinline__ int weight_row(const FusedArgs& a, int b, int i, int lr) {
   int row;
@@ -201,6 +202,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
   // of this wave together (steps s0, s0 + 4, ...).
   constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
+  const bool last_tile_row = EPI != kEpiSilu || 16 * (NT - 1) + lr < 2 * a.rows_per_block;   // this lane's row of the last tile is one of the block's
   uint4 wa[UN][NT][2];
   auto load_weights = [&](int s0) {
 #pragma unroll
@@ -210,6 +212,12 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         if (step_there) {   // a scalar branch
 #pragma unroll
           for (int i = 0; i < NT; ++i) {
+            if (EPI == kEpiSilu && NT == 3 && i == 2 && !last_tile_row) {
+              // the third tile is only partly filled (the block's 2 x rows_per_block rows end in it): lanes
+              // without a row ask for nothing
+              wa[u][i][0] = wa[u][i][1] = make_uint4(0, 0, 0, 0);
+              continue;
+            }
             wa[u][i][0] = ldg128(wrow[i] + 64 * s0 + 256 * u);
             wa[u][i][1] = ldg128(wrow[i] + 64 * s0 + 256 * u + 8);
           }
@@ -222,8 +230,9 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         const bool in0 = step_there && k < k_end, in1 = step_there && k + 8 < k_end;
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
-          wa[u][i][0] = in0 ? ldg128(wrow[i] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
-          wa[u][i][1] = in1 ? ldg128(wrow[i] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
+          const bool row_there = i < NT - 1 || last_tile_row;
+          wa[u][i][0] = in0 && row_there ? ldg128(wrow[i] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
+          wa[u][i][1] = in1 && row_there ? ldg128(wrow[i] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
         }
       }
     }
