@@ -10,10 +10,12 @@
 //                    the norm kernel would have stored, so a token's activations do not depend on which of
 //                    the two ways a step takes.
 //   epilogue  kEpiStore / kEpiAccumulate / kEpiStoreF32   as the plain product (+ bias)
-//             kEpiRope   the block's rows are rotation partners (dims d and d + head/2 of one head): two tiles
-//                        of 16, or (NT = 1, up to 16 tokens) one tile of 8 dimensions and their 8 partners, so
-//                        that the few rows of q, k and v are spread over twice the blocks; adds the bias,
-//                        rotates q and k heads, writes q and scatters k, v into the paged cache
+//             kEpiRope   the block's rows are `rows_per_block` rotation pairs (dims d and d + head/2 of a head,
+//                        counted through all heads): their first rows in one tile and their partners in the other
+//                        (up to 16 pairs), or both in one gathered tile (NT = 1, up to 8 pairs: rows 0-7 and
+//                        8-15); the pairs a block takes are chosen so that the blocks are a whole number per CU
+//                        where they can be (a CU pulls its rows no faster for having them in fewer blocks); adds
+//                        the bias, rotates q and k heads, writes q and scatters k, v into the paged cache
 //             kEpiSilu   the block owns `rows_per_block` inner columns: their gate rows and the matching up rows
 //                        fill its tiles one after the other (two tiles hold 16 of each; three hold up to 24, which
 //                        lets a matrix be cut into a whole number of blocks per CU); writes silu(gate) * up
@@ -41,7 +43,7 @@ struct FusedArgs {
   void* out;                 // [T, N] (store / accumulate); [T, N / 2] for kEpiSilu; q rows [T, nq * hd] for kEpiRope
   int T, N, K, k_per_split;
   int partner;               // rows between a row and its partner (kEpiRope: hd / 2, kEpiSilu: N / 2)
-  int rows_per_block;        // kEpiSilu: inner columns a block owns (at most 8 * NT)
+  int rows_per_block;        // kEpiSilu: inner columns a block owns (at most 8 * NT); kEpiRope: rotation pairs a block owns
   // kEpiRope
   const int32_t* positions;
   const float* inv_freq;
@@ -158,11 +160,11 @@ template <int EPI, int NT>
 __device__ __forceinline__ int weight_row(const FusedArgs& a, int b, int i, int lr) {
   int row;
   if (EPI == kEpiRope) {
-    const int dims = NT == 1 ? 8 : 16;                    // dimensions of a head's first half that a block takes
-    const int per_head = a.hd / (2 * dims);
-    const int first = (b / per_head) * a.hd + dims * (b % per_head);
-    // one gathered tile: rows 0..7 are dims first .. + 7 of the head, rows 8..15 their partners half a head on
-    row = NT == 1 ? first + (lr < 8 ? lr : a.partner + lr - 8) : first + i * a.partner + lr;
+    // pair p of all heads' pairs is dimension p % (hd / 2) of head p / (hd / 2) and its partner half a head on;
+    // one gathered tile: rows 0..7 are the block's pairs' first rows, rows 8..15 their partners
+    const int slot = NT == 1 ? (lr & 7) : lr, second = NT == 1 ? lr >> 3 : i;
+    const int pair = b * a.rows_per_block + slot;
+    row = (pair / a.partner) * a.hd + pair % a.partner + second * a.partner;
   } else if (EPI == kEpiSilu) {
     // the block's gate rows, then its up rows, fill the tiles one after the other
     const int slot = 16 * i + lr, r = a.rows_per_block;
@@ -173,7 +175,7 @@ __device__ __forceinline__ int weight_row(const FusedArgs& a, int b, int i, int 
   return min(a.N - 1, row);
 }
 
-template <int TN, int EPI, bool NORM, int NT, bool K64>
+template <int TN, int EPI, bool NORM, int NT, bool K64, int UN>
 __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   static_assert(NT == 2 || EPI == kEpiRope || EPI == kEpiSilu, "one or three tiles a block only where rows are paired");
   static_assert(!NORM || TN == 1, "the norm prologue takes one tile of 16 tokens");
@@ -201,8 +203,22 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
 
   // The weights' way from memory is the longest wait of the kernel: they are requested at once, UN steps
   // of this wave together (steps s0, s0 + 4, ...).
-  constexpr int UN = TN >= 4 ? 2 : 4;   // steps of 64 requested together: fewer with many token tiles (registers)
-  const bool last_tile_row = EPI != kEpiSilu || 16 * (NT - 1) + lr < 2 * a.rows_per_block;   // this lane's row of the last tile is one of the block's
+  // UN: steps of 64 requested together (a pass of the four waves is 4 UN steps): 4, 2 with four token tiles
+  // (registers), 8 where a block has a CU to itself and a long K, so that fewer trips to memory follow each other
+  // Whether this lane's row of tile i is one of the block's rows: the gated product's last tile and the rotating
+  // product's tiles may be filled in part, and a lane without a row asks for nothing.
+  bool row_there[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    if (EPI == kEpiSilu) {
+      row_there[i] = 16 * i + lr < 2 * a.rows_per_block;
+    } else if (EPI == kEpiRope) {
+      const int slot = NT == 1 ? (lr & 7) : lr;
+      row_there[i] = slot < a.rows_per_block && int(blockIdx.x) * a.rows_per_block + slot < a.N / a.hd * a.partner;
+    } else {
+      row_there[i] = true;
+    }
+  }
   uint4 wa[UN][NT][2];
   auto load_weights = [&](int s0) {
 #pragma unroll
@@ -212,9 +228,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         if (step_there) {   // a scalar branch
 #pragma unroll
           for (int i = 0; i < NT; ++i) {
-            if (EPI == kEpiSilu && NT == 3 && i == 2 && !last_tile_row) {
-              // the third tile is only partly filled (the block's 2 x rows_per_block rows end in it): lanes
-              // without a row ask for nothing
+            if (((EPI == kEpiSilu && NT == 3 && i == 2) || EPI == kEpiRope) && !row_there[i]) {
               wa[u][i][0] = wa[u][i][1] = make_uint4(0, 0, 0, 0);
               continue;
             }
@@ -230,9 +244,8 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         const bool in0 = step_there && k < k_end, in1 = step_there && k + 8 < k_end;
 #pragma unroll
         for (int i = 0; i < NT; ++i) {
-          const bool row_there = i < NT - 1 || last_tile_row;
-          wa[u][i][0] = in0 && row_there ? ldg128(wrow[i] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
-          wa[u][i][1] = in1 && row_there ? ldg128(wrow[i] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
+          wa[u][i][0] = in0 && row_there[i] ? ldg128(wrow[i] + 64 * s0 + 256 * u) : make_uint4(0, 0, 0, 0);
+          wa[u][i][1] = in1 && row_there[i] ? ldg128(wrow[i] + 64 * s0 + 256 * u + 8) : make_uint4(0, 0, 0, 0);
         }
       }
     }
@@ -264,21 +277,20 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
   if (PLAIN) {
     if (a.bias && blockIdx.y == 0 && 32 * int(blockIdx.x) + pr < a.N)
       bias_bits[0] = load_param_bits(a.bias, a.bias_bf16, 32 * blockIdx.x + pr);
-  } else if (EPI != kEpiSilu && a.bias && blockIdx.y == 0) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int n = EPI == kEpiRope ? weight_row<EPI, NT>(a, blockIdx.x, NT == 1 ? 0 : i, NT == 1 ? er + 8 * i : er)
-                                    : 16 * (NT * blockIdx.x + i) + ei;
-      if (n < a.N) bias_bits[i] = load_param_bits(a.bias, a.bias_bf16, n);
-    }
   }
   int position_of[TN], slot_of[TN];
   float frequency = 0.f;
   int rope_head = 0, rope_dim = 0;
+  bool rope_pair = false;          // this thread finishes a pair of the block
   if (EPI == kEpiRope) {
-    const int dims = NT == 1 ? 8 : 16, per_head = a.hd / (2 * dims);
-    rope_head = blockIdx.x / per_head;
-    rope_dim = dims * (blockIdx.x % per_head) + er;           // < hd / 2; the partner is hd / 2 further
+    const int pair = blockIdx.x * a.rows_per_block + er;
+    rope_pair = (NT == 2 || ei < 8) && er < a.rows_per_block && pair < a.N / a.hd * a.partner;
+    rope_head = rope_pair ? pair / a.partner : 0;
+    rope_dim = rope_pair ? pair - rope_head * a.partner : 0;   // < hd / 2; the partner is hd / 2 further
+    if (rope_pair && a.bias) {
+      bias_bits[0] = load_param_bits(a.bias, a.bias_bf16, rope_head * a.hd + rope_dim);
+      bias_bits[1] = load_param_bits(a.bias, a.bias_bf16, rope_head * a.hd + rope_dim + a.partner);
+    }
     if (rope_dim < a.rotary_dim / 2) frequency = a.inv_freq[rope_dim];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -414,7 +426,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
       const float sum = (EPI == kEpiRope && NT == 1) ? summed(0, er + 8 * i, tn) : summed(i, ei, tn);
       v[i] = sum + param_value(bias_bits[i], a.bias_bf16);
     }
-    if (t >= a.T || (EPI == kEpiRope && NT == 1 && ei >= 8)) continue;
+    if (t >= a.T || (EPI == kEpiRope && !rope_pair)) continue;
     {  // kEpiRope
       const int head = rope_head, d = rope_dim;      // d < hd / 2; partner dim d + hd / 2
       // projections are kept as bfloat16 before the rotation, as in the unfused path
@@ -462,28 +474,47 @@ static size_t fused_lds_bytes(int TN, bool norm, int NT = 2) {
   return sizeof(float4) * 4 * NT * TN * 64 + (norm ? sizeof(float) * 4 * 16 : 0);
 }
 
-template <int TN, int EPI, bool NORM, int NT = 2>
-static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+template <int TN, int EPI, bool NORM, int NT, int UN>
+static int launch_fused_un(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
   const size_t lds = fused_lds_bytes(TN, NORM, NT);     // at most 48 KB (four token tiles of three tiles)
   const dim3 grid(blocks, splits, (a.T + 16 * TN - 1) / (16 * TN));   // z: the tokens in tiles of 16 TN
   if (a.K % 64 == 0 && a.k_per_split % 64 == 0)
-    gemm_fused_kernel<TN, EPI, NORM, NT, true><<<grid, 256, lds, s>>>(a);
+    gemm_fused_kernel<TN, EPI, NORM, NT, true, UN><<<grid, 256, lds, s>>>(a);
   else
-    gemm_fused_kernel<TN, EPI, NORM, NT, false><<<grid, 256, lds, s>>>(a);
+    gemm_fused_kernel<TN, EPI, NORM, NT, false, UN><<<grid, 256, lds, s>>>(a);
   return check_launch("sp_gemm_fused");
 }
 
-// Whether the q/k/v product takes one gathered tile a block: with up to 16 tokens, where twice the blocks pull
-// the rows twice as fast, as long as every block still finds a CU of its own (36 heads of 128: 288 blocks of
-// one tile against 144 of two, 14.0 against 13.1 us at 8 tokens, 16.2 against 13.9 at 16); with more tokens,
-// every block reads all the activations again, which then costs more (28 heads of 128 at a width of 3,584,
-// 64 tokens: 36 us against about 20).  Head sizes that 32 does not divide have no other way.
-static bool rope_one_tile(int T, int hd, int N = 0) { return hd % 32 != 0 || (T <= 16 && N / 16 <= 256); }
-// With the norm prologue a block takes 16 tokens whatever their number (further tiles of tokens are further
-// blocks, each normalising its own rows): one gathered tile a block as long as all the blocks find a CU of
-// their own, two tiles (half the blocks) beyond that, where a CU would have to pull for two blocks.
-static bool rope_one_tile_normed(int T, int N, int hd) {
-  return hd % 32 != 0 || (N / 16) * ((T + 15) / 16) <= 256;
+template <int TN, int EPI, bool NORM, int NT = 2>
+static int launch_fused(hipStream_t s, const FusedArgs& a, int blocks, int splits) {
+  if constexpr (TN == 1 && !NORM && NT <= 2) {
+    // Few blocks with a long K each: a block alone on its CU hides no trip to memory behind another block's, so
+    // its waves ask for twice the steps at once and make half the trips (registers allow it without the norm's
+    // inputs; 28 heads of 128 at a width of 3,584: four passes become two).
+    const int steps_a_wave = (min(a.K, a.k_per_split) + 255) / 256;
+    if (blocks * splits * ((a.T + 15) / 16) <= 256 && steps_a_wave > 4)
+      return launch_fused_un<TN, EPI, NORM, NT, 8>(s, a, blocks, splits);
+  }
+  return launch_fused_un<TN, EPI, NORM, NT, TN >= 4 ? 2 : 4>(s, a, blocks, splits);
+}
+
+// Rotation pairs a block of the q/k/v product owns (all heads' pairs are counted through: a block may end in one
+// head and go on in the next).  A CU pulls its rows at about the same rate however many blocks it holds, and no
+// faster for having more of them in flight, so the rows are cut for the CU that gets the most: bytes a block asks
+// for (two rows a pair, and the activations, which every block reads whole) times blocks per CU, rounded up.  Up
+// to 8 pairs lie in one gathered tile, up to 16 in two.  (Blocks of 8 or 16 pairs whatever the sizes: 18 heads of
+// 64 at a width of 896, 8 tokens: 72 blocks; 36 heads of 128 at 3,584: 144 blocks on 256 CUs.)
+static int rope_pairs_per_block(int T, int N, int K, bool norm) {
+  const int pairs = N / 2, token_tiles = norm ? (T + 15) / 16 : 1;
+  int best_pairs = 8;
+  double best = 1e30;
+  for (int r = 2; r <= 16; ++r) {
+    const int blocks = (pairs + r - 1) / r;
+    const double bytes = 4.0 * r * K + (norm ? 4.0 * min(T, 16) * K + 2.0 * K : 2.0 * T * K);
+    const double cost = double((blocks * token_tiles + 255) / 256) * bytes;
+    if (cost <= best) { best = cost; best_pairs = r; }
+  }
+  return best_pairs;
 }
 
 template <int EPI, bool NORM>
@@ -493,11 +524,11 @@ static int fused_tokens(hipStream_t s, const FusedArgs& a, int blocks, int split
   }
   if constexpr (NORM) {   // tiles of 16 tokens, each a block of its own
     if constexpr (EPI == kEpiRope) {
-      if (rope_one_tile_normed(a.T, a.N, a.hd)) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);
+      if (a.rows_per_block <= 8) return launch_fused<1, EPI, true, 1>(s, a, blocks, splits);   // one gathered tile
     }
     return launch_fused<1, EPI, true>(s, a, blocks, splits);
   } else {
-    if (EPI == kEpiRope && rope_one_tile(a.T, a.hd, a.N)) {
+    if (EPI == kEpiRope && a.rows_per_block <= 8) {
       if constexpr (EPI == kEpiRope) {
         if (a.T <= 16) return launch_fused<1, EPI, false, 1>(s, a, blocks, splits);
         if (a.T <= 32) return launch_fused<2, EPI, false, 1>(s, a, blocks, splits);
@@ -649,8 +680,8 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
   a.page_shift = -1;
   if (page_size > 0 && (page_size & (page_size - 1)) == 0)
     for (a.page_shift = 0; (1 << a.page_shift) < page_size;) ++a.page_shift;
-  const bool one_tile = residual ? rope_one_tile_normed(T, N, hd) : rope_one_tile(T, hd, N);
-  const int blocks = (nq + 2 * nkv) * (hd / (one_tile ? 16 : 32));
+  a.rows_per_block = rope_pairs_per_block(T, N, K, residual != nullptr);
+  const int blocks = (N / 2 + a.rows_per_block - 1) / a.rows_per_block;
   return fused_norm<kEpiRope>((hipStream_t)stream, a, residual != nullptr, blocks, 1);
 }
 
