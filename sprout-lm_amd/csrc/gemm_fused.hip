@@ -694,11 +694,13 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
   // Many tokens, or a few with whole steps of 64 along K: the tiled kernels stream the weights better.  From 17
-  // tokens on always; from 5 on where the matrix is large (2 x 18,944 x 3,584 at 8 tokens: 52.2 against 56.8 us,
-  // at 16 53.4 against 62.4; at one token the fused kernel's 49.1 against 52.3; 2 x 8,960 x 1,536 at 8 tokens
-  // 16.7 against the fused kernel's 15.5).
-  const bool large = size_t(2) * I * K >= (size_t(64) << 20);
-  if (T > 64 || (T > (large ? 4 : 16) && !residual && gemm_pipe_takes(T, 2 * I, K)))
+  // tokens on always; from 9 on where the matrix is large, from 5 on where it is very large (a step of the
+  // whole model at 8 tokens, fused against tiled: 2 x 18,944 x 3,584 3.77 against 3.84 ms, at 16 tokens 4.35 against
+  // 4.30; 2 x 27,648 x 5,120 at 8 tokens 14.82 against 14.70, at 16 17.17 against 16.30; 2 x 8,960 x 1,536 at 8
+  // tokens 15.5 us fused against 16.7).
+  const size_t weights = size_t(2) * I * K;
+  const int fused_up_to = weights >= (size_t(200) << 20) ? 4 : weights >= (size_t(64) << 20) ? 8 : 16;
+  if (T > 64 || (T > fused_up_to && !residual && gemm_pipe_takes(T, 2 * I, K)))
     return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
