@@ -644,10 +644,12 @@ def _normed(res, w, eps):
 
 
 @pytest.mark.parametrize("T", [1, 3, 16, 17, 40, 64, 65, 200, 513])   # above 64: the tiled product's rotating epilogue
-# the last two: few rows with a long K, which eight waves of a block share instead of four
+# (4, 2, 128, 3584) and (3, 1, 64, 2120): few rows with a long K (a block asks for twice the steps at once); (28, 4, 128,
+# 512): more rotation pairs than 256 blocks of 8 hold, so a block takes 9 of them in two tiles, across the heads' ends;
+# (14, 2, 64, 896): 3 pairs a block, which 32 pairs a head do not divide
 @pytest.mark.parametrize("nq,nkv,hd,K,page", [(14, 2, 64, 896, 16), (3, 1, 32, 96, 8), (4, 4, 128, 264, 16), (5, 1, 96, 240, 4),
                                               (4, 2, 128, 3584, 16), (3, 1, 64, 2120, 8), (4, 2, 16, 64, 16), (5, 5, 48, 240, 16),
-                                              (2, 1, 80, 160, 4), (5, 1, 64, 320, 8), (3, 3, 128, 384, 16)])
+                                              (2, 1, 80, 160, 4), (5, 1, 64, 320, 8), (3, 3, 128, 384, 16), (28, 4, 128, 512, 16)])
 @pytest.mark.parametrize("norm", [False, True])
 def test_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm):
     check_fused_qkv_rope_cache(T, nq, nkv, hd, K, page, norm)
